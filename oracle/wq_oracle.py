@@ -1,0 +1,181 @@
+"""CPU oracle for the weight-only-quantized dequantize + matmul path (NumPy).
+
+TEST INFRASTRUCTURE ONLY.  Nothing that ships (the `relax_amd` package, the
+C-ABI library) may import this module; only `tests/`, the smoke check and the
+`cpu_baseline` leg of the benchmark use it, and only as the checker.
+
+It restates, in closed form, what the reference's llvm-CPU path computes for the
+canonical module
+
+    Wd  = call_tir(decode_q{4,8}f16, (Wq, S))      # [N, K] float16
+    y32 = matmul(x, permute_dims(Wd), out_dtype="float32")
+    y   = astype(y32, "float16")
+
+Reference semantics followed (file:line under the reference tree):
+
+* integer unpack: `shift_right` on an unsigned operand is a logical shift,
+  `bitwise_and` is a plain AND -- src/target/llvm/codegen_llvm.cc:1271-1285;
+  uint -> int8 is an integer truncation and int/uint -> float16 is an exact
+  SIToFP/UIToFP -- src/target/llvm/codegen_llvm.cc:820-852.
+* float16 arithmetic in `decode` rounds to float16 after every operation
+  (the result is stored to a float16 buffer in the unfused module).
+* matmul: products `float32(a) * float32(b)` summed by a sequential float32
+  reduction over ascending k starting from 0 --
+  python/tvm/relax/transform/legalize_ops.py:203-264 and the golden TIR in
+  tests/python/relax/test_transform_legalize_ops_index_linear_algebra.py:283-313.
+* final cast float32 -> float16 is round-to-nearest-even (FPCast) --
+  python/tvm/relax/transform/legalize_ops.py:157-162,
+  src/target/llvm/codegen_llvm.cc:849-850.
+
+Layout decisions frozen by this build (the reference holds no quantized path):
+element k of a row lives in word k // per_word at bit offset
+(k % per_word) * bits, least-significant field first.
+
+Pinning (see tests/test_oracle.py): unpack against an independent pure-Python
+bit walk over every field value and position; dequantize exhaustively against a
+float64 closed form for all 16 x 65536 (q4) and 256 x 65536 (q8) operand pairs;
+matmul against exact integer arithmetic, one-hot readback, a float64 bound and an
+order-sensitive hand-computed case.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+Q4_ZERO_POINT = 7
+Q4_GROUP = 32
+Q8_GROUP = 128
+
+
+# ----------------------------------------------------------------------------
+# packing (inverse of the decode index arithmetic; used to build test inputs)
+# ----------------------------------------------------------------------------
+def pack_q4(w: np.ndarray) -> np.ndarray:
+    """[N, K] integers in 0..15 -> uint32 [N, K/8], field k%8 at bit (k%8)*4."""
+    w = np.asarray(w)
+    n, k = w.shape
+    assert k % 8 == 0
+    assert w.min(initial=0) >= 0 and w.max(initial=0) <= 15
+    f = w.astype(np.uint32).reshape(n, k // 8, 8)
+    out = np.zeros((n, k // 8), dtype=np.uint32)
+    for i in range(8):
+        out |= f[:, :, i] << np.uint32(4 * i)
+    return out
+
+
+def pack_q8(w: np.ndarray) -> np.ndarray:
+    """[N, K] integers in -128..127 -> uint32 [N, K/4], byte k%4 at bit (k%4)*8."""
+    w = np.asarray(w)
+    n, k = w.shape
+    assert k % 4 == 0
+    assert w.min(initial=0) >= -128 and w.max(initial=0) <= 127
+    f = (w.astype(np.int64) & 0xFF).astype(np.uint32).reshape(n, k // 4, 4)
+    out = np.zeros((n, k // 4), dtype=np.uint32)
+    for i in range(4):
+        out |= f[:, :, i] << np.uint32(8 * i)
+    return out
+
+
+# ----------------------------------------------------------------------------
+# decode: integer part
+# ----------------------------------------------------------------------------
+def unpack_q4(wq: np.ndarray) -> np.ndarray:
+    """uint32 [N, K/8] -> uint8 [N, K]: (Wq[n, k//8] >> ((k%8)*4)) & 15."""
+    wq = np.ascontiguousarray(wq, dtype=np.uint32)
+    n, kw = wq.shape
+    sh = (np.arange(8, dtype=np.uint32) * np.uint32(4))[None, None, :]
+    return ((wq[:, :, None] >> sh) & np.uint32(15)).astype(np.uint8).reshape(n, kw * 8)
+
+
+def unpack_q8(wq: np.ndarray) -> np.ndarray:
+    """uint32 [N, K/4] -> int8 [N, K]: int8((Wq[n, k//4] >> ((k%4)*8)) & 255)."""
+    wq = np.ascontiguousarray(wq, dtype=np.uint32)
+    n, kw = wq.shape
+    sh = (np.arange(4, dtype=np.uint32) * np.uint32(8))[None, None, :]
+    b = ((wq[:, :, None] >> sh) & np.uint32(255)).astype(np.uint8)
+    return b.view(np.int8).reshape(n, kw * 4)  # two's-complement truncation
+
+
+# ----------------------------------------------------------------------------
+# decode: float16 part (one rounding per float16 operation)
+# ----------------------------------------------------------------------------
+def dequant_q4f16(wq, s, group: int = Q4_GROUP, zero_point: int = Q4_ZERO_POINT) -> np.ndarray:
+    """Wd[n,k] = (f16(w) - f16(zp)) * S[n, k//group], each op rounded to f16."""
+    w = unpack_q4(wq)
+    n, k = w.shape
+    s = np.asarray(s, dtype=np.float16)
+    assert s.shape == (n, k // group) and k % group == 0
+    centred = w.astype(np.float16) - np.float16(zero_point)  # exact, |.| <= 15
+    with np.errstate(all="ignore"):
+        return centred * np.repeat(s, group, axis=1)  # float16 multiply: single RNE
+
+
+def dequant_q8f16(wq, s, group: int = Q8_GROUP) -> np.ndarray:
+    """Wd[n,k] = f16(int8 field) * S[n, k//group]."""
+    w = unpack_q8(wq)
+    n, k = w.shape
+    s = np.asarray(s, dtype=np.float16)
+    assert s.shape == (n, k // group) and k % group == 0
+    with np.errstate(all="ignore"):
+        return w.astype(np.float16) * np.repeat(s, group, axis=1)
+
+
+def dequant(wq, s, bits: int, group: int) -> np.ndarray:
+    if bits == 4:
+        return dequant_q4f16(wq, s, group)
+    if bits == 8:
+        return dequant_q8f16(wq, s, group)
+    raise ValueError(f"bits must be 4 or 8, got {bits}")
+
+
+# ----------------------------------------------------------------------------
+# matmul + cast
+# ----------------------------------------------------------------------------
+def matmul_f32acc(x: np.ndarray, wd: np.ndarray) -> np.ndarray:
+    """y32[m,n] = sum_k f32(x[m,k]) * f32(Wd[n,k]); float32, k ascending, init 0.
+
+    Vectorised over (m, n); the k loop is explicit so every output element sees
+    exactly the reference's sequence of float32 additions.
+    """
+    x32 = np.asarray(x, dtype=np.float16).astype(np.float32)
+    w32 = np.asarray(wd, dtype=np.float16).astype(np.float32)
+    m, k = x32.shape
+    n, k2 = w32.shape
+    assert k == k2
+    acc = np.zeros((m, n), dtype=np.float32)
+    wt = np.ascontiguousarray(w32.T)  # [K, N]
+    with np.errstate(all="ignore"):
+        for kk in range(k):
+            acc += x32[:, kk, None] * wt[kk][None, :]  # product exact in f32, one f32 add
+    return acc
+
+
+def cast_f16(y32: np.ndarray) -> np.ndarray:
+    with np.errstate(all="ignore"):
+        return np.asarray(y32, dtype=np.float32).astype(np.float16)
+
+
+def wq_matmul(x, wq, s, bits: int, group: int) -> np.ndarray:
+    """The whole path: y = f16( x @ dequant(Wq, S)^T ) with float32 accumulation."""
+    return cast_f16(matmul_f32acc(x, dequant(wq, s, bits, group)))
+
+
+# ----------------------------------------------------------------------------
+# synthetic inputs of the benchmark's distributions
+# ----------------------------------------------------------------------------
+def make_case(seed: int, m: int, n: int, k: int, bits: int, group: int | None = None):
+    """x ~ N(0,1) f16; q4: w ~ U{0..15}, S ~ U(0.005,0.02); q8: w ~ U{-127..127}, S ~ U(0.002,0.01)."""
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((m, k), dtype=np.float32).astype(np.float16)
+    if bits == 4:
+        group = group or Q4_GROUP
+        w = rng.integers(0, 16, size=(n, k), dtype=np.int64)
+        wq = pack_q4(w)
+        s = rng.uniform(0.005, 0.02, size=(n, k // group)).astype(np.float16)
+    elif bits == 8:
+        group = group or Q8_GROUP
+        w = rng.integers(-127, 128, size=(n, k), dtype=np.int64)
+        wq = pack_q8(w)
+        s = rng.uniform(0.002, 0.01, size=(n, k // group)).astype(np.float16)
+    else:
+        raise ValueError(bits)
+    return x, wq, s, group

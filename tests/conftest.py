@@ -1,0 +1,28 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+def pytest_collection_modifyitems(config, items):
+    """GPU tests are skipped, not failed, when collected on a machine without a GPU."""
+    have_gpu = None
+    for item in items:
+        if "gpu" in item.keywords:
+            if have_gpu is None:
+                try:
+                    import torch
+
+                    have_gpu = torch.cuda.is_available()
+                except Exception:  # pragma: no cover
+                    have_gpu = False
+            if not have_gpu:
+                item.add_marker(pytest.mark.skip(reason="no GPU in this process"))
