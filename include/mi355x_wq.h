@@ -1,0 +1,91 @@
+/*
+ * mi355x_wq.h -- C ABI of the MI355X (gfx950) weight-only-quantized
+ * dequantize + matmul library.  Plain pointers and sizes only: no TVM, DLPack or
+ * torch types appear below this line.  The TVM PackedFunc entries that Relax's VM
+ * calls are declared in mi355x_wq_packed.h and forward to the functions here.
+ *
+ * Data layout (row-major, compact):
+ *   x       [M, K]            float16 activations
+ *   wq      [N, K*bits/32]    uint32; element k of row n is the field at bit
+ *                             (k % (32/bits)) * bits of word k / (32/bits)
+ *                             (least-significant field first)
+ *   scales  [N, K/group]      float16, one scale per `group` consecutive k
+ *   wd      [N, K]            float16 dequantized weights
+ *   y       [M, N]            float16 = f16( sum_k f32(x[m,k]) * f32(wd[n,k]) )
+ *
+ *   bits = 4: wd = (f16(field) - f16(zero_point)) * scale   (one float16 rounding)
+ *   bits = 8: wd = f16(int8(field)) * scale                 (zero_point must be 0)
+ *
+ * Every pointer is device memory of the current HIP device.  All launches are
+ * asynchronous on `stream` (a hipStream_t passed as void*; NULL = the null
+ * stream); synchronisation is the caller's.  Functions return 0 on success and
+ * -1 on failure, in which case nothing was launched and
+ * mi355x_wq_last_error() describes the reason (thread-local string).
+ */
+#ifndef MI355X_WQ_H_
+#define MI355X_WQ_H_
+
+#include <stdint.h>
+
+#ifndef MI355X_WQ_API
+#define MI355X_WQ_API __attribute__((visibility("default")))
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Describes one quantized weight matrix.  Counterpart of the per-kernel
+ * attributes the reference attaches to a partitioned function before codegen
+ * (arg shapes, dtypes, leading dimensions):
+ * python/tvm/contrib/cutlass/build.py:623-672 (handle_matmul). */
+typedef struct mi355x_wq_desc {
+  int32_t bits;       /* 4 or 8 */
+  int32_t group;      /* k per scale: multiple of 32 (bits=4) or 16 (bits=8), divides K */
+  int32_t zero_point; /* bits=4: 0..15 (7 for q4f16); bits=8: 0 */
+  int32_t reserved;   /* must be 0 */
+  int64_t n;          /* rows of the weight matrix = output features */
+  int64_t k;          /* reduction length; multiple of `group` */
+} mi355x_wq_desc;
+
+/* Kernel families; MI355X_WQ_KERNEL_AUTO picks by M (skinny for M <= 64). */
+enum {
+  MI355X_WQ_KERNEL_AUTO = 0,
+  MI355X_WQ_KERNEL_SKINNY = 1, /* HBM-bound GEMV / skinny path, M <= 64 */
+  MI355X_WQ_KERNEL_GEMM = 2    /* LDS-tiled MFMA GEMM, any M */
+};
+
+/* y[M,N] = f16( x[M,K] @ dequant(wq, scales)^T ), float32 accumulation.
+ * Replaces the generated CUTLASS host glue `<sym>_(DLTensor* x, DLTensor* w,
+ * DLTensor* out)`: python/tvm/contrib/cutlass/gemm_operation.py:265-303
+ * (pointer/shape extraction, launch on the current stream, no host sync). */
+MI355X_WQ_API int mi355x_wq_matmul(const mi355x_wq_desc* desc, const void* x, const void* wq, const void* scales,
+                     void* y, int64_t m, void* stream);
+
+/* Same, with the kernel family forced (tests and benchmarks). */
+MI355X_WQ_API int mi355x_wq_matmul_ex(const mi355x_wq_desc* desc, const void* x, const void* wq,
+                        const void* scales, void* y, int64_t m, void* stream, int kernel);
+
+/* wd[N,K] = dequant(wq, scales), bit-exact with the float16 arithmetic of the
+ * `decode` PrimFunc as the llvm target lowers it
+ * (src/target/llvm/codegen_llvm.cc:820-852, 1271-1285). */
+MI355X_WQ_API int mi355x_wq_dequantize(const mi355x_wq_desc* desc, const void* wq, const void* scales, void* wd,
+                         void* stream);
+
+/* Validates a descriptor and a row count without touching the GPU: 0 if
+ * mi355x_wq_matmul would accept them. */
+MI355X_WQ_API int mi355x_wq_check(const mi355x_wq_desc* desc, int64_t m);
+
+/* Which family AUTO dispatch uses for `m` rows (MI355X_WQ_KERNEL_*), or -1. */
+MI355X_WQ_API int mi355x_wq_select_kernel(const mi355x_wq_desc* desc, int64_t m);
+
+/* Thread-local description of the last failure on this thread ("" if none). */
+MI355X_WQ_API const char* mi355x_wq_last_error(void);
+
+/* Library version: major * 10000 + minor * 100 + patch. */
+MI355X_WQ_API int mi355x_wq_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355X_WQ_H_ */

@@ -1,0 +1,150 @@
+// C ABI of the library (include/mi355x_wq.h): argument validation, kernel-family
+// dispatch and the thread-local error string.  No kernel is launched unless every
+// shape, size and alignment assumption of the kernels has been checked here.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/mi355x_wq.h"
+#include "wq_internal.h"
+
+namespace wq {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+namespace {
+
+constexpr int64_t kMaxBufferBytes = 0x7FFFFFF0ll;  // kernels address buffers with 32-bit offsets
+
+bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+
+bool check_desc(const mi355x_wq_desc* d, int64_t m) {
+  if (d == nullptr) {
+    set_error("descriptor is NULL");
+    return false;
+  }
+  if (d->bits != 4 && d->bits != 8) {
+    set_error("bits must be 4 or 8, got %d", d->bits);
+    return false;
+  }
+  if (d->reserved != 0) {
+    set_error("descriptor.reserved must be 0, got %d", d->reserved);
+    return false;
+  }
+  const int ch = 128 / d->bits;
+  if (d->group <= 0 || d->group % ch != 0 || !is_pow2(d->group / ch)) {
+    set_error("group must be %d times a power of two for %d-bit weights, got %d", ch, d->bits,
+              d->group);
+    return false;
+  }
+  if (d->bits == 4 && (d->zero_point < 0 || d->zero_point > 15)) {
+    set_error("zero_point must be in 0..15 for 4-bit weights, got %d", d->zero_point);
+    return false;
+  }
+  if (d->bits == 8 && d->zero_point != 0) {
+    set_error("zero_point must be 0 for 8-bit weights, got %d", d->zero_point);
+    return false;
+  }
+  if (d->n < 0 || d->k < 0 || m < 0) {
+    set_error("negative extent: M=%lld N=%lld K=%lld", (long long)m, (long long)d->n,
+              (long long)d->k);
+    return false;
+  }
+  if (d->k % d->group != 0) {
+    set_error("K=%lld is not a multiple of the group size %d", (long long)d->k, d->group);
+    return false;
+  }
+  const int64_t w_bytes = d->n * (d->k * d->bits / 8);
+  const int64_t s_bytes = d->n * (d->k / d->group) * 2;
+  const int64_t x_bytes = m * d->k * 2;
+  if (d->n > 0x7FFFFFFF || d->k > 0x7FFFFFFF || m > 0x7FFFFFFF || w_bytes > kMaxBufferBytes ||
+      s_bytes > kMaxBufferBytes || x_bytes > kMaxBufferBytes) {
+    set_error("operand too large (each of x, wq, scales must stay below 2 GiB): M=%lld N=%lld K=%lld",
+              (long long)m, (long long)d->n, (long long)d->k);
+    return false;
+  }
+  return true;
+}
+
+bool check_ptr(const void* p, const char* name, size_t align) {
+  if (p == nullptr) {
+    set_error("%s is NULL", name);
+    return false;
+  }
+  if (reinterpret_cast<uintptr_t>(p) % align != 0) {
+    set_error("%s (%p) is not %zu-byte aligned", name, p, align);
+    return false;
+  }
+  return true;
+}
+
+int select_kernel(const mi355x_wq_desc*, int64_t m) {
+  return m <= kSkinnyMaxM ? MI355X_WQ_KERNEL_SKINNY : MI355X_WQ_KERNEL_GEMM;
+}
+
+}  // namespace
+}  // namespace wq
+
+extern "C" {
+
+const char* mi355x_wq_last_error(void) { return wq::g_error; }
+
+int mi355x_wq_version(void) { return 0 * 10000 + 1 * 100 + 0; }
+
+int mi355x_wq_check(const mi355x_wq_desc* desc, int64_t m) {
+  return wq::check_desc(desc, m) ? 0 : -1;
+}
+
+int mi355x_wq_select_kernel(const mi355x_wq_desc* desc, int64_t m) {
+  if (!wq::check_desc(desc, m)) return -1;
+  return wq::select_kernel(desc, m);
+}
+
+int mi355x_wq_matmul_ex(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
+                        void* y, int64_t m, void* stream, int kernel) {
+  using namespace wq;
+  if (!check_desc(desc, m)) return -1;
+  if (m == 0 || desc->n == 0) return 0;  // empty output
+  if (desc->k == 0) {
+    set_error("K = 0 is not supported (the output would be all zeros)");
+    return -1;
+  }
+  if (!check_ptr(x, "x", 16) || !check_ptr(wq_, "wq", 16) || !check_ptr(scales, "scales", 2) ||
+      !check_ptr(y, "y", 2))
+    return -1;
+  const int family = kernel & 0xFF, variant = (kernel >> 8) & 0xFF;
+  Problem p{x, wq_, scales, y, m, desc->n, desc->k, desc->bits, desc->group, desc->zero_point,
+            static_cast<hipStream_t>(stream)};
+  int chosen = family == MI355X_WQ_KERNEL_AUTO ? select_kernel(desc, m) : family;
+  switch (chosen) {
+    case MI355X_WQ_KERNEL_SKINNY: return launch_skinny(p, variant);
+    case MI355X_WQ_KERNEL_GEMM: return launch_gemm(p, variant);
+    default: set_error("unknown kernel family %d", family); return -1;
+  }
+}
+
+int mi355x_wq_matmul(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
+                     void* y, int64_t m, void* stream) {
+  return mi355x_wq_matmul_ex(desc, x, wq_, scales, y, m, stream, MI355X_WQ_KERNEL_AUTO);
+}
+
+int mi355x_wq_dequantize(const mi355x_wq_desc* desc, const void* wq_, const void* scales, void* wd,
+                         void* stream) {
+  using namespace wq;
+  if (!check_desc(desc, 0)) return -1;
+  if (desc->n == 0 || desc->k == 0) return 0;
+  if (!check_ptr(wq_, "wq", 16) || !check_ptr(scales, "scales", 2) || !check_ptr(wd, "wd", 16))
+    return -1;
+  Problem p{nullptr, wq_, scales, nullptr, 0, desc->n, desc->k, desc->bits, desc->group,
+            desc->zero_point, static_cast<hipStream_t>(stream)};
+  return launch_dequant(p, wd);
+}
+
+}  // extern "C"

@@ -1,0 +1,127 @@
+// Device-side building blocks shared by the gfx950 kernels: vector types, raw
+// buffer loads (out-of-range lanes read 0, which removes every tail branch from
+// the hot loops) and the exact int4/int8 -> float16 conversions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace wq {
+
+typedef _Float16 half_t;
+typedef half_t half2_t __attribute__((ext_vector_type(2)));
+typedef half_t half4_t __attribute__((ext_vector_type(4)));
+typedef half_t half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// An offset no buffer of this library can contain (sizes are checked < 2^31 on
+// the host): a lane that must not load uses it and receives zeros.
+constexpr uint32_t kOobOffset = 0x80000000u;
+
+__device__ __forceinline__ half2_t as_h2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+__device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
+__device__ __forceinline__ half2_t bcast_h2(half_t s) { return half2_t{s, s}; }
+
+// ---- raw buffer access ------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  // dword3 0x00020000: 32-bit untyped data format, raw (stride 0) addressing.
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 load_b128(rsrc_t r, uint32_t voff) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0);
+}
+__device__ __forceinline__ u32x2 load_b64(rsrc_t r, uint32_t voff) {
+  return __builtin_amdgcn_raw_buffer_load_b64(r, voff, 0, 0);
+}
+__device__ __forceinline__ uint32_t load_b32(rsrc_t r, uint32_t voff) {
+  return __builtin_amdgcn_raw_buffer_load_b32(r, voff, 0, 0);
+}
+__device__ __forceinline__ uint32_t load_b16(rsrc_t r, uint32_t voff) {
+  return __builtin_amdgcn_raw_buffer_load_b16(r, voff, 0, 0);
+}
+
+// (a & mask) | bits in one VALU op; mask must be wave-uniform (SGPR operand).
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t bits) {
+  uint32_t d;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(bits));
+  return d;
+}
+
+// ---- exact integer -> float16 conversions -------------------------------------
+// A float16 with exponent field 25 (0x6400) has a unit in the last place of 1:
+// OR-ing a 4-bit field into mantissa bits 0..3 yields exactly 1024 + field, and
+// into bits 4..7 exactly 1024 + 16*field.  Subtracting the offset (and the zero
+// point) is exact because the result is a small integer, so the only rounding in
+// the whole dequantization is the final multiply by the scale -- the same single
+// rounding the CPU path performs.
+struct Q4Consts {
+  uint32_t magic;   // 0x64006400, kept in a VGPR (gfx9 VOP3 reads one SGPR)
+  half2_t sub_lo;   // 1024 + zero_point, both halves
+  half2_t mul_hi;   // 1/16
+  half2_t sub_hi;   // 64 + zero_point
+  half2_t mix_mul;  // (1, 1/16)
+  half2_t mix_sub;  // (1024 + zp, 64 + zp)
+};
+
+__device__ __forceinline__ Q4Consts make_q4_consts(int zero_point) {
+  Q4Consts c;
+  c.magic = 0x64006400u;
+  asm volatile("" : "+v"(c.magic));  // keep it a register, not a literal
+  half_t lo = (half_t)(1024 + zero_point), hi = (half_t)(64 + zero_point);
+  c.sub_lo = half2_t{lo, lo};
+  c.mul_hi = half2_t{(half_t)0.0625f, (half_t)0.0625f};
+  c.sub_hi = half2_t{hi, hi};
+  c.mix_mul = half2_t{(half_t)1.0f, (half_t)0.0625f};
+  c.mix_sub = half2_t{lo, hi};
+  return c;
+}
+
+// One packed word -> 4 half2 holding (field - zp) * scale, in the pair order
+// (k0,k4) (k1,k5) (k2,k6) (k3,k7).  13 VALU ops per word.
+__device__ __forceinline__ void q4_word_paired(uint32_t w, half2_t s2, const Q4Consts& c,
+                                               half2_t out[4]) {
+  uint32_t w8 = w >> 8;
+  half2_t a0 = as_h2(and_or(w, 0x000F000Fu, c.magic)) - c.sub_lo;
+  half2_t a1 = __builtin_elementwise_fma(as_h2(and_or(w, 0x00F000F0u, c.magic)), c.mul_hi, -c.sub_hi);
+  half2_t a2 = as_h2(and_or(w8, 0x000F000Fu, c.magic)) - c.sub_lo;
+  half2_t a3 = __builtin_elementwise_fma(as_h2(and_or(w8, 0x00F000F0u, c.magic)), c.mul_hi, -c.sub_hi);
+  out[0] = a0 * s2;
+  out[1] = a1 * s2;
+  out[2] = a2 * s2;
+  out[3] = a3 * s2;
+}
+
+// One packed word -> 4 half2 in natural order (k0,k1) (k2,k3) (k4,k5) (k6,k7).
+// Byte i of the word is copied under both halves (v_perm), the low half keeps
+// field 2i at mantissa bits 0..3 and the high half field 2i+1 at bits 4..7.
+// 16 VALU ops per word.
+__device__ __forceinline__ void q4_word_natural(uint32_t w, half2_t s2, const Q4Consts& c,
+                                                half2_t out[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint32_t t = __builtin_amdgcn_perm(0u, w, 0x0c000c00u | (uint32_t)i | ((uint32_t)i << 16));
+    half2_t h = as_h2(and_or(t, 0x00F0000Fu, c.magic));
+    out[i] = __builtin_elementwise_fma(h, c.mix_mul, -c.mix_sub) * s2;
+  }
+}
+
+// int8: byte b (two's complement) xor 0x80 = b + 128 as an unsigned byte, so
+// 0x6400 | (byte ^ 0x80) is exactly 1152 + b.  One word -> 2 half2, natural order.
+// 8 VALU ops per word.
+__device__ __forceinline__ void q8_word_natural(uint32_t w, half2_t s2, half2_t out[2]) {
+  const half2_t off = half2_t{(half_t)1152.0f, (half_t)1152.0f};
+  uint32_t t0 = __builtin_amdgcn_perm(0u, w, 0x0c010c00u) ^ 0x64806480u;
+  uint32_t t1 = __builtin_amdgcn_perm(0u, w, 0x0c030c02u) ^ 0x64806480u;
+  out[0] = (as_h2(t0) - off) * s2;
+  out[1] = (as_h2(t1) - off) * s2;
+}
+
+__device__ __forceinline__ half8_t pack_h8(half2_t a, half2_t b, half2_t c, half2_t d) {
+  return half8_t{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+}
+
+}  // namespace wq

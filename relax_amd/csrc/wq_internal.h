@@ -1,0 +1,29 @@
+// Host-side contract between the C ABI (wq_capi.cpp) and the kernel launchers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace wq {
+
+struct Problem {
+  const void* x;
+  const void* wq;
+  const void* scales;
+  void* y;
+  int64_t m, n, k;
+  int bits, group, zero_point;
+  hipStream_t stream;
+};
+
+// Tuning variant: 0 = library default for the shape, >0 = explicit choice
+// (only reachable through mi355x_wq_matmul_ex; used by sweeps).
+int launch_skinny(const Problem& p, int variant);
+int launch_gemm(const Problem& p, int variant);
+int launch_dequant(const Problem& p, void* wd);
+
+// Upper bound of rows the skinny family accepts.
+constexpr int64_t kSkinnyMaxM = 64;
+
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+
+}  // namespace wq

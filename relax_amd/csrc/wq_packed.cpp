@@ -1,0 +1,256 @@
+// TVM PackedFunc boundary (include/mi355x_wq_packed.h): unpacks DLPack tensors
+// handed over by Relax's VM, validates them and forwards to the C ABI.
+#include <dlfcn.h>
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/mi355x_wq.h"
+#include "../../include/mi355x_wq_packed.h"
+#include "wq_internal.h"
+
+namespace {
+
+thread_local void* g_stream = nullptr;
+
+// Report through TVM's error slot when the host process has one, so that the
+// loader's `LOG(FATAL) << TVMGetLastError()` shows our message.
+int fail() {
+  typedef void (*set_last_error_t)(const char*);
+  static set_last_error_t fn =
+      reinterpret_cast<set_last_error_t>(dlsym(RTLD_DEFAULT, "TVMAPISetLastError"));
+  if (fn != nullptr) fn(mi355x_wq_last_error());
+  return -1;
+}
+
+struct Dtype {
+  uint8_t code, bits;
+  const char* name;
+};
+constexpr Dtype kF16{2, 16, "float16"};
+constexpr Dtype kU32{1, 32, "uint32"};
+
+// Checks one tensor argument; on success stores the (byte_offset adjusted) pointer.
+bool take_tensor(mi355x_tvm_value* args, int* type_codes, int idx, const char* role, Dtype want,
+                 int device_id_expected, const mi355x_dl_tensor** out, void** ptr) {
+  const int tc = type_codes[idx];
+  if (tc != MI355X_TVM_DLTENSOR_HANDLE && tc != MI355X_TVM_NDARRAY_HANDLE) {
+    wq::set_error("argument %d (%s): expected a tensor (type code 7 or 13), got type code %d", idx,
+                  role, tc);
+    return false;
+  }
+  const mi355x_dl_tensor* t = static_cast<const mi355x_dl_tensor*>(args[idx].v_handle);
+  if (t == nullptr) {
+    wq::set_error("argument %d (%s): NULL tensor handle", idx, role);
+    return false;
+  }
+  if (t->ndim != 2 || t->shape == nullptr) {
+    wq::set_error("argument %d (%s): expected a 2-d tensor, got ndim=%d", idx, role, t->ndim);
+    return false;
+  }
+  if (t->dtype.code != want.code || t->dtype.bits != want.bits || t->dtype.lanes != 1) {
+    wq::set_error("argument %d (%s): expected dtype %s, got code=%d bits=%d lanes=%d", idx, role,
+                  want.name, t->dtype.code, t->dtype.bits, t->dtype.lanes);
+    return false;
+  }
+  if (t->device.device_type != MI355X_DL_ROCM) {
+    wq::set_error("argument %d (%s): expected a ROCm tensor (device type 10), got device type %d",
+                  idx, role, t->device.device_type);
+    return false;
+  }
+  if (device_id_expected >= 0 && t->device.device_id != device_id_expected) {
+    wq::set_error("argument %d (%s): on device %d but the first tensor is on device %d", idx, role,
+                  t->device.device_id, device_id_expected);
+    return false;
+  }
+  if (t->shape[0] < 0 || t->shape[1] < 0) {
+    wq::set_error("argument %d (%s): negative extent", idx, role);
+    return false;
+  }
+  if (t->strides != nullptr) {
+    // only compact row-major; a stride is irrelevant where the extent is 1
+    const bool ok1 = t->shape[1] <= 1 || t->strides[1] == 1;
+    const bool ok0 = t->shape[0] <= 1 || t->strides[0] == t->shape[1];
+    if (!ok0 || !ok1) {
+      wq::set_error("argument %d (%s): strides (%lld, %lld) are not compact row-major for shape (%lld, %lld)",
+                    idx, role, (long long)t->strides[0], (long long)t->strides[1],
+                    (long long)t->shape[0], (long long)t->shape[1]);
+      return false;
+    }
+  }
+  if (t->data == nullptr && t->shape[0] * t->shape[1] != 0) {
+    wq::set_error("argument %d (%s): NULL data pointer", idx, role);
+    return false;
+  }
+  *out = t;
+  *ptr = static_cast<char*>(t->data) + t->byte_offset;
+  return true;
+}
+
+}  // namespace
+
+extern "C" {
+
+void mi355x_wq_packed_set_stream(void* stream) { g_stream = stream; }
+void* mi355x_wq_packed_get_stream(void) { return g_stream; }
+
+int mi355x_wq_packed_call(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes,
+                          int num_args) {
+  if (spec == nullptr) {
+    wq::set_error("call spec is NULL");
+    return fail();
+  }
+  const bool is_matmul = spec->op == 0;
+  if (spec->op != 0 && spec->op != 1) {
+    wq::set_error("call spec: unknown op %d", spec->op);
+    return fail();
+  }
+  const int expect = is_matmul ? 4 : 3;
+  if (num_args != expect || spec->num_args != expect) {
+    wq::set_error("%s expects %d arguments, got %d", is_matmul ? "matmul" : "dequantize", expect,
+                  num_args);
+    return fail();
+  }
+  if (args == nullptr || type_codes == nullptr) {
+    wq::set_error("NULL argument array");
+    return fail();
+  }
+  // role indices must be a permutation of 0..expect-1
+  int roles[4] = {spec->arg_wq, spec->arg_scales, spec->arg_out, spec->arg_x};
+  unsigned seen = 0;
+  for (int i = 0; i < expect; ++i) {
+    if (roles[i] < 0 || roles[i] >= expect || (seen & (1u << roles[i]))) {
+      wq::set_error("call spec: argument roles are not a permutation of 0..%d", expect - 1);
+      return fail();
+    }
+    seen |= 1u << roles[i];
+  }
+
+  const mi355x_dl_tensor *tx = nullptr, *tw = nullptr, *ts = nullptr, *to = nullptr;
+  void *px = nullptr, *pw = nullptr, *ps = nullptr, *po = nullptr;
+  if (!take_tensor(args, type_codes, spec->arg_wq, "wq", kU32, -1, &tw, &pw)) return fail();
+  const int dev = tw->device.device_id;
+  if (!take_tensor(args, type_codes, spec->arg_scales, "scales", kF16, dev, &ts, &ps)) return fail();
+  if (!take_tensor(args, type_codes, spec->arg_out, is_matmul ? "y" : "wd", kF16, dev, &to, &po))
+    return fail();
+  if (is_matmul && !take_tensor(args, type_codes, spec->arg_x, "x", kF16, dev, &tx, &px)) return fail();
+
+  const int per_word = 32 / (spec->bits == 8 ? 8 : 4);
+  mi355x_wq_desc d;
+  memset(&d, 0, sizeof(d));
+  d.bits = spec->bits;
+  d.zero_point = spec->zero_point;
+  d.n = tw->shape[0];
+  d.k = tw->shape[1] * per_word;
+  if (ts->shape[0] != d.n) {
+    wq::set_error("scales has %lld rows but wq has %lld", (long long)ts->shape[0], (long long)d.n);
+    return fail();
+  }
+  if (spec->group > 0) {
+    d.group = spec->group;
+    if (d.k % d.group != 0 || ts->shape[1] != d.k / d.group) {
+      wq::set_error("scales shape (%lld, %lld) does not match K=%lld / group=%d", (long long)ts->shape[0],
+                    (long long)ts->shape[1], (long long)d.k, d.group);
+      return fail();
+    }
+  } else {
+    if (ts->shape[1] <= 0 || d.k % ts->shape[1] != 0) {
+      wq::set_error("cannot infer the group size: K=%lld, scales has %lld columns", (long long)d.k,
+                    (long long)ts->shape[1]);
+      return fail();
+    }
+    d.group = (int32_t)(d.k / ts->shape[1]);
+  }
+
+  int64_t m = 0;
+  if (is_matmul) {
+    m = tx->shape[0];
+    if (tx->shape[1] != d.k) {
+      wq::set_error("x has %lld columns but the weights have K=%lld", (long long)tx->shape[1],
+                    (long long)d.k);
+      return fail();
+    }
+    if (to->shape[0] != m || to->shape[1] != d.n) {
+      wq::set_error("y has shape (%lld, %lld), expected (%lld, %lld)", (long long)to->shape[0],
+                    (long long)to->shape[1], (long long)m, (long long)d.n);
+      return fail();
+    }
+  } else if (to->shape[0] != d.n || to->shape[1] != d.k) {
+    wq::set_error("wd has shape (%lld, %lld), expected (%lld, %lld)", (long long)to->shape[0],
+                  (long long)to->shape[1], (long long)d.n, (long long)d.k);
+    return fail();
+  }
+  if (mi355x_wq_check(&d, m) != 0) return fail();
+  if (d.n == 0 || (is_matmul && m == 0)) return 0;  // nothing to compute
+
+  int cur = -1;
+  if (hipGetDevice(&cur) != hipSuccess) {
+    (void)hipGetLastError();
+    wq::set_error("no usable HIP device in this process");
+    return fail();
+  }
+  if (cur != dev) {
+    wq::set_error("tensors live on ROCm device %d but the current HIP device is %d", dev, cur);
+    return fail();
+  }
+  const int rc = is_matmul ? mi355x_wq_matmul(&d, px, pw, ps, po, m, g_stream)
+                           : mi355x_wq_dequantize(&d, pw, ps, po, g_stream);
+  return rc == 0 ? 0 : fail();
+}
+
+#define MI355X_FIXED_ENTRY(NAME, OP, BITS, ZP)                                                    \
+  int NAME(mi355x_tvm_value* args, int* type_codes, int num_args, mi355x_tvm_value*, int*, void*) { \
+    static const mi355x_wq_callspec spec = {OP, BITS, 0, ZP, 0, (OP) == 0 ? 1 : 0, (OP) == 0 ? 2 : 1, \
+                                            (OP) == 0 ? 3 : 2, (OP) == 0 ? 4 : 3};                \
+    return mi355x_wq_packed_call(&spec, args, type_codes, num_args);                              \
+  }
+MI355X_FIXED_ENTRY(mi355x_q4f16_matmul, 0, 4, 7)
+MI355X_FIXED_ENTRY(mi355x_q8f16_matmul, 0, 8, 0)
+MI355X_FIXED_ENTRY(mi355x_q4f16_dequantize, 1, 4, 7)
+MI355X_FIXED_ENTRY(mi355x_q8f16_dequantize, 1, 8, 0)
+#undef MI355X_FIXED_ENTRY
+
+// ---- registration in TVM's global table through its C API -----------------------
+typedef int (*backend_fn_t)(mi355x_tvm_value*, int*, int, mi355x_tvm_value*, int*, void*);
+
+// TVMPackedCFunc has (args, type_codes, num_args, ret, resource_handle); the
+// resource handle carries the backend-style entry to call.
+static int registry_adapter(mi355x_tvm_value* args, int* type_codes, int num_args, void* /*ret*/,
+                            void* resource_handle) {
+  backend_fn_t fn = reinterpret_cast<backend_fn_t>(resource_handle);
+  return fn(args, type_codes, num_args, nullptr, nullptr, nullptr);
+}
+
+int mi355x_wq_register_tvm_globals(int allow_override) {
+  typedef int (*adapter_t)(mi355x_tvm_value*, int*, int, void*, void*);
+  typedef int (*create_t)(adapter_t, void*, void (*)(void*), void**);
+  typedef int (*register_t)(const char*, void*, int);
+  create_t create = reinterpret_cast<create_t>(dlsym(RTLD_DEFAULT, "TVMFuncCreateFromCFunc"));
+  register_t reg = reinterpret_cast<register_t>(dlsym(RTLD_DEFAULT, "TVMFuncRegisterGlobal"));
+  if (create == nullptr || reg == nullptr) {
+    wq::set_error("no TVM runtime is loaded in this process (TVMFuncCreateFromCFunc not found)");
+    return -1;
+  }
+  struct Entry {
+    const char* name;
+    backend_fn_t fn;
+  };
+  const Entry entries[] = {{"mi355x.q4f16_matmul", mi355x_q4f16_matmul},
+                           {"mi355x.q8f16_matmul", mi355x_q8f16_matmul},
+                           {"mi355x.q4f16_dequantize", mi355x_q4f16_dequantize},
+                           {"mi355x.q8f16_dequantize", mi355x_q8f16_dequantize}};
+  int count = 0;
+  for (const Entry& e : entries) {
+    void* handle = nullptr;
+    if (create(registry_adapter, reinterpret_cast<void*>(e.fn), nullptr, &handle) != 0 ||
+        reg(e.name, handle, allow_override) != 0) {
+      wq::set_error("registering %s in the TVM global table failed", e.name);
+      return -1;
+    }
+    ++count;
+  }
+  return count;
+}
+
+}  // extern "C"

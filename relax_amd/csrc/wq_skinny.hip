@@ -1,0 +1,241 @@
+// Skinny (GEMV-class) kernel for M <= 64: y[M,N] = x[M,K] @ dequant(Wq,S)^T.
+//
+// Bound: HBM bandwidth.  Each byte of packed weight is read exactly once with a
+// 16-byte buffer load per lane, dequantized in registers (exactly the float16
+// value the CPU path materialises) and consumed by v_mfma_f32_16x16x32_f16 with
+// the activations as the other operand, so the same kernel serves M = 1 .. 64
+// without the VALU ever becoming the limit at large M.
+//
+// Work split: a workgroup owns R row tiles of 16 output features; its WAVES
+// wavefronts split K between them and add their partial tiles through LDS.
+// Inside a wavefront, lane (col = lane % 16, kq = lane / 16) owns weight row
+// `col` of the tile and the kq-th 16-byte chunk of every 64-byte row segment, so
+// one load instruction covers 16 rows x 64 contiguous bytes.
+//
+// Tails never branch: activation rows >= M, chunks >= K and k-steps past the
+// wavefront's share are loaded from an out-of-range buffer offset, which returns
+// zeros (zero scale => zero weight, zero activation); weight rows >= N are
+// clamped to the last row and their results are not stored.
+#include "wq_device.h"
+#include "wq_internal.h"
+
+namespace wq {
+
+template <int BITS, int R, int MT, int U>
+struct SkinnyBatch {
+  static constexpr int NJ = (128 / BITS) / 8;
+  u32x4 w[U][R];
+  uint32_t sc[U][R];
+  u32x4 xa[U][MT][NJ];
+};
+
+template <int BITS, int R, int MT, int WAVES, int U>
+__global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
+    const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
+    half_t* __restrict__ y, int M, int N, int K, int group_shift, int zero_point) {
+  constexpr int CH = 128 / BITS;  // k covered by one 16-byte lane load: 32 / 16
+  constexpr int NJ = CH / 8;      // MFMAs fed by one lane load: 4 / 2
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int col = lane & 15;
+  const int kq = lane >> 4;
+
+  const uint32_t row_bytes = (uint32_t)K * BITS / 8;
+  const int nchunks = K / CH;
+  const int nsteps = (nchunks + 3) >> 2;
+  const int per_wave = (nsteps + WAVES - 1) / WAVES;
+  const int ks_begin = wave * per_wave;
+  const int ks_end = min(ks_begin + per_wave, nsteps);
+  const uint32_t groups_per_row = (uint32_t)nchunks >> group_shift;
+
+  const rsrc_t rw = make_rsrc(wq, (uint32_t)N * row_bytes);
+  const rsrc_t rs = make_rsrc(scales, (uint32_t)N * groups_per_row * 2u);
+  const rsrc_t rx = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
+
+  // per-lane row bases.  Weight rows past N are clamped to the last row (their
+  // results are never stored); activation rows past M read zeros.
+  uint32_t wbase[R], sbase[R], xbase[MT];
+  bool xrow_ok[MT];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int n = min((int)(blockIdx.x * R + r) * 16 + col, N - 1);
+    wbase[r] = (uint32_t)n * row_bytes;
+    sbase[r] = (uint32_t)n * groups_per_row * 2u;
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + col;
+    xrow_ok[mt] = m < M;
+    xbase[mt] = (uint32_t)m * (uint32_t)K * 2u;
+  }
+
+  float4_t acc[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[r][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  Q4Consts qc = make_q4_consts(zero_point);
+
+  auto load_batch = [&](SkinnyBatch<BITS, R, MT, U>& b, int ks0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int ks = ks0 + u;
+      const int chunk = ks * 4 + kq;
+      const bool ok = (ks < ks_end) && (chunk < nchunks);
+      const uint32_t winc = ok ? (uint32_t)chunk * 16u : kOobOffset;
+      const uint32_t sinc = ok ? ((uint32_t)chunk >> group_shift) * 2u : kOobOffset;
+      const uint32_t xinc = (uint32_t)chunk * (CH * 2u);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        b.w[u][r] = load_b128(rw, wbase[r] + winc);  // valid base < 2^31: the sum cannot wrap
+        b.sc[u][r] = load_b16(rs, sbase[r] + sinc);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const uint32_t xo = (ok && xrow_ok[mt]) ? xbase[mt] + xinc : kOobOffset;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) b.xa[u][mt][j] = load_b128(rx, xo + j * 16u);
+      }
+    }
+  };
+
+  auto compute_batch = [&](const SkinnyBatch<BITS, R, MT, U>& b) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      half8_t a[MT][NJ];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+          const u32x4 v = b.xa[u][mt][j];
+          if constexpr (BITS == 4) {
+            // activations follow the weight pair order (k0,k4)(k1,k5)(k2,k6)(k3,k7)
+            u32x4 p;
+            p[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
+            p[1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
+            p[2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
+            p[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
+            a[mt][j] = __builtin_bit_cast(half8_t, p);
+          } else {
+            a[mt][j] = __builtin_bit_cast(half8_t, v);
+          }
+        }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const half2_t s2 = bcast_h2(__builtin_bit_cast(half_t, (uint16_t)b.sc[u][r]));
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+          half8_t bm;
+          if constexpr (BITS == 4) {
+            half2_t h[4];
+            q4_word_paired(b.w[u][r][j], s2, qc, h);
+            bm = pack_h8(h[0], h[1], h[2], h[3]);
+          } else {
+            half2_t h0[2], h1[2];
+            q8_word_natural(b.w[u][r][2 * j], s2, h0);
+            q8_word_natural(b.w[u][r][2 * j + 1], s2, h1);
+            bm = pack_h8(h0[0], h0[1], h1[0], h1[1]);
+          }
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt][j], bm, acc[r][mt], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  // register double buffering: the next batch is in flight while this one is consumed
+  SkinnyBatch<BITS, R, MT, U> b0, b1;
+  load_batch(b0, ks_begin);
+  for (int ks = ks_begin; ks < ks_end; ks += 2 * U) {
+    load_batch(b1, ks + U);
+    compute_batch(b0);
+    load_batch(b0, ks + 2 * U);
+    compute_batch(b1);
+  }
+
+  // cross-wave reduction of the K split
+  __shared__ float red[WAVES][R * MT][4][64];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][r * MT + mt][i][lane] = acc[r][mt][i];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < R * MT * 256; idx += WAVES * 64) {
+    const int t = idx >> 8, i = (idx >> 6) & 3, l = idx & 63;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) sum += red[w][t][i][l];
+    const int r = t / MT, mt = t % MT;
+    const int m = mt * 16 + 4 * (l >> 4) + i;
+    const int n = (blockIdx.x * R + r) * 16 + (l & 15);
+    if (m < M && n < N) y[(size_t)m * N + n] = (half_t)sum;
+  }
+}
+
+namespace {
+
+template <int BITS, int R, int MT, int WAVES, int U>
+void launch_one(const Problem& p, int group_shift) {
+  const int tiles = (int)((p.n + 15) / 16);
+  dim3 grid((tiles + R - 1) / R), block(WAVES * 64);
+  hipLaunchKernelGGL((wq_skinny_kernel<BITS, R, MT, WAVES, U>), grid, block, 0, p.stream,
+                     (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
+                     (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point);
+}
+
+template <int BITS, int MT>
+bool dispatch_variant(const Problem& p, int group_shift, int variant) {
+  switch (variant) {
+    case 1: launch_one<BITS, 1, MT, 4, 2>(p, group_shift); return true;
+    case 2: launch_one<BITS, 2, MT, 4, 2>(p, group_shift); return true;
+    case 3: launch_one<BITS, 1, MT, 8, 2>(p, group_shift); return true;
+    case 4: launch_one<BITS, 1, MT, 4, 4>(p, group_shift); return true;
+    case 5: launch_one<BITS, 2, MT, 8, 1>(p, group_shift); return true;
+    case 6: launch_one<BITS, 1, MT, 8, 1>(p, group_shift); return true;
+    default: return false;
+  }
+}
+
+}  // namespace
+
+int launch_skinny(const Problem& p, int variant) {
+  const int ch = 128 / p.bits;
+  int ratio = p.group / ch, group_shift = 0;
+  while ((1 << group_shift) < ratio) ++group_shift;
+  if (ratio < 1 || (1 << group_shift) != ratio || p.group % ch != 0) {
+    set_error("skinny kernel: group %d must be %d times a power of two", p.group, ch);
+    return -1;
+  }
+  if (p.m > kSkinnyMaxM) {
+    set_error("skinny kernel: M = %lld exceeds %lld", (long long)p.m, (long long)kSkinnyMaxM);
+    return -1;
+  }
+  const int mt = (int)((p.m + 15) / 16);
+  if (variant == 0) variant = mt >= 3 ? 1 : 2;
+  bool ok;
+  if (p.bits == 4) {
+    ok = mt <= 1   ? dispatch_variant<4, 1>(p, group_shift, variant)
+         : mt == 2 ? dispatch_variant<4, 2>(p, group_shift, variant)
+                   : dispatch_variant<4, 4>(p, group_shift, variant);
+  } else {
+    ok = mt <= 1   ? dispatch_variant<8, 1>(p, group_shift, variant)
+         : mt == 2 ? dispatch_variant<8, 2>(p, group_shift, variant)
+                   : dispatch_variant<8, 4>(p, group_shift, variant);
+  }
+  if (!ok) {
+    set_error("skinny kernel: unknown variant %d", variant);
+    return -1;
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("skinny kernel launch failed: %s", hipGetErrorString(e));
+    return -1;
+  }
+  return 0;
+}
+
+}  // namespace wq

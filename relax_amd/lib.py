@@ -1,0 +1,87 @@
+"""ctypes binding of libmi355x_wq.so (the C ABI declared in include/*.h)."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+SO_PATH = os.path.join(CSRC, "libmi355x_wq.so")
+
+KERNEL_AUTO, KERNEL_SKINNY, KERNEL_GEMM = 0, 1, 2
+
+# every symbol include/mi355x_wq.h and include/mi355x_wq_packed.h declare
+EXPORTED_SYMBOLS = (
+    "mi355x_wq_matmul", "mi355x_wq_matmul_ex", "mi355x_wq_dequantize", "mi355x_wq_check",
+    "mi355x_wq_select_kernel", "mi355x_wq_last_error", "mi355x_wq_version",
+    "mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_dequantize",
+    "mi355x_q8f16_dequantize", "mi355x_wq_packed_call", "mi355x_wq_packed_set_stream",
+    "mi355x_wq_packed_get_stream", "mi355x_wq_register_tvm_globals",
+)
+
+
+class WqDesc(C.Structure):
+    """mi355x_wq_desc"""
+    _fields_ = [("bits", C.c_int32), ("group", C.c_int32), ("zero_point", C.c_int32),
+                ("reserved", C.c_int32), ("n", C.c_int64), ("k", C.c_int64)]
+
+
+class WqError(RuntimeError):
+    """A call into the library returned -1; the message is the library's own."""
+
+
+_lib = None
+
+
+def build(verbose: bool = False) -> str:
+    """Compile the library for gfx950 in-tree (hipcc cross-compiles without a GPU)."""
+    cmd = ["make", "-B", "-j8", "-C", CSRC, "libmi355x_wq.so"]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if verbose or res.returncode != 0:
+        print(res.stdout)
+    if res.returncode != 0:
+        raise RuntimeError("building libmi355x_wq.so failed")
+    return SO_PATH
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(SO_PATH):
+        raise ImportError(
+            f"{SO_PATH} is missing: build it with `make -C {CSRC}` "
+            "(or __graft_entry__.build()); there is no fallback path")
+    L = C.CDLL(SO_PATH)
+    vp, i64, ci = C.c_void_p, C.c_int64, C.c_int
+    dp = C.POINTER(WqDesc)
+    L.mi355x_wq_matmul.argtypes = [dp, vp, vp, vp, vp, i64, vp]
+    L.mi355x_wq_matmul_ex.argtypes = [dp, vp, vp, vp, vp, i64, vp, ci]
+    L.mi355x_wq_dequantize.argtypes = [dp, vp, vp, vp, vp]
+    L.mi355x_wq_check.argtypes = [dp, i64]
+    L.mi355x_wq_select_kernel.argtypes = [dp, i64]
+    L.mi355x_wq_last_error.restype = C.c_char_p
+    L.mi355x_wq_packed_set_stream.argtypes = [vp]
+    L.mi355x_wq_packed_get_stream.restype = vp
+    L.mi355x_wq_register_tvm_globals.argtypes = [ci]
+    for name in ("mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_dequantize",
+                 "mi355x_q8f16_dequantize"):
+        getattr(L, name).argtypes = [vp, C.POINTER(ci), ci, vp, C.POINTER(ci), vp]
+    L.mi355x_wq_packed_call.argtypes = [vp, vp, C.POINTER(ci), ci]
+    _lib = L
+    return L
+
+
+def last_error() -> str:
+    return load().mi355x_wq_last_error().decode()
+
+
+def make_desc(bits: int, group: int, n: int, k: int, zero_point: int | None = None) -> WqDesc:
+    if zero_point is None:
+        zero_point = 7 if bits == 4 else 0
+    return WqDesc(bits, group, zero_point, 0, n, k)
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise WqError(last_error())

@@ -1,0 +1,34 @@
+"""Writes the golden fixtures (inputs + oracle outputs) used by the CPU and GPU tests.
+
+The reference holds no vectors for a quantized matmul (it has no such operator), so the
+fixtures are outputs of the pinned CPU oracle on seeded inputs; they freeze the layout
+(least-significant field first) and the rounding sequence.  Run from the repo root:
+
+    python tests/golden/make_golden.py
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from oracle import wq_oracle as O  # noqa: E402
+
+CASES = [  # name, seed, M, N, K, bits, group
+    ("q4f16_m3_n48_k96", 11, 3, 48, 96, 4, 32),
+    ("q4f16_m1_n64_k352", 12, 1, 64, 352, 4, 32),
+    ("q4f16_m70_n40_k128", 13, 70, 40, 128, 4, 32),
+    ("q8f16_m5_n40_k256", 14, 5, 40, 256, 8, 128),
+    ("q8f16_m66_n24_k384", 15, 66, 24, 384, 8, 128),
+]
+
+if __name__ == "__main__":
+    here = os.path.dirname(os.path.abspath(__file__))
+    for name, seed, m, n, k, bits, group in CASES:
+        x, wq, s, g = O.make_case(seed, m, n, k, bits, group)
+        wd = O.dequant(wq, s, bits, g)
+        y = O.wq_matmul(x, wq, s, bits, g)
+        np.savez_compressed(os.path.join(here, name + ".npz"), x=x, wq=wq, scales=s, wd=wd, y=y,
+                            bits=np.int32(bits), group=np.int32(g))
+        print(name, y.shape, float(np.abs(y).max()))

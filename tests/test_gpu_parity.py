@@ -1,0 +1,205 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle.
+
+Bar: integer unpack + dequantized weights bit-exact; float16 outputs within
+max-abs 1e-2 and relative 1e-2 of the oracle (float32 accumulation in a
+different order is the only permitted difference).
+"""
+import numpy as np
+import pytest
+
+from oracle import c_oracle, wq_oracle as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+ATOL = 1e-2
+RTOL = 1e-2
+
+
+def _dev(a: np.ndarray):
+    if a.dtype == np.uint32:
+        return torch.from_numpy(a.view(np.int32)).cuda()
+    return torch.from_numpy(a).cuda()
+
+
+def assert_close(got: np.ndarray, want: np.ndarray, what=""):
+    got64, want64 = got.astype(np.float64), want.astype(np.float64)
+    assert got.shape == want.shape, what
+    assert np.all(np.isfinite(got64)), what
+    err = np.abs(got64 - want64)
+    bound = ATOL + RTOL * np.abs(want64)
+    worst = int(np.argmax(err - bound))
+    assert np.all(err <= bound), (what, float(err.flat[worst]), float(want64.flat[worst]))
+    # the tolerance above is the contract; the kernels are expected to sit within ~1 float16 ulp
+    ulp = np.maximum(np.abs(want64), 2.0**-14) * 2.0**-10
+    assert np.mean(err <= 1.01 * ulp + 1e-6) > 0.999, (what, "more than 0.1% of outputs off by > 1 ulp")
+
+
+def run_matmul(x, wq, s, bits, group, kernel=0, variant=0):
+    import relax_amd
+
+    y = relax_amd.wq_matmul(_dev(x), _dev(wq), _dev(s), bits, group, kernel=kernel, variant=variant)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+# ------------------------------------------------------------------ dequantize: bit exact
+@pytest.mark.parametrize("bits,n,k", [(4, 64, 256), (4, 37, 352), (4, 4096, 4096), (8, 64, 256),
+                                       (8, 21, 384), (8, 5120, 5120)])
+def test_dequantize_bit_exact(bits, n, k):
+    import relax_amd
+
+    _, wq, s, g = O.make_case(10 + bits, 1, n, k, bits)
+    wd = relax_amd.wq_dequantize(_dev(wq), _dev(s), bits, g)
+    torch.cuda.synchronize()
+    want = c_oracle.dequant(wq, s, bits, g, nthreads=8)
+    assert np.array_equal(wd.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_dequantize_every_field_value_and_special_scales(bits):
+    """All field values against scales that give zeros, subnormals, the largest finite value and inf."""
+    import relax_amd
+
+    g = 32 if bits == 4 else 128
+    special = np.array([0.0, -0.0, 1.0, -1.0, 6e-8, 1e-5, 6.1e-5, 0.0123, 511.75, 8188.0, 65504.0, np.inf],
+                       dtype=np.float16)
+    n, groups = 16 if bits == 4 else 256, special.size
+    if bits == 4:
+        w = np.repeat(np.arange(16)[:, None], groups * g, axis=1)
+        wq = O.pack_q4(w)
+    else:
+        w = np.repeat((np.arange(256) - 128)[:, None], groups * g, axis=1)
+        wq = O.pack_q8(w)
+    s = np.repeat(special[None, :], n, axis=0)
+    got = relax_amd.wq_dequantize(_dev(wq), _dev(s), bits, g).cpu().numpy()
+    want = O.dequant(wq, s, bits, g)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+
+
+# ------------------------------------------------------------------ skinny (GEMV-class) kernel
+SKINNY_VARIANTS = [1, 2, 3, 4, 5, 6]
+
+
+@pytest.mark.parametrize("variant", SKINNY_VARIANTS)
+@pytest.mark.parametrize("bits,m,n,k", [
+    (4, 1, 64, 256), (4, 1, 40, 352), (4, 3, 16, 32), (4, 8, 200, 1024), (4, 16, 48, 2048),
+    (4, 17, 33, 352), (4, 33, 64, 512), (4, 64, 80, 1152),
+    (8, 1, 64, 256), (8, 2, 40, 384), (8, 16, 24, 128), (8, 20, 72, 640), (8, 64, 16, 1280),
+])
+def test_skinny_kernel_matches_oracle(variant, bits, m, n, k):
+    from relax_amd import lib
+
+    x, wq, s, g = O.make_case(100 + m + n, m, n, k, bits)
+    got = run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_SKINNY, variant=variant)
+    want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=8)
+    assert_close(got, want, (variant, bits, m, n, k))
+
+
+def test_config1_single_gemv_4096():
+    """The reference's CPU-runnable case: x[1,4096] ~ N(0,1), W int4 4096x4096, group 32, zero point 7."""
+    x, wq, s, g = O.make_case(0, 1, 4096, 4096, 4)
+    got = run_matmul(x, wq, s, 4, g)
+    want = c_oracle.wq_matmul(x, wq, s, 4, g, nthreads=8)
+    assert_close(got, want, "config 1")
+
+
+@pytest.mark.parametrize("m", [1, 8])
+@pytest.mark.parametrize("n,k", [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)])
+def test_config2_llama7b_decode_projections(m, n, k):
+    x, wq, s, g = O.make_case(2, m, n, k, 4)
+    got = run_matmul(x, wq, s, 4, g)
+    want = c_oracle.wq_matmul(x, wq, s, 4, g, nthreads=16)
+    assert_close(got, want, ("config 2", m, n, k))
+
+
+@pytest.mark.parametrize("m", [1, 16])
+@pytest.mark.parametrize("n,k", [(5120, 5120), (5120, 13824)])
+def test_config4_q8_llama13b_skinny(m, n, k):
+    x, wq, s, g = O.make_case(4, m, n, k, 8)
+    got = run_matmul(x, wq, s, 8, g)
+    want = c_oracle.wq_matmul(x, wq, s, 8, g, nthreads=16)
+    assert_close(got, want, ("config 4", m, n, k))
+
+
+# ------------------------------------------------------------------ GEMM kernel
+@pytest.mark.parametrize("bits,m,n,k", [
+    (4, 65, 128, 64), (4, 128, 128, 512), (4, 200, 200, 352), (4, 300, 72, 96), (4, 1, 16, 32),
+    (8, 65, 128, 64), (8, 129, 136, 384), (8, 256, 256, 1152), (8, 7, 40, 16 * 9),
+])
+def test_gemm_kernel_matches_oracle(bits, m, n, k):
+    from relax_amd import lib
+
+    group = (32 if bits == 4 else 16) if k % 128 else None
+    x, wq, s, g = O.make_case(200 + m + n, m, n, k, bits, group)
+    got = run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_GEMM)
+    want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=8)
+    assert_close(got, want, (bits, m, n, k))
+
+
+@pytest.mark.parametrize("bits,m,n,k", [(4, 512, 4096, 4096), (4, 2048, 4096, 11008), (8, 256, 5120, 5120)])
+def test_gemm_full_size_rows_against_oracle_and_all_tiles_against_torch(bits, m, n, k):
+    """Full-size prefill shapes: a sample of rows against the oracle (seconds on the host), and every
+    output tile against a float32 torch matmul of the bit-exact dequantized weights."""
+    import relax_amd
+
+    x, wq, s, g = O.make_case(3, m, n, k, bits)
+    xd, wqd, sd = _dev(x), _dev(wq), _dev(s)
+    y = relax_amd.wq_matmul(xd, wqd, sd, bits, g)
+    wd = relax_amd.wq_dequantize(wqd, sd, bits, g)
+    ref = (xd.float() @ wd.float().T)
+    torch.cuda.synchronize()
+    err = (y.float() - ref).abs()
+    bound = ATOL + RTOL * ref.abs()
+    assert bool((err <= bound).all()), float((err - bound).max())
+    rows = np.random.default_rng(5).choice(m, size=4, replace=False)
+    want = c_oracle.wq_matmul(x[rows], wq, s, bits, g, nthreads=16)
+    assert_close(y.cpu().numpy()[rows], want, ("rows", bits, m, n, k))
+
+
+# ------------------------------------------------------------------ properties at full size
+def test_one_hot_rows_read_back_dequantized_weights_full_size():
+    """x = e_j: y[r, :] must equal column j of the dequantized weights exactly (no accumulation)."""
+    import relax_amd
+
+    n, k = 22016, 4096
+    _, wq, s, g = O.make_case(6, 1, n, k, 4)
+    picks = [0, 31, 32, 2047, 4095]
+    x = np.zeros((len(picks), k), dtype=np.float16)
+    for r, j in enumerate(picks):
+        x[r, j] = 1
+    got = run_matmul(x, wq, s, 4, g)
+    wd = relax_amd.wq_dequantize(_dev(wq), _dev(s), 4, g).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(wd[:, picks].T).view(np.uint16))
+
+
+def test_identical_rows_give_identical_outputs_and_kernel_families_agree():
+    from relax_amd import lib
+
+    x1, wq, s, g = O.make_case(7, 1, 4096, 4096, 4)
+    x = np.repeat(x1, 48, axis=0)
+    a = run_matmul(x, wq, s, 4, g, kernel=lib.KERNEL_SKINNY)
+    assert np.all(a.view(np.uint16) == a.view(np.uint16)[0:1])
+    b = run_matmul(x, wq, s, 4, g, kernel=lib.KERNEL_GEMM)
+    assert np.all(b.view(np.uint16) == b.view(np.uint16)[0:1])
+    assert_close(a, b.astype(np.float16), "families")
+
+
+# ------------------------------------------------------------------ golden fixtures
+def test_golden_fixtures():
+    import glob
+    import os
+
+    files = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
+    assert files, "no golden fixtures found"
+    import relax_amd
+
+    for f in files:
+        z = np.load(f)
+        bits, g = int(z["bits"]), int(z["group"])
+        got = run_matmul(z["x"], z["wq"], z["scales"], bits, g)
+        assert_close(got, z["y"], f)
+        wd = relax_amd.wq_dequantize(_dev(z["wq"]), _dev(z["scales"]), bits, g).cpu().numpy()
+        assert np.array_equal(wd.view(np.uint16), z["wd"].view(np.uint16)), f
