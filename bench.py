@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Benchmark of the weight-only-quantized matmul hot path on one MI355X.
+
+Headline workload (one "step"): the quantized projections of a Llama-2-7B decode
+pass -- 32 decoder layers, each with its own q4f16 (group 32) weights for
+(N,K) = (12288,4096) fused QKV, (4096,4096) O, (22016,4096) gate+up and
+(4096,11008) down -- run once at batch 1 and once at batch 8: 256 GEMV launches over
+3.6 GB of distinct packed weights, so no launch finds its weights in a cache.
+`value` is algorithmic bytes (packed weights + scales + x + y) per second with all
+operands resident in HBM.  The step is captured in a HIP graph so that the host's
+launch rate does not enter the figure.
+
+The same JSON line carries the prefill GEMM leg (M = 2048, the four shapes) as
+`gemm`/`roofline_gemm`, and the CPU oracle timed on the host as `cpu_baseline`.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+LLAMA7B = [("qkv", 12288, 4096), ("o", 4096, 4096), ("gate_up", 22016, 4096), ("down", 4096, 11008)]
+N_LAYERS = 32
+DECODE_BATCHES = (1, 8)
+PREFILL_M = 2048
+HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
+
+
+def algorithmic_bytes(bits: int, group: int, m: int, n: int, k: int) -> int:
+    return n * k * bits // 8 + n * (k // group) * 2 + 2 * m * k + 2 * m * n
+
+
+def cpu_baseline(quick: bool):
+    """The C oracle (scalar restatement of the CPU path) on the host cores.
+
+    Sample: every projection shape of one decoder layer at batch 1 and batch 8,
+    single-threaded, as an unscheduled llvm PrimFunc runs; then the same with
+    OpenMP over the output rows on all host cores.
+    """
+    import numpy as np
+
+    from oracle import c_oracle, wq_oracle as O
+
+    c_oracle.lib()
+    shapes = LLAMA7B[1:2] if quick else LLAMA7B
+    cases = []
+    total_bytes = 0
+    for _, n, k in shapes:
+        for m in DECODE_BATCHES:
+            cases.append(O.make_case(0, m, n, k, 4))
+            total_bytes += algorithmic_bytes(4, 32, m, n, k)
+
+    def run(nthreads):
+        t0 = time.perf_counter()
+        for x, wq, s, g in cases:
+            c_oracle.wq_matmul(x, wq, s, 4, g, nthreads=nthreads)
+        return time.perf_counter() - t0
+
+    t1 = run(1)
+    cores = min(c_oracle.max_threads(), 16)
+    tn = run(cores)
+    sample = ("one decoder layer's projections (%s) at batch 1 and 8, q4f16 g32, C oracle"
+              % ", ".join("%dx%d" % (n, k) for _, n, k in shapes))
+    return ({"value": round(total_bytes / t1 / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+             "sample": sample, "seconds": round(t1, 3)},
+            {"value": round(total_bytes / tn / 1e9, 4), "unit": "GB/s", "cores": cores, "kind": "port",
+             "sample": sample + ", OpenMP over output rows", "seconds": round(tn, 3)})
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=N_LAYERS)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the hot path is a single-GPU kernel and this build has no "
+              "multi-GPU leg (--gpus must be 1)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import relax_amd
+    from relax_amd import lib
+
+    lib.load()  # fails loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    torch.manual_seed(0)
+
+    # ---- synthetic weights: every bit pattern is a valid packed int4 row ------------------
+    layers = []
+    for _ in range(args.layers):
+        mats = []
+        for _, n, k in LLAMA7B:
+            wq = torch.randint(-2**31, 2**31 - 1, (n, k // 8), dtype=torch.int32, device=dev)
+            s = (torch.rand((n, k // 32), device=dev) * 0.015 + 0.005).to(torch.float16)
+            mats.append((wq, s, n, k))
+        layers.append(mats)
+    xs = {(m, k): torch.randn((m, k), device=dev).to(torch.float16)
+          for m in DECODE_BATCHES for k in (4096, 11008)}
+    ys = {(m, n): torch.empty((m, n), dtype=torch.float16, device=dev)
+          for m in DECODE_BATCHES for _, n, _ in LLAMA7B}
+
+    def decode_pass():
+        for m in DECODE_BATCHES:
+            for mats in layers:
+                for wq, s, n, k in mats:
+                    relax_amd.wq_matmul(xs[(m, k)], wq, s, 4, 32, out=ys[(m, n)])
+
+    launches_per_step = len(DECODE_BATCHES) * args.layers * len(LLAMA7B)
+    bytes_per_step = sum(algorithmic_bytes(4, 32, m, n, k)
+                         for m in DECODE_BATCHES for _, n, k in LLAMA7B) * args.layers
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        decode_pass()  # loads code objects, sets function attributes
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            decode_pass()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(args.steps):
+            graph.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1)
+    ms_per_step = ms / args.steps
+    gbs = bytes_per_step / (ms_per_step * 1e-3) / 1e9
+    avg_launch_us = ms_per_step * 1e3 / launches_per_step
+
+    result = {
+        "metric": "q4f16 GEMV GB/s + GEMM TFLOP/s (% roofline), Llama-7B shapes, 1 GPU",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int4 weights x f16, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "Llama-2-7B decode projections q4f16 g32, %d layers x "
+                               "{12288x4096, 4096x4096, 22016x4096, 4096x11008}, batch 1 and batch 8, "
+                               "one HIP graph per step" % args.layers,
+                   "launches_per_step": launches_per_step, "bytes_per_step": bytes_per_step},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "wq::wq_gemv_kernel (all decode launches)",
+                     "bytes_per_launch": bytes_per_step // launches_per_step,
+                     "avg_launch_us": round(avg_launch_us, 3)},
+    }
+    traffic_file = os.path.join(ROOT, "profiles", "gemv_traffic.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file) as f:
+            result["roofline"]["traffic"] = json.load(f).get("hbm_bytes_per_launch")
+
+    # ---- prefill GEMM leg: M = 2048, the four shapes, layer-rotated weights -----------------
+    if not args.no_gemm:
+        xg = {k: torch.randn((PREFILL_M, k), device=dev).to(torch.float16) for k in (4096, 11008)}
+        yg = {n: torch.empty((PREFILL_M, n), dtype=torch.float16, device=dev) for _, n, _ in LLAMA7B}
+        use = layers[:4]
+
+        def prefill_pass():
+            for mats in use:
+                for wq, s, n, k in mats:
+                    relax_amd.wq_matmul(xg[k], wq, s, 4, 32, out=yg[n])
+
+        flops = sum(2 * PREFILL_M * n * k for _, n, k in LLAMA7B) * len(use)
+        with torch.cuda.stream(stream):
+            prefill_pass()
+            torch.cuda.synchronize()
+            g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = max(2, args.steps // 4)
+            g0.record(stream)
+            for _ in range(reps):
+                prefill_pass()
+            g1.record(stream)
+            torch.cuda.synchronize()
+        gms = g0.elapsed_time(g1) / reps
+        tflops = flops / (gms * 1e-3) / 1e12
+        result["gemm"] = {"value": round(tflops, 1), "unit": "TFLOP/s", "ms_per_pass": round(gms, 4),
+                          "workload": "q4f16 g32 prefill, M=2048, the four Llama-2-7B shapes x %d layers"
+                                      % len(use)}
+        result["roofline_gemm"] = {"bound": "mfma", "achieved": round(tflops, 1),
+                                   "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                   "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                                   "kernel": "wq::wq_gemm_kernel"}
+
+    if not args.no_cpu:
+        one, omp = cpu_baseline(quick=False)
+        result["cpu_baseline"] = one
+        result["cpu_baseline_all_cores"] = omp
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

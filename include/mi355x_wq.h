@@ -48,11 +48,12 @@ typedef struct mi355x_wq_desc {
   int64_t k;          /* reduction length; multiple of `group` */
 } mi355x_wq_desc;
 
-/* Kernel families; MI355X_WQ_KERNEL_AUTO picks by M (skinny for M <= 64). */
+/* Kernel families; MI355X_WQ_KERNEL_AUTO picks by M and K. */
 enum {
   MI355X_WQ_KERNEL_AUTO = 0,
-  MI355X_WQ_KERNEL_SKINNY = 1, /* HBM-bound GEMV / skinny path, M <= 64 */
-  MI355X_WQ_KERNEL_GEMM = 2    /* LDS-tiled MFMA GEMM, any M */
+  MI355X_WQ_KERNEL_GEMV = 1,  /* HBM-bound decode path: M <= 16, activations staged in LDS */
+  MI355X_WQ_KERNEL_GEMM = 2,  /* LDS-tiled MFMA GEMM, any M */
+  MI355X_WQ_KERNEL_SKINNY = 3 /* HBM-bound path for M <= 64, activations in registers */
 };
 
 /* y[M,N] = f16( x[M,K] @ dequant(wq, scales)^T ), float32 accumulation.

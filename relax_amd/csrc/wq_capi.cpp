@@ -85,7 +85,9 @@ bool check_ptr(const void* p, const char* name, size_t align) {
   return true;
 }
 
-int select_kernel(const mi355x_wq_desc*, int64_t m) {
+int select_kernel(const mi355x_wq_desc* d, int64_t m) {
+  Problem p{nullptr, nullptr, nullptr, nullptr, m, d->n, d->k, d->bits, d->group, d->zero_point, nullptr};
+  if (gemv_applicable(p)) return MI355X_WQ_KERNEL_GEMV;
   return m <= kSkinnyMaxM ? MI355X_WQ_KERNEL_SKINNY : MI355X_WQ_KERNEL_GEMM;
 }
 
@@ -124,6 +126,7 @@ int mi355x_wq_matmul_ex(const mi355x_wq_desc* desc, const void* x, const void* w
             static_cast<hipStream_t>(stream)};
   int chosen = family == MI355X_WQ_KERNEL_AUTO ? select_kernel(desc, m) : family;
   switch (chosen) {
+    case MI355X_WQ_KERNEL_GEMV: return launch_gemv(p, variant);
     case MI355X_WQ_KERNEL_SKINNY: return launch_skinny(p, variant);
     case MI355X_WQ_KERNEL_GEMM: return launch_gemm(p, variant);
     default: set_error("unknown kernel family %d", family); return -1;

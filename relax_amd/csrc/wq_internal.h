@@ -17,6 +17,8 @@ struct Problem {
 
 // Tuning variant: 0 = library default for the shape, >0 = explicit choice
 // (only reachable through mi355x_wq_matmul_ex; used by sweeps).
+int launch_gemv(const Problem& p, int variant);
+bool gemv_applicable(const Problem& p);  // M <= 16 and the activations fit the LDS staging area
 int launch_skinny(const Problem& p, int variant);
 int launch_gemm(const Problem& p, int variant);
 int launch_dequant(const Problem& p, void* wd);

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
   constexpr int CH = 128 / BITS;  // k covered by one 16-byte lane load: 32 / 16
   constexpr int NJ = CH / 8;      // MFMAs fed by one lane load: 4 / 2
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform loop control
   const int col = lane & 15;
   const int kq = lane >> 4;
 
@@ -150,9 +150,13 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
   load_batch(b0, ks_begin);
   for (int ks = ks_begin; ks < ks_end; ks += 2 * U) {
     load_batch(b1, ks + U);
+    __builtin_amdgcn_sched_barrier(0);
     compute_batch(b0);
+    __builtin_amdgcn_sched_barrier(0);
     load_batch(b0, ks + 2 * U);
+    __builtin_amdgcn_sched_barrier(0);
     compute_batch(b1);
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // cross-wave reduction of the K split

@@ -8,7 +8,7 @@ import subprocess
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 SO_PATH = os.path.join(CSRC, "libmi355x_wq.so")
 
-KERNEL_AUTO, KERNEL_SKINNY, KERNEL_GEMM = 0, 1, 2
+KERNEL_AUTO, KERNEL_GEMV, KERNEL_GEMM, KERNEL_SKINNY = 0, 1, 2, 3
 
 # every symbol include/mi355x_wq.h and include/mi355x_wq_packed.h declare
 EXPORTED_SYMBOLS = (

@@ -79,7 +79,44 @@ def test_dequantize_every_field_value_and_special_scales(bits):
     assert np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
 
 
-# ------------------------------------------------------------------ skinny (GEMV-class) kernel
+# ------------------------------------------------------------------ GEMV kernel (activations staged in LDS)
+GEMV_SHAPES = [
+    (4, 1, 64, 256), (4, 1, 40, 352), (4, 3, 16, 32), (4, 8, 200, 1024), (4, 16, 48, 2048),
+    (4, 5, 33, 1152), (4, 2, 24, 11008),
+    (8, 1, 64, 256), (8, 2, 40, 384), (8, 16, 24, 128), (8, 7, 72, 640), (8, 4, 16, 1280),
+]
+
+
+@pytest.mark.parametrize("variant", list(range(1, 17)))
+def test_gemv_kernel_variants_match_oracle(variant):
+    """Every tuning variant on every shape it accepts (a variant that needs K to be a multiple of
+    its super step refuses other shapes with an error, which is checked to be exactly that)."""
+    from relax_amd import lib
+
+    ran = 0
+    for bits, m, n, k in GEMV_SHAPES:
+        x, wq, s, g = O.make_case(300 + m + n, m, n, k, bits)
+        try:
+            got = run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_GEMV, variant=variant)
+        except lib.WqError as e:
+            assert "does not apply" in str(e)
+            continue
+        ran += 1
+        want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=8)
+        assert_close(got, want, (variant, bits, m, n, k))
+    assert ran >= 4
+
+
+def test_gemv_refuses_what_does_not_fit_lds():
+    from relax_amd import lib
+
+    x, wq, s, g = O.make_case(1, 16, 16, 4096, 4)
+    with pytest.raises(lib.WqError, match="do not fit"):
+        run_matmul(x, wq, s, 4, g, kernel=lib.KERNEL_GEMV)
+    assert_close(run_matmul(x, wq, s, 4, g), c_oracle.wq_matmul(x, wq, s, 4, g), "auto falls back")
+
+
+# ------------------------------------------------------------------ skinny kernel (activations in registers)
 SKINNY_VARIANTS = [1, 2, 3, 4, 5, 6]
 
 
