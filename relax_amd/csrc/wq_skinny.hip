@@ -200,6 +200,10 @@ bool dispatch_variant(const Problem& p, int group_shift, int variant) {
     case 4: launch_one<BITS, 1, MT, 4, 4>(p, group_shift); return true;
     case 5: launch_one<BITS, 2, MT, 8, 1>(p, group_shift); return true;
     case 6: launch_one<BITS, 1, MT, 8, 1>(p, group_shift); return true;
+    case 7: launch_one<BITS, 4, MT, 4, 1>(p, group_shift); return true;
+    case 8: launch_one<BITS, 4, MT, 8, 1>(p, group_shift); return true;
+    case 9: launch_one<BITS, 4, MT, 2, 1>(p, group_shift); return true;
+    case 10: launch_one<BITS, 2, MT, 2, 2>(p, group_shift); return true;
     default: return false;
   }
 }
