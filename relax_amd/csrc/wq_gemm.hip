@@ -212,16 +212,38 @@ int launch_gemm(const Problem& p, int variant) {
     set_error("gemm kernel: group %d must be %d times a power of two", p.group, ch);
     return -1;
   }
+  if (variant == 0 && gemm_pipe_applicable(p)) {
+    // measured on MI355X: the 256x128 tile wins once M fills it a few times over;
+    // smaller M keeps more workgroups in flight with 128x128 tiles
+    variant = p.m >= 1024 ? 11 : 12;
+  }
+  if (variant >= 11) {
+    if (!launch_gemm_pipe(p, group_shift, variant - 10)) {
+      set_error("gemm kernel: pipelined variant %d does not apply to M=%lld N=%lld K=%lld", variant,
+                (long long)p.m, (long long)p.n, (long long)p.k);
+      return -1;
+    }
+    variant = -1;
+  }
   if (variant == 0) variant = 1;
+#define WQ_GEMM_CASE(ID, BM, BN, WM, WN)                                  \
+  case ID:                                                                \
+    if (p.bits == 4) launch_one<4, BM, BN, WM, WN>(p, group_shift);       \
+    else launch_one<8, BM, BN, WM, WN>(p, group_shift);                   \
+    break;
   switch (variant) {
-    case 1:
-      if (p.bits == 4) launch_one<4, 128, 128, 2, 2>(p, group_shift);
-      else launch_one<8, 128, 128, 2, 2>(p, group_shift);
-      break;
+    case -1: break;  // already launched above
+    WQ_GEMM_CASE(1, 128, 128, 2, 2)
+    WQ_GEMM_CASE(2, 256, 128, 2, 2)
+    WQ_GEMM_CASE(3, 128, 256, 2, 2)
+    WQ_GEMM_CASE(4, 256, 256, 2, 2)
+    WQ_GEMM_CASE(5, 256, 256, 2, 4)
+    WQ_GEMM_CASE(6, 256, 256, 4, 2)
     default:
       set_error("gemm kernel: unknown variant %d", variant);
       return -1;
   }
+#undef WQ_GEMM_CASE
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("gemm kernel launch failed: %s", hipGetErrorString(e));

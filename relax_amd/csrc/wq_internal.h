@@ -21,6 +21,8 @@ int launch_gemv(const Problem& p, int variant);
 bool gemv_applicable(const Problem& p);  // M <= 16 and the activations fit the LDS staging area
 int launch_skinny(const Problem& p, int variant);
 int launch_gemm(const Problem& p, int variant);
+bool gemm_pipe_applicable(const Problem& p);  // K % 64 == 0, operands below 1 GiB
+bool launch_gemm_pipe(const Problem& p, int group_shift, int variant);
 int launch_dequant(const Problem& p, void* wd);
 
 // Upper bound of rows the skinny family accepts.

@@ -190,6 +190,28 @@ def test_gemm_kernel_matches_oracle(bits, m, n, k):
     assert_close(got, want, (bits, m, n, k))
 
 
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 11, 12, 13])
+@pytest.mark.parametrize("bits,m,n,k", [(4, 300, 200, 128), (4, 70, 136, 448), (4, 513, 72, 320),
+                                         (8, 129, 72, 256), (8, 513, 260, 1024)])
+def test_gemm_tile_variants_match_oracle(variant, bits, m, n, k):
+    """Generic (1-6) and software-pipelined (11-13) tile shapes, ragged M and N, odd and even k-step counts."""
+    from relax_amd import lib
+
+    x, wq, s, g = O.make_case(400 + m + n, m, n, k, bits)
+    got = run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_GEMM, variant=variant)
+    want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
+    assert_close(got, want, (variant, bits, m, n, k))
+
+
+def test_gemm_pipelined_variant_refuses_k_not_multiple_of_64():
+    from relax_amd import lib
+
+    x, wq, s, g = O.make_case(1, 70, 32, 96, 4)
+    with pytest.raises(lib.WqError, match="does not apply"):
+        run_matmul(x, wq, s, 4, g, kernel=lib.KERNEL_GEMM, variant=11)
+    assert_close(run_matmul(x, wq, s, 4, g, kernel=lib.KERNEL_GEMM), c_oracle.wq_matmul(x, wq, s, 4, g), "generic")
+
+
 @pytest.mark.parametrize("bits,m,n,k", [(4, 512, 4096, 4096), (4, 2048, 4096, 11008), (8, 256, 5120, 5120)])
 def test_gemm_full_size_rows_against_oracle_and_all_tiles_against_torch(bits, m, n, k):
     """Full-size prefill shapes: a sample of rows against the oracle (seconds on the host), and every
