@@ -1,0 +1,233 @@
+"""Host-side tests of the C ABI and the PackedFunc boundary that need no GPU: the library
+loads, exports every declared symbol, and rejects bad arguments before touching the device."""
+import ctypes as C
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from relax_amd import lib, vm_harness  # noqa: E402
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = []
+    for h in ("mi355x_wq.h", "mi355x_wq_packed.h"):
+        text = open(os.path.join(ROOT, "include", h)).read()
+        names += re.findall(r"MI355X_WQ_API\s+[\w\s\*]+?\b(mi355x_\w+)\s*\(", text)
+    return names
+
+
+def test_library_exports_every_declared_symbol():
+    L = lib.load()
+    names = declared_symbols()
+    assert len(names) == 15 and set(names) == set(lib.EXPORTED_SYMBOLS)
+    for n in names:
+        assert hasattr(L, n), n
+    assert L.mi355x_wq_version() >= 100
+    # only the C ABI is exported: no C++ symbols leak out of the shared object
+    out = subprocess.run(["nm", "-D", "--defined-only", lib.SO_PATH], capture_output=True, text=True).stdout
+    exported = [l.split()[-1] for l in out.splitlines() if " T " in l]
+    assert sorted(exported) == sorted(names)
+
+
+@pytest.mark.parametrize("kw,msg", [
+    (dict(bits=5), "bits must be 4 or 8"),
+    (dict(group=48), "group must be 32 times a power of two"),
+    (dict(bits=8, group=24, zero_point=0), "group must be 16 times a power of two"),
+    (dict(zero_point=16), "zero_point must be in 0..15"),
+    (dict(bits=8, group=128, zero_point=3), "zero_point must be 0 for 8-bit"),
+    (dict(k=4096 + 32, group=64), "not a multiple of the group size"),
+    (dict(n=-1), "negative extent"),
+    (dict(n=1 << 30, k=1 << 14), "operand too large"),
+])
+def test_descriptor_validation(kw, msg):
+    L = lib.load()
+    args = dict(bits=4, group=32, n=4096, k=4096, zero_point=7)
+    args.update(kw)
+    d = lib.make_desc(args["bits"], args["group"], args["n"], args["k"], args["zero_point"])
+    assert L.mi355x_wq_check(d, 1) == -1
+    assert msg in lib.last_error()
+
+
+def test_reserved_field_and_null_descriptor():
+    L = lib.load()
+    d = lib.make_desc(4, 32, 64, 64)
+    d.reserved = 1
+    assert L.mi355x_wq_check(d, 1) == -1 and "reserved" in lib.last_error()
+    assert L.mi355x_wq_check(None, 1) == -1 and "NULL" in lib.last_error()
+
+
+def test_kernel_selection_by_rows():
+    L = lib.load()
+    d = lib.make_desc(4, 32, 4096, 4096)
+    assert L.mi355x_wq_select_kernel(d, 1) == lib.KERNEL_GEMV
+    assert L.mi355x_wq_select_kernel(d, 16) == lib.KERNEL_GEMV
+    assert L.mi355x_wq_select_kernel(d, 17) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(d, 64) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(d, 65) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(d, -1) == -1
+
+
+def test_pointer_checks_happen_before_any_launch():
+    L = lib.load()
+    d = lib.make_desc(4, 32, 64, 64)
+    ok = 0x10000
+    assert L.mi355x_wq_matmul(d, None, ok, ok, ok, 1, None) == -1 and "x is NULL" in lib.last_error()
+    assert L.mi355x_wq_matmul(d, ok, ok + 8, ok, ok, 1, None) == -1 and "wq" in lib.last_error() \
+        and "16-byte aligned" in lib.last_error()
+    assert L.mi355x_wq_matmul(d, ok, ok, ok + 1, ok, 1, None) == -1 and "scales" in lib.last_error()
+    assert L.mi355x_wq_dequantize(d, ok, ok, ok + 4, None) == -1 and "wd" in lib.last_error()
+    # empty problems succeed without touching the device
+    assert L.mi355x_wq_matmul(d, None, None, None, None, 0, None) == 0
+    d0 = lib.make_desc(4, 32, 0, 64)
+    assert L.mi355x_wq_matmul(d0, None, None, None, None, 3, None) == 0
+    assert L.mi355x_wq_dequantize(d0, None, None, None, None) == 0
+    assert L.mi355x_wq_matmul_ex(d, ok, ok, ok, ok, 100, None, lib.KERNEL_SKINNY) == -1 \
+        and "exceeds 64" in lib.last_error()
+    assert L.mi355x_wq_matmul_ex(d, ok, ok, ok, ok, 1, None, 77) == -1 and "unknown kernel family" in lib.last_error()
+
+
+# ---------------------------------------------------------------- PackedFunc boundary, error paths
+def _cpu_case(m=2, n=16, k=64, bits=4):
+    per = 32 // bits
+    g = 32 if bits == 4 else 16
+    x = torch.zeros((m, k), dtype=torch.float16)
+    wq = torch.zeros((n, k // per), dtype=torch.int32)
+    s = torch.zeros((n, k // g), dtype=torch.float16)
+    y = torch.zeros((m, n), dtype=torch.float16)
+    return x, wq, s, y
+
+
+def _args(x, wq, s, y, **kw):
+    return [vm_harness.TensorArg(x, **kw), vm_harness.TensorArg(wq, as_uint32=True, **kw),
+            vm_harness.TensorArg(s, **kw), vm_harness.TensorArg(y, **kw)]
+
+
+def test_packed_rejects_host_tensors():
+    with pytest.raises(vm_harness.PackedError, match="expected a ROCm tensor"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", _args(*_cpu_case()))
+
+
+def test_packed_argument_count_and_type_codes():
+    x, wq, s, y = _cpu_case()
+    a = _args(x, wq, s, y, device_type=10)
+    with pytest.raises(vm_harness.PackedError, match="expects 4 arguments, got 3"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", a[:3])
+    with pytest.raises(vm_harness.PackedError, match="expects 3 arguments, got 4"):
+        vm_harness.call_packed("mi355x_q4f16_dequantize", a)
+    with pytest.raises(vm_harness.PackedError, match="expected a tensor"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", [a[0], 5, a[2], a[3]])
+    with pytest.raises(vm_harness.PackedError, match="expected a tensor"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", [a[0], None, a[2], a[3]])
+
+
+def test_packed_dtype_shape_and_stride_checks():
+    x, wq, s, y = _cpu_case()
+    dev = dict(device_type=10)
+    with pytest.raises(vm_harness.PackedError, match=r"argument 1 \(wq\): expected dtype uint32"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", [
+            vm_harness.TensorArg(x, **dev), vm_harness.TensorArg(wq, **dev),  # int32, not uint32
+            vm_harness.TensorArg(s, **dev), vm_harness.TensorArg(y, **dev)])
+    with pytest.raises(vm_harness.PackedError, match=r"argument 0 \(x\): expected dtype float16"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", _args(x.float(), wq, s, y, **dev))
+    with pytest.raises(vm_harness.PackedError, match="x has 32 columns but the weights have K=64"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", _args(x[:, :32].contiguous(), wq, s, y, **dev))
+    with pytest.raises(vm_harness.PackedError, match=r"y has shape \(2, 8\), expected \(2, 16\)"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", _args(x, wq, s, y[:, :8].contiguous(), **dev))
+    with pytest.raises(vm_harness.PackedError, match="scales has 8 rows but wq has 16"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", _args(x, wq, s[:8].contiguous(), y, **dev))
+    with pytest.raises(vm_harness.PackedError, match="expected a 2-d tensor"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", _args(x.reshape(-1), wq, s, y, **dev)[:1] +
+                               _args(x, wq, s, y, **dev)[1:])
+    xt = torch.zeros((64, 2), dtype=torch.float16).t()  # shape (2, 64), strides (1, 2)
+    with pytest.raises(vm_harness.PackedError, match="not compact row-major"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", [
+            vm_harness.TensorArg(xt, with_strides=True, **dev)] + _args(x, wq, s, y, **dev)[1:])
+    # K / scales columns must give a legal group: 64 / 3 is not an integer
+    with pytest.raises(vm_harness.PackedError, match="cannot infer the group size"):
+        vm_harness.call_packed("mi355x_q4f16_matmul",
+                               _args(x, wq, torch.zeros((16, 3), dtype=torch.float16), y, **dev))
+    # q8 entry on q4-shaped data: K = 8 words * 4 = 32, x has 64 columns
+    with pytest.raises(vm_harness.PackedError, match="x has 64 columns but the weights have K=32"):
+        vm_harness.call_packed("mi355x_q8f16_matmul", _args(x, wq, s, y, **dev))
+
+
+def test_packed_empty_output_is_a_no_op():
+    x, wq, s, y = _cpu_case(m=0)
+    vm_harness.call_packed("mi355x_q4f16_matmul", _args(x, wq, s, y, device_type=10))
+
+
+def test_generic_entry_checks_the_call_spec():
+    x, wq, s, y = _cpu_case()
+    a = _args(x, wq, s, y, device_type=10)
+    bad = vm_harness.CallSpec(0, 4, 0, 7, 0, 1, 1, 3, 4)  # two roles on argument 1
+    with pytest.raises(vm_harness.PackedError, match="not a permutation"):
+        vm_harness.call_packed(None, a, spec=bad)
+    with pytest.raises(vm_harness.PackedError, match="unknown op"):
+        vm_harness.call_packed(None, a, spec=vm_harness.CallSpec(7, 4, 0, 7, 0, 1, 2, 3, 4))
+    # explicit group that contradicts the scales shape
+    with pytest.raises(vm_harness.PackedError, match="does not match K=64 / group=64"):
+        vm_harness.call_packed(None, a, spec=vm_harness.CallSpec(0, 4, 64, 7, 0, 1, 2, 3, 4))
+    # roles permuted the way FuseOpsByPattern orders them: (wq, scales, x, y)
+    permuted = [a[1], a[2], a[0], a[3]]
+    spec = vm_harness.CallSpec(0, 4, 0, 7, 2, 0, 1, 3, 4)
+    if not torch.cuda.is_available():  # all checks pass; only the missing device stops the call
+        with pytest.raises(vm_harness.PackedError, match="no usable HIP device"):
+            vm_harness.call_packed(None, permuted, spec=spec)
+
+
+def test_stream_setter_round_trip():
+    L = lib.load()
+    L.mi355x_wq_packed_set_stream(0x1230)
+    assert L.mi355x_wq_packed_get_stream() == 0x1230
+    L.mi355x_wq_packed_set_stream(None)
+    assert not L.mi355x_wq_packed_get_stream()
+
+
+# ---------------------------------------------------------------- registration in a TVM-like registry
+REGISTRY_SCRIPT = r"""
+import ctypes as C, os, sys
+sys.path.insert(0, {root!r})
+from relax_amd import lib, vm_harness
+import torch
+L = lib.load()
+assert L.mi355x_wq_register_tvm_globals(0) == -1 and "no TVM runtime" in lib.last_error()
+fake = C.CDLL({fake!r}, mode=C.RTLD_GLOBAL)
+fake.fake_tvm_name.restype = C.c_char_p
+fake.fake_tvm_last_error.restype = C.c_char_p
+assert L.mi355x_wq_register_tvm_globals(0) == 4
+names = sorted(fake.fake_tvm_name(i).decode() for i in range(fake.fake_tvm_count()))
+assert names == ["mi355x.q4f16_dequantize", "mi355x.q4f16_matmul", "mi355x.q8f16_dequantize",
+                 "mi355x.q8f16_matmul"], names
+# call a registered function the way the registry would, with host tensors: it must fail and the
+# message must arrive in the host's last-error slot (what LOG(FATAL) << TVMGetLastError() prints)
+idx = [fake.fake_tvm_name(i).decode() for i in range(4)].index("mi355x.q4f16_matmul")
+x = torch.zeros((1, 64), dtype=torch.float16); wq = torch.zeros((16, 8), dtype=torch.int32)
+s = torch.zeros((16, 2), dtype=torch.float16); y = torch.zeros((1, 16), dtype=torch.float16)
+ta = [vm_harness.TensorArg(x), vm_harness.TensorArg(wq, as_uint32=True), vm_harness.TensorArg(s),
+      vm_harness.TensorArg(y)]
+vals = (vm_harness.TVMValue * 4)(); codes = (C.c_int * 4)()
+for i, t in enumerate(ta):
+    vals[i].v_handle = t.handle; codes[i] = 13
+fake.fake_tvm_call.argtypes = [C.c_int, C.c_void_p, C.POINTER(C.c_int), C.c_int]
+assert fake.fake_tvm_call(idx, C.addressof(vals), codes, 4) == -1
+assert b"expected a ROCm tensor" in fake.fake_tvm_last_error()
+print("registry ok")
+"""
+
+
+def test_registration_through_the_tvm_c_api(tmp_path):
+    fake = str(tmp_path / "libfake_tvm.so")
+    subprocess.check_call(["gcc", "-shared", "-fPIC", "-o", fake,
+                           os.path.join(ROOT, "tests", "support", "fake_tvm_registry.c")])
+    # own process: the fake registry must not stay loaded for the other tests
+    out = subprocess.run([sys.executable, "-c", REGISTRY_SCRIPT.format(root=ROOT, fake=fake)],
+                         capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "registry ok" in out.stdout, out.stdout + out.stderr

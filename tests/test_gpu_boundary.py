@@ -1,0 +1,124 @@
+"""GPU tests of the PackedFunc boundary: the VM-style call path (DLPack tensors, DPS output,
+generated entries with permuted roles) and the decoder-layer chain of configuration 5."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+from oracle import c_oracle, wq_oracle as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+from tests.test_gpu_parity import ATOL, RTOL, _dev, assert_close  # noqa: E402
+
+
+def test_fixed_name_entries_called_vm_style():
+    from relax_amd import vm_harness
+
+    vm_harness.set_stream()
+    for bits, m, n, k in [(4, 1, 4096, 4096), (4, 8, 64, 352), (4, 200, 136, 256), (8, 16, 5120, 5120)]:
+        x, wq, s, g = O.make_case(21, m, n, k, bits)
+        y = vm_harness.call_dps("mi355x_q%df16_matmul" % bits, [_dev(x), _dev(wq), _dev(s)], (m, n))
+        wd = vm_harness.call_dps("mi355x_q%df16_dequantize" % bits, [_dev(wq), _dev(s)], (n, k))
+        torch.cuda.synchronize()
+        assert_close(y.cpu().numpy(), c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16), (bits, m, n, k))
+        assert np.array_equal(wd.cpu().numpy().view(np.uint16), c_oracle.dequant(wq, s, bits, g, 8).view(np.uint16))
+
+
+def test_dltensor_handle_type_code_strides_and_byte_offset():
+    """Type code 7 as well as 13; explicit compact strides; a view whose data pointer is the base of
+    the allocation and whose start is carried in byte_offset (the cutlass glue ignores that field,
+    python/tvm/contrib/cutlass/gemm_operation.py:280-283; this boundary honours it)."""
+    from relax_amd import vm_harness
+
+    vm_harness.set_stream()
+    x, wq, s, g = O.make_case(22, 4, 48, 128, 4)
+    big = torch.zeros((8, 128), dtype=torch.float16, device="cuda")
+    big[4:] = _dev(x)
+    y = torch.empty((4, 48), dtype=torch.float16, device="cuda")
+    args = [vm_harness.TensorArg(big[4:], with_strides=True, byte_offset=4 * 128 * 2),
+            vm_harness.TensorArg(_dev(wq), as_uint32=True), vm_harness.TensorArg(_dev(s)),
+            vm_harness.TensorArg(y)]
+    vm_harness.call_packed("mi355x_q4f16_matmul", args, type_code=vm_harness.K_TVM_DLTENSOR_HANDLE)
+    torch.cuda.synchronize()
+    assert_close(y.cpu().numpy(), c_oracle.wq_matmul(x, wq, s, 4, g), "byte_offset view")
+    # a misaligned view is refused, not silently mis-read
+    odd = vm_harness.TensorArg(big.view(-1)[4:4 + 4 * 128].view(4, 128))
+    with pytest.raises(vm_harness.PackedError, match="16-byte aligned"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", [odd] + args[1:])
+    # tensors on another device id than the current one
+    other = vm_harness.TensorArg(_dev(x))
+    other.dl.device.device_id = 3
+    with pytest.raises(vm_harness.PackedError, match="on device 3 but the first tensor is on device 0"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", [other] + args[1:])
+
+
+def test_generated_entry_with_permuted_roles(tmp_path):
+    from relax_amd import vm_harness
+    from relax_amd.tvm_glue import CallSpec
+    from tests.test_tvm_glue_cpu import SYM, build_entries, call_entry
+
+    L = build_entries(tmp_path, [(SYM, CallSpec(0, 4, 0, 7, 2, 0, 1, 3))])
+    vm_harness.set_stream()
+    x, wq, s, g = O.make_case(23, 8, 4096, 4096, 4)
+    y = torch.empty((8, 4096), dtype=torch.float16, device="cuda")
+    t = [vm_harness.TensorArg(_dev(wq), as_uint32=True), vm_harness.TensorArg(_dev(s)),
+         vm_harness.TensorArg(_dev(x)), vm_harness.TensorArg(y)]
+    rc, code = call_entry(L, SYM, t)
+    torch.cuda.synchronize()
+    assert rc == 0 and code == vm_harness.K_TVM_NULLPTR
+    assert_close(y.cpu().numpy(), c_oracle.wq_matmul(x, wq, s, 4, g, nthreads=16), "generated entry")
+
+
+@pytest.mark.parametrize("m", [4, 1024])
+def test_config5_decoder_layer_chain(m):
+    """One Llama-2-7B-shaped decoder layer's four quantized matmuls back to back, as the VM would call
+    them (DPS externs), the float16 residual flowing through.  Attention and the MLP activation are
+    replaced by fixed elementwise stand-ins that are identical on both sides:
+        qkv = x Wqkv^T;  a = (qkv[:, :4096] / 2 + qkv[:, 4096:8192] / 4 + qkv[:, 8192:] / 4) / 32
+        h   = x + (a Wo^T) / 32
+        gu  = h Wgu^T;   z = (gu[:, :11008] / 32) * (gu[:, 11008:] / 32)      (float16 products)
+        out = h + (z Wd^T) / 32
+    (powers of two keep the stand-ins exact and the activations of random-weight layers bounded.)
+    The CPU side runs the oracle on a sample of rows (each row is independent)."""
+    from relax_amd import vm_harness
+
+    vm_harness.set_stream()
+    shapes = {"qkv": (12288, 4096), "o": (4096, 4096), "gu": (22016, 4096), "down": (4096, 11008)}
+    rng = np.random.default_rng(55)
+    x = (rng.standard_normal((m, 4096)) * 0.5).astype(np.float16)
+    W = {}
+    for i, (name, (n, k)) in enumerate(shapes.items()):
+        _, wq, s, g = O.make_case(60 + i, 1, n, k, 4)
+        W[name] = (wq, s)
+
+    def layer(xh, matmul, f16):
+        qkv = matmul(xh, "qkv")
+        a = f16(f16(f16(qkv[:, :4096] * f16(0.5)) + f16(qkv[:, 4096:8192] * f16(0.25))) + f16(qkv[:, 8192:] * f16(0.25)))
+        a = f16(a * f16(1 / 32))
+        h = f16(xh + f16(matmul(a, "o") * f16(1 / 32)))
+        gu = matmul(h, "gu")
+        z = f16(f16(gu[:, :11008] * f16(1 / 32)) * f16(gu[:, 11008:] * f16(1 / 32)))
+        return f16(h + f16(matmul(z, "down") * f16(1 / 32)))
+
+    dW = {k: (_dev(v[0]), _dev(v[1])) for k, v in W.items()}
+
+    def gpu_matmul(t, name):
+        return vm_harness.call_dps("mi355x_q4f16_matmul", [t.contiguous(), dW[name][0], dW[name][1]],
+                                   (t.shape[0], shapes[name][0]))
+
+    out = layer(_dev(x), gpu_matmul, lambda v: v if torch.is_tensor(v) else torch.tensor(v, dtype=torch.float16, device="cuda"))
+    torch.cuda.synchronize()
+    rows = np.arange(m) if m <= 4 else np.random.default_rng(5).choice(m, size=4, replace=False)
+
+    def cpu_matmul(t, name):
+        return c_oracle.wq_matmul(np.ascontiguousarray(t), W[name][0], W[name][1], 4, 32, nthreads=16)
+
+    want = layer(x[rows], cpu_matmul, lambda v: np.asarray(v, dtype=np.float16))
+    got = out.cpu().numpy()[rows]
+    # four chained matmuls: each adds at most the single-matmul tolerance on top of the propagated error
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    assert np.all(np.isfinite(got)) and np.all(err <= 4 * (ATOL + RTOL * np.abs(want.astype(np.float64)))), float(err.max())
+    assert float(np.mean(err)) < 2e-3

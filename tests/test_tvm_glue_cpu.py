@@ -1,0 +1,105 @@
+"""The text side of the Relax glue: generated entries compile against the restated C ABI,
+export the requested symbols and forward to the library with the recorded argument roles."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from relax_amd import lib, vm_harness  # noqa: E402
+from relax_amd.tvm_glue import CallSpec, trampoline_source  # noqa: E402
+from relax_amd.tvm_glue.patterns import BACKEND, DECODE_FUNCS  # noqa: E402
+
+SYM = "fused_decode_q4f16_relax_permute_dims_relax_matmul_relax_astype_mi355x"
+
+
+def build_entries(tmp_path, entries):
+    src = tmp_path / "entries.c"
+    src.write_text(trampoline_source(entries))
+    so = str(tmp_path / "libentries.so")
+    libdir = os.path.dirname(lib.SO_PATH)
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-DMI355X_WQ_STANDALONE", "-shared", "-fPIC",
+                           "-o", so, str(src), "-L" + libdir, "-lmi355x_wq", "-Wl,-rpath," + libdir])
+    lib.load()
+    return C.CDLL(so)
+
+
+def call_entry(entry_lib, symbol, tensors):
+    n = len(tensors)
+    vals = (vm_harness.TVMValue * n)()
+    codes = (C.c_int * n)()
+    for i, t in enumerate(tensors):
+        vals[i].v_handle = t.handle
+        codes[i] = vm_harness.K_TVM_NDARRAY_HANDLE
+    ret = vm_harness.TVMValue()
+    rc_code = C.c_int(vm_harness.K_TVM_NULLPTR)
+    fn = getattr(entry_lib, symbol)
+    fn.argtypes = [C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_void_p, C.POINTER(C.c_int), C.c_void_p]
+    rc = fn(C.addressof(vals), codes, n, C.addressof(ret), C.byref(rc_code), None)
+    return rc, rc_code.value
+
+
+def test_generated_entries_compile_and_forward(tmp_path):
+    # FuseOpsByPattern hands the extern (wq, scales, x, y): roles x=2, wq=0, scales=1, out=3
+    entries = [(SYM, CallSpec(0, 4, 0, 7, 2, 0, 1, 3)),
+               ("fused_q8_mi355x", CallSpec(0, 8, 128, 0, 2, 0, 1, 3)),
+               ("decode_only_mi355x", CallSpec(1, 4, 0, 7, 0, 0, 1, 2))]
+    L = build_entries(tmp_path, entries)
+    x = torch.zeros((2, 64), dtype=torch.float16)
+    wq = torch.zeros((16, 8), dtype=torch.int32)
+    s = torch.zeros((16, 2), dtype=torch.float16)
+    y = torch.zeros((2, 16), dtype=torch.float16)
+    dev = dict(device_type=10)
+    t = [vm_harness.TensorArg(wq, as_uint32=True, **dev), vm_harness.TensorArg(s, **dev),
+         vm_harness.TensorArg(x, **dev), vm_harness.TensorArg(y, **dev)]
+    # the roles are honoured: with the arguments in (x, wq, scales, y) order the entry sees a float16 "wq"
+    wrong = [t[2], t[0], t[1], t[3]]
+    rc, code = call_entry(L, SYM, wrong)
+    assert rc == -1 and code == vm_harness.K_TVM_NULLPTR
+    assert "argument 0 (wq): expected dtype uint32" in lib.last_error()
+    if not torch.cuda.is_available():
+        rc, _ = call_entry(L, SYM, t)  # every check passes; there is just no device here
+        assert rc == -1 and "no usable HIP device" in lib.last_error()
+    # explicit group 128 contradicts the 2 scale columns of K = 32 (q8 reading of the same words)
+    rc, _ = call_entry(L, "fused_q8_mi355x", t)
+    assert rc == -1 and "does not match K=32 / group=128" in lib.last_error()
+    rc, _ = call_entry(L, "decode_only_mi355x", t)
+    assert rc == -1 and "expects 3 arguments, got 4" in lib.last_error()
+
+
+def test_trampoline_generator_rejects_bad_input():
+    with pytest.raises(ValueError, match="not a C identifier"):
+        trampoline_source([("bad-name", CallSpec(0, 4, 0, 7, 0, 1, 2, 3))])
+    with pytest.raises(ValueError, match="not a permutation"):
+        trampoline_source([("f", CallSpec(0, 4, 0, 7, 0, 0, 2, 3))])
+    with pytest.raises(ValueError, match="duplicate"):
+        trampoline_source([("f", CallSpec(0, 4, 0, 7, 0, 1, 2, 3)), ("f", CallSpec(0, 4, 0, 7, 0, 1, 2, 3))])
+    with pytest.raises(ValueError, match="bits"):
+        trampoline_source([("f", CallSpec(0, 3, 0, 7, 0, 1, 2, 3))])
+
+
+def test_pattern_table_metadata():
+    assert BACKEND == "mi355x"
+    assert DECODE_FUNCS["decode_q4f16"] == {"bits": 4, "zero_point": 7}
+    assert DECODE_FUNCS["decode_q8f16"] == {"bits": 8, "zero_point": 0}
+
+
+def test_quantize_helpers_round_trip():
+    from oracle import wq_oracle as O
+    from relax_amd import pack_q4, pack_q8, quantize_q4f16, quantize_q8f16
+
+    rng = np.random.default_rng(0)
+    w4 = rng.integers(0, 16, size=(5, 64))
+    w8 = rng.integers(-128, 128, size=(5, 64))
+    assert np.array_equal(pack_q4(w4), O.pack_q4(w4)) and np.array_equal(O.unpack_q4(pack_q4(w4)), w4)
+    assert np.array_equal(pack_q8(w8), O.pack_q8(w8)) and np.array_equal(O.unpack_q8(pack_q8(w8)), w8)
+    w = rng.standard_normal((8, 256)).astype(np.float32)
+    wq, s = quantize_q4f16(w)
+    assert np.abs(O.dequant_q4f16(wq, s).astype(np.float32) - w).max() <= 0.51 * float(s.max()) + 1e-3
+    wq, s = quantize_q8f16(w)
+    assert np.abs(O.dequant_q8f16(wq, s).astype(np.float32) - w).max() <= 0.51 * float(s.max()) + 1e-3
+    with pytest.raises(ValueError):
+        pack_q4(np.full((1, 8), 16))
