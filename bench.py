@@ -30,6 +30,10 @@ DECODE_BATCHES = (1, 8)
 PREFILL_M = 2048
 HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
+# HBM bytes per GEMV launch of this workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (mean per dispatch, scaled by a 256 MiB copy: FETCH_SIZE reads half the true KiB, WRITE_SIZE
+# the true KiB); measurement and commands in profiles/gemv_decode_llama7b.md.
+GEMV_HBM_TRAFFIC_PER_LAUNCH = int((14153.8 * 2.0 + 93.4 * 1.0) * 1024)
 
 
 def algorithmic_bytes(bits: int, group: int, m: int, n: int, k: int) -> int:
@@ -81,6 +85,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=N_LAYERS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy three times (a kernel of known HBM "
+                         "traffic, used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the hot path is a single-GPU kernel and this build has no "
@@ -96,6 +103,14 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     torch.manual_seed(0)
+
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.int32, device=dev)  # 256 MiB read + 256 MiB written
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- synthetic weights: every bit pattern is a valid packed int4 row ------------------
     layers = []
@@ -146,7 +161,7 @@ def main() -> int:
         "metric": "q4f16 GEMV GB/s + GEMM TFLOP/s (% roofline), Llama-7B shapes, 1 GPU",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "int4 weights x f16, f32 accumulate",
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "Llama-2-7B decode projections q4f16 g32, %d layers x "
                                "{12288x4096, 4096x4096, 22016x4096, 4096x11008}, batch 1 and batch 8, "
@@ -158,10 +173,7 @@ def main() -> int:
                      "bytes_per_launch": bytes_per_step // launches_per_step,
                      "avg_launch_us": round(avg_launch_us, 3)},
     }
-    traffic_file = os.path.join(ROOT, "profiles", "gemv_traffic.json")
-    if os.path.exists(traffic_file):
-        with open(traffic_file) as f:
-            result["roofline"]["traffic"] = json.load(f).get("hbm_bytes_per_launch")
+    result["roofline"]["traffic"] = GEMV_HBM_TRAFFIC_PER_LAUNCH
 
     # ---- prefill GEMM leg: M = 2048, the four shapes, layer-rotated weights -----------------
     if not args.no_gemm:
