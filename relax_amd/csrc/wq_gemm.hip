@@ -217,7 +217,14 @@ int launch_gemm(const Problem& p, int variant) {
     // smaller M keeps more workgroups in flight with 128x128 tiles
     variant = p.m >= 1024 ? 11 : 12;
   }
-  if (variant >= 11) {
+  if (variant >= 21) {
+    if (!launch_gemm_direct(p, group_shift, variant - 20)) {
+      set_error("gemm kernel: direct-weight variant %d does not apply to M=%lld N=%lld K=%lld group=%d",
+                variant, (long long)p.m, (long long)p.n, (long long)p.k, p.group);
+      return -1;
+    }
+    variant = -1;
+  } else if (variant >= 11) {
     if (!launch_gemm_pipe(p, group_shift, variant - 10)) {
       set_error("gemm kernel: pipelined variant %d does not apply to M=%lld N=%lld K=%lld", variant,
                 (long long)p.m, (long long)p.n, (long long)p.k);

@@ -1,0 +1,354 @@
+// MFMA GEMM for prefill (M > 64) whose weight operand never touches LDS:
+// y[M,N] = x[M,K] @ dequant(Wq,S)^T.
+//
+// Bound: dense float16 MFMA; the design goal is to keep LDS traffic (128 B/clk/CU on
+// gfx950) well below the matrix pipe's appetite.  A workgroup owns a BM x (64*WAVES)
+// output tile; all wavefronts share the same BM activation rows (staged in LDS) and
+// each owns 64 distinct weight rows, i.e. a BM x 64 sub-tile of 32x32x16 MFMAs.  The
+// MFMA B operand of lane (col = lane % 32, kh = lane / 32) for 16-wide k slice kk is
+// the 8 weights k = k0 + (kh*4 + kk)*8 .. +8 of row `col` -- exactly one packed int4
+// word, or two int8 words -- so a lane loads the 16 bytes (int4) it needs for a whole
+// 64-wide K step straight from global memory with one buffer load, together with the
+// one group scale that covers them, and dequantizes word by word in registers, to
+// exactly the float16 values the CPU path materialises.  No wavefront dequantizes a
+// weight twice, and LDS carries only the activations: BM*128 B written and
+// WAVES*BM*128 B read per K step.
+//
+// The A operand follows the same k assignment: lane (row, kh) reads chunk kh*4 + kk
+// of its activation row.  LDS rows are 128 bytes, their eight 16-byte chunks
+// XOR-swizzled with (row & 7), conflict-free for the reads (8 rows x same chunk, and
+// chunk c with chunk c+4 of the other half-wave) and for the row-contiguous writes.
+//
+// Pipeline per K step t (four activation stages in LDS, rings of four register sets for
+// activations and packed weights: workgroups sharing a tile run in lockstep, so every
+// global load sees close to the full memory latency and is issued 2.5 - 3 steps ahead);
+// program order is issue order, a handful of independent instructions after every MFMA,
+// fenced with sched_barrier:
+//   global -> registers : activations of step t+4, packed weights + scales of step t+3
+//   registers -> LDS    : activations of step t+2
+//   LDS -> registers    : A fragments of the next k slice (of step t+1 at the end)
+//   dequantize          : one stage each of four pair conversions per MFMA slot
+//
+// Shape requirements (checked by the launcher): K a multiple of 256, group 32 (int4) or
+// 128 (int8), operands < 1 GiB; other shapes use the other GEMM kernels.
+#include <type_traits>
+
+#include "wq_device.h"
+#include "wq_internal.h"
+
+namespace wq {
+
+namespace {
+constexpr uint32_t kRowOobD = 0x80000000u;   // offset of a row that must read zeros
+constexpr uint32_t kStepOobD = 0x40000000u;  // added for a K step past K: beyond any buffer < 1 GiB
+
+template <int B, int E, class F>
+__device__ __forceinline__ void static_for_d(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for_d<B + 1, E>(f);
+  }
+}
+}  // namespace
+
+template <int BITS>
+struct RawB {
+  static constexpr int NV = BITS == 4 ? 1 : 2;  // 16-byte loads per 32 k of one row
+  u32x4 w[2][NV];                               // [column tile][load]
+};
+
+template <int BITS, int TM, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
+    const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
+    half_t* __restrict__ y, int M, int N, int K, int group_shift, int zero_point, int tiles_m,
+    int tiles_n) {
+  constexpr int BK = 64;
+  static_assert(TM == 4, "the pair-conversion pipeline is laid out for four MFMA slots per B fragment");
+  constexpr int BM = TM * 32, BN = WAVES * 64;
+  constexpr int NT = WAVES * 64;
+  constexpr int CH = 128 / BITS;   // k per 16-byte packed chunk
+  constexpr int NV = RawB<BITS>::NV;
+  constexpr int XL = BM * 8 / NT;  // 16-byte activation chunks per thread per step
+  constexpr int STAGE = BM * 128;  // bytes per LDS stage
+  static_assert(XL >= 1 && BM * 8 % NT == 0 && (NT / 8) % 8 == 0, "activation tile / thread split");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char wq_gemm_direct_smem[];
+  unsigned char* const lds = wq_gemm_direct_smem;
+
+  // XCD-aware tile order: consecutive workgroup ids land on different XCDs; regroup them so
+  // that each XCD owns a contiguous range of activation row blocks (which then stay in its
+  // L2) and streams the much smaller packed weights once.
+  const int nblocks = tiles_m * tiles_n;
+  int bid = blockIdx.x;
+  if ((nblocks & 7) == 0) bid = (bid & 7) * (nblocks >> 3) + (bid >> 3);
+  const int tile_m = bid / tiles_n, tile_n = bid % tiles_n;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int fr = lane & 31, fh = lane >> 5;
+
+  const uint32_t row_bytes = (uint32_t)K * BITS / 8;
+  const uint32_t groups_per_row = ((uint32_t)K / CH) >> group_shift;
+  const rsrc_t rw = make_rsrc(wq, (uint32_t)N * row_bytes);
+  const rsrc_t rs = make_rsrc(scales, (uint32_t)N * groups_per_row * 2u);
+  const rsrc_t rx = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
+
+  // ---- activations: global offsets and LDS store address of this thread ---------------
+  uint32_t xg[XL];
+  const int x_row0 = tid >> 3, x_c = tid & 7;
+#pragma unroll
+  for (int i = 0; i < XL; ++i) {
+    const int m = m0 + x_row0 + i * (NT / 8);
+    xg[i] = m < M ? (uint32_t)m * (uint32_t)K * 2u + (uint32_t)x_c * 16u : kRowOobD;
+  }
+  const uint32_t x_lds = (uint32_t)x_row0 * 128u + (uint32_t)((x_c ^ (x_row0 & 7)) << 4);
+
+  // ---- weights: this lane's two rows (column tiles j = 0, 1) --------------------------
+  uint32_t wg[2], sg[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int n = min(n0 + wave * 64 + j * 32 + fr, N - 1);  // rows past N: computed, not stored
+    wg[j] = (uint32_t)n * row_bytes + (uint32_t)fh * (32u * BITS / 8);
+    sg[j] = (uint32_t)n * groups_per_row * 2u;
+  }
+
+  // ---- A fragment read addresses: row fr, chunk fh*4 + kk ------------------------------
+  uint32_t a_rd[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk)
+    a_rd[kk] = (uint32_t)fr * 128u + (uint32_t)(((fh * 4 + kk) ^ (fr & 7)) << 4);
+
+  const Q4Consts qc = make_q4_consts(zero_point);
+  const int ksteps = K / BK;
+
+  auto load_x = [&](u32x4 (&xr)[XL], int kt, auto ic) {
+    constexpr int i = decltype(ic)::value;
+    const uint32_t xk = kt < ksteps ? (uint32_t)kt * BK * 2u : kStepOobD;
+    xr[i] = load_b128(rx, xg[i] + xk);
+  };
+  auto store_x = [&](const u32x4 (&xr)[XL], uint32_t stage_base, auto ic) {
+    constexpr int i = decltype(ic)::value;
+    *reinterpret_cast<u32x4*>(lds + stage_base + x_lds + (uint32_t)i * (NT / 8) * 128u) = xr[i];
+  };
+  // piece c of the packed-weight loads of step kt
+  auto load_b = [&](RawB<BITS>& b, int kt, auto cc) {
+    constexpr int c = decltype(cc)::value, j = c / NV, v = c % NV;
+    const uint32_t k0 = (uint32_t)kt * BK;
+    b.w[j][v] = load_b128(rw, wg[j] + (kt < ksteps ? k0 * BITS / 8 : kStepOobD) + v * 16u);
+  };
+  constexpr int PBL = 2 * NV;  // packed-weight load pieces per step
+
+  // Group scales are fetched once per four K steps (256 k of a row): eight float16 for
+  // int4 / group 32, two for int8 / group 128.  2-byte loads per step would touch 32 cache
+  // lines per instruction for 128 useful bytes and dominate the L1 pipeline.
+  constexpr int SW = BITS == 4 ? 4 : 1;  // 32-bit words of scales per row and macro step
+  uint32_t sc_cur[2][SW], sc_nxt[2][SW];
+  auto load_scales = [&](uint32_t (&sc)[2][SW], int kt0) {
+    // kt0: first step of the macro step (a multiple of 4)
+    const bool ok = kt0 < ksteps;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint32_t off = ok ? sg[j] + (uint32_t)kt0 * (BK / (BITS == 4 ? 32 : 128)) * 2u : kStepOobD;
+      if constexpr (BITS == 4) {
+        const u32x4 v = load_b128(rs, off);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sc[j][q] = v[q];
+      } else {
+        sc[j][0] = load_b32(rs, off);
+      }
+    }
+  };
+  // scale of (column tile j, step t of the macro step) in the low half of a register
+  auto pick_scale = [&](const uint32_t (&sc)[2][SW], int j, int t) -> uint32_t {
+    if constexpr (BITS == 4) return __builtin_amdgcn_alignbit(sc[j][t], sc[j][t], (uint32_t)fh * 16u);
+    else return t < 2 ? sc[j][0] : sc[j][0] >> 16;
+  };
+  uint32_t s_step[2][2];  // [step parity][column tile]
+
+  // The conversion of one pair of weights is a chain of four dependent VALU ops (byte
+  // permute, and-or, fma, scale multiply).  The chain is software-pipelined over four
+  // MFMA slots -- every slot advances four different pairs by one stage -- so no slot
+  // contains dependent instructions.  Pair g (counted from the start of the K step)
+  // belongs to B fragment g/4 = slice (g/8), column tile (g/4)%2, position g%4.
+  auto stage_perm = [&](const RawB<BITS>& b, auto gc) -> uint32_t {
+    constexpr int g = decltype(gc)::value, kk = (g / 8) & 3, j = (g / 4) & 1, pp = g & 3;
+    if constexpr (BITS == 4) {
+      return __builtin_amdgcn_perm(0u, b.w[j][0][kk], 0x0c000c00u | (uint32_t)pp | ((uint32_t)pp << 16));
+    } else {
+      return __builtin_amdgcn_perm(0u, b.w[j][kk >> 1][(kk & 1) * 2 + (pp >> 1)],
+                                   (pp & 1) ? 0x0c030c02u : 0x0c010c00u);
+    }
+  };
+  auto stage_bits = [&](uint32_t v) -> uint32_t {
+    if constexpr (BITS == 4) return and_or(v, 0x00F0000Fu, qc.magic);
+    else return v ^ 0x64806480u;
+  };
+  auto stage_center = [&](uint32_t v) -> half2_t {
+    if constexpr (BITS == 4) return __builtin_elementwise_fma(as_h2(v), qc.mix_mul, -qc.mix_sub);
+    else return as_h2(v) - half2_t{(half_t)1152.0f, (half_t)1152.0f};
+  };
+  auto stage_scale = [&](int parity, half2_t v, auto gc) -> uint32_t {
+    constexpr int g = decltype(gc)::value, j = (g / 4) & 1;
+    return as_u32(v * bcast_h2(__builtin_bit_cast(half_t, (uint16_t)s_step[parity][j])));
+  };
+
+  half8_t fa[2][TM];
+  u32x4 fbq[4];  // ring of B fragments (fragment q of a step lives in fbq[q % 4])
+  uint32_t t_perm, t_bits;  // pipeline registers of the pair conversion
+  half2_t t_center;
+  auto read_a = [&](int buf, uint32_t base, auto ic) {
+    constexpr int i = decltype(ic)::value;
+    fa[buf][i] = *reinterpret_cast<const half8_t*>(lds + base + (uint32_t)i * 4096u);
+  };
+
+  float16_t acc[TM][2];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // ---- prologue: rings of four register sets and four LDS stages, everything modulo 4 -----
+  // activations of step T: global -> registers during step T-4, registers -> LDS stage T%4
+  // during step T-2, multiplied in step T;  packed weights of step T: loaded during step T-3.
+  u32x4 xr[4][XL];
+  RawB<BITS> rb[4];
+  static_for_d<0, 3>([&](auto tc) {
+    constexpr int T = decltype(tc)::value;
+    static_for_d<0, PBL>([&](auto cc) { load_b(rb[T], T, cc); });
+  });
+  load_scales(sc_cur, 0);
+  load_scales(sc_nxt, 4);
+  static_for_d<0, 4>([&](auto tc) {
+    constexpr int T = decltype(tc)::value;
+    static_for_d<0, XL>([&](auto ic) { load_x(xr[T], T, ic); });
+  });
+  static_for_d<0, 2>([&](auto tc) {
+    constexpr int T = decltype(tc)::value;
+    static_for_d<0, XL>([&](auto ic) { store_x(xr[T], (uint32_t)(T * STAGE), ic); });
+  });
+  __syncthreads();
+  static_for_d<0, TM>([&](auto ic) { read_a(0, a_rd[0], ic); });
+#pragma unroll
+  for (int j = 0; j < 2; ++j) s_step[0][j] = pick_scale(sc_cur, j, 0);
+  // prime the conversion pipeline: pairs 0..4 complete, 5 / 6 / 7 three / two / one stage in
+  static_for_d<0, 5>([&](auto gc) {
+    constexpr int g = decltype(gc)::value;
+    fbq[g / 4][g & 3] = stage_scale(0, stage_center(stage_bits(stage_perm(rb[0], gc))), gc);
+  });
+  t_center = stage_center(stage_bits(stage_perm(rb[0], std::integral_constant<int, 5>{})));
+  t_bits = stage_bits(stage_perm(rb[0], std::integral_constant<int, 6>{}));
+  t_perm = stage_perm(rb[0], std::integral_constant<int, 7>{});
+
+  // One K step, P = kt % 4 fixes every register set and LDS stage at compile time.
+  constexpr int NMFMA = TM * 2 * 4;
+  auto step = [&](auto pc, int kt) {
+    constexpr int P = decltype(pc)::value;
+    RawB<BITS>& bcur = rb[P];
+    RawB<BITS>& bnxt = rb[(P + 1) & 3];
+    RawB<BITS>& bload = rb[(P + 3) & 3];   // receives step kt+3
+    constexpr uint32_t st_rd = (uint32_t)(P * STAGE), st_next = (uint32_t)(((P + 1) & 3) * STAGE);
+    constexpr uint32_t st_wr = (uint32_t)(((P + 2) & 3) * STAGE);
+    // scales of the next step (its first pairs are converted at the end of this one)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      s_step[(P + 1) & 1][j] = P < 3 ? pick_scale(sc_cur, j, P + 1) : pick_scale(sc_nxt, j, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for_d<0, NMFMA>([&](auto sc) {
+      constexpr int s = decltype(sc)::value;
+      constexpr int kk = s / (2 * TM), j = (s / TM) % 2, i = s % TM;
+      constexpr int q = kk * 2 + j;  // index of the B fragment in use
+      const half8_t bm = __builtin_bit_cast(half8_t, fbq[q & 3]);
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk & 1][i], bm, acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // pair conversion pipeline: slot s finishes pair s+5 and starts pair s+8 (pairs 32..
+      // belong to the next step's packed weights)
+      {
+        constexpr int gd = s + 5, ga = s + 8;
+        fbq[(gd / 4) & 3][gd & 3] = stage_scale(gd < 32 ? (P & 1) : ((P + 1) & 1), t_center,
+                                                std::integral_constant<int, gd & 31>{});
+        t_center = stage_center(t_bits);
+        t_bits = stage_bits(t_perm);
+        t_perm = ga < 32 ? stage_perm(bcur, std::integral_constant<int, ga & 31>{})
+                         : stage_perm(bnxt, std::integral_constant<int, ga & 31>{});
+      }
+      // A fragments of the next slice (slice 0 of the next stage at the end), one per slot
+      if constexpr (j == 0)
+        read_a((kk + 1) & 1, a_rd[(kk + 1) & 3] + (kk == 3 ? st_next : st_rd), std::integral_constant<int, i>{});
+      // packed weights of step kt+3
+      if constexpr (s < PBL) load_b(bload, kt + 3, std::integral_constant<int, s>{});
+      // activations: global -> registers (step kt+4), registers -> LDS (step kt+2)
+      if constexpr (j == 1 && kk < 2) {
+        if constexpr (kk * TM + i < XL) load_x(xr[P], kt + 4, std::integral_constant<int, kk * TM + i>{});
+      }
+      if constexpr (j == 1 && kk >= 2) {
+        if constexpr ((kk - 2) * TM + i < XL)
+          store_x(xr[(P + 2) & 3], st_wr, std::integral_constant<int, (kk - 2) * TM + i>{});
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    __syncthreads();
+  };
+
+  const int ksteps4 = (ksteps + 3) & ~3;  // padded steps load zeros (out-of-range offsets)
+  for (int kt = 0; kt < ksteps4; kt += 4) {
+    step(std::integral_constant<int, 0>{}, kt);
+    step(std::integral_constant<int, 1>{}, kt + 1);
+    step(std::integral_constant<int, 2>{}, kt + 2);
+    step(std::integral_constant<int, 3>{}, kt + 3);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < SW; ++q) sc_cur[j][q] = sc_nxt[j][q];
+    load_scales(sc_nxt, kt + 8);
+  }
+
+  // ---- epilogue: lane holds column (lane % 32) and rows 8*(v/4) + 4*(lane/32) + v%4 ------
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wave * 64 + j * 32 + fr;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
+        if (m < M && n < N) y[(size_t)m * N + n] = (half_t)acc[i][j][v];
+      }
+    }
+}
+
+namespace {
+
+template <int BITS, int TM, int WAVES>
+void launch_direct(const Problem& p, int group_shift) {
+  constexpr int BM = TM * 32, BN = WAVES * 64;
+  const int tiles_m = (int)((p.m + BM - 1) / BM);
+  const int tiles_n = (int)((p.n + BN - 1) / BN);
+  dim3 grid(tiles_m * tiles_n), block(WAVES * 64);
+  constexpr size_t lds_bytes = 4 * (size_t)BM * 128;
+  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, TM, WAVES>), grid, block, lds_bytes, p.stream,
+                     (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
+                     (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
+                     tiles_n);
+}
+
+}  // namespace
+
+// variant: 1 = 128 x 256 tile (four wavefronts of 128 x 64)
+bool launch_gemm_direct(const Problem& p, int group_shift, int variant) {
+  if (!gemm_pipe_applicable(p)) return false;
+  // scales are fetched per 256 k: the kernel is laid out for the two benchmark quantizations
+  if (p.k % 256 != 0 || p.group != (p.bits == 4 ? 32 : 128)) return false;
+  switch (variant) {
+    case 1:
+      if (p.bits == 4) launch_direct<4, 4, 4>(p, group_shift);
+      else launch_direct<8, 4, 4>(p, group_shift);
+      return true;
+    default: return false;
+  }
+}
+
+}  // namespace wq

@@ -23,6 +23,7 @@ int launch_skinny(const Problem& p, int variant);
 int launch_gemm(const Problem& p, int variant);
 bool gemm_pipe_applicable(const Problem& p);  // K % 64 == 0, operands below 1 GiB
 bool launch_gemm_pipe(const Problem& p, int group_shift, int variant);
+bool launch_gemm_direct(const Problem& p, int group_shift, int variant);
 int launch_dequant(const Problem& p, void* wd);
 
 // Upper bound of rows the skinny family accepts.
