@@ -213,11 +213,15 @@ int launch_gemm(const Problem& p, int variant) {
     return -1;
   }
   if (variant == 0 && gemm_pipe_applicable(p)) {
-    // measured on MI355X: the 256x128 tile wins once M fills it a few times over;
-    // smaller M keeps more workgroups in flight with 128x128 tiles
-    variant = p.m >= 1024 ? 11 : 12;
+    // measured on MI355X, M = 128 .. 4096 on the Llama shapes: the direct-weight kernel with
+    // two K groups wins everywhere it applies; next the same kernel with one group, then the
+    // LDS-staged pipeline (256x128 tile once M fills it a few times over, else 128x128)
+    if (launch_gemm_direct(p, group_shift, 2) || launch_gemm_direct(p, group_shift, 1)) variant = -1;
+    else variant = p.m >= 1024 ? 11 : 12;
   }
-  if (variant >= 21) {
+  if (variant == -1) {
+    // launched above
+  } else if (variant >= 21) {
     if (!launch_gemm_direct(p, group_shift, variant - 20)) {
       set_error("gemm kernel: direct-weight variant %d does not apply to M=%lld N=%lld K=%lld group=%d",
                 variant, (long long)p.m, (long long)p.n, (long long)p.k, p.group);

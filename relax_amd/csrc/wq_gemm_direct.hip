@@ -19,18 +19,24 @@
 // XOR-swizzled with (row & 7), conflict-free for the reads (8 rows x same chunk, and
 // chunk c with chunk c+4 of the other half-wave) and for the row-contiguous writes.
 //
-// Pipeline per K step t (four activation stages in LDS, rings of four register sets for
-// activations and packed weights: workgroups sharing a tile run in lockstep, so every
-// global load sees close to the full memory latency and is issued 2.5 - 3 steps ahead);
-// program order is issue order, a handful of independent instructions after every MFMA,
-// fenced with sched_barrier:
-//   global -> registers : activations of step t+4, packed weights + scales of step t+3
+// Pipeline per K step t (four activation stages in LDS; program order is issue order, a
+// handful of independent instructions after every MFMA, fenced with sched_barrier):
+//   global -> registers : activations of step t+4 (t+3 with K groups), packed weights of
+//                         step t+3 (t+2 with two register sets), scales per four steps
 //   registers -> LDS    : activations of step t+2
 //   LDS -> registers    : A fragments of the next k slice (of step t+1 at the end)
 //   dequantize          : one stage each of four pair conversions per MFMA slot
 //
-// Shape requirements (checked by the launcher): K a multiple of 256, group 32 (int4) or
-// 128 (int8), operands < 1 GiB; other shapes use the other GEMM kernels.
+// K groups (GROUPS = 2): eight wavefronts, two per SIMD.  Wavefronts 0-3 accumulate the
+// first half of K and wavefronts 4-7 the second half of the same 128 x 256 tile, each group
+// with its own activation stages; at the end the second group hands its partial sums to the
+// first through LDS.  A stall of one wavefront (barrier, memory wait) is covered by the
+// other one on its SIMD, and a tile takes half as many sequential K steps, which is what
+// counts when M is too small to give every CU a tile.
+//
+// Shape requirements (checked by the launcher): K a multiple of 256 (at least 512 for K
+// groups), group 32 (int4) or 128 (int8), operands < 1 GiB; other shapes use the other GEMM
+// kernels.
 #include <type_traits>
 
 #include "wq_device.h"
@@ -57,23 +63,25 @@ struct RawB {
   u32x4 w[2][NV];                               // [column tile][load]
 };
 
-template <int BITS, int TM, int WAVES>
-__global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
+template <int BITS, int GROUPS>
+__global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
     half_t* __restrict__ y, int M, int N, int K, int group_shift, int zero_point, int tiles_m,
     int tiles_n) {
-  constexpr int BK = 64;
-  static_assert(TM == 4, "the pair-conversion pipeline is laid out for four MFMA slots per B fragment");
-  constexpr int BM = TM * 32, BN = WAVES * 64;
-  constexpr int NT = WAVES * 64;
+  constexpr int BK = 64, TM = 4, WAVES = 4;
+  constexpr int BM = TM * 32;
+  constexpr int NT = WAVES * 64;   // threads of one K group
   constexpr int CH = 128 / BITS;   // k per 16-byte packed chunk
   constexpr int NV = RawB<BITS>::NV;
   constexpr int XL = BM * 8 / NT;  // 16-byte activation chunks per thread per step
   constexpr int STAGE = BM * 128;  // bytes per LDS stage
-  static_assert(XL >= 1 && BM * 8 % NT == 0 && (NT / 8) % 8 == 0, "activation tile / thread split");
+  // register sets: two wavefronts per SIMD leave 128 VGPRs beside the accumulators and hide
+  // latency by themselves, so the K-group variant prefetches only one step deep
+  constexpr int RB = (BITS == 4 && GROUPS == 1) ? 4 : 2;  // packed weights
+  constexpr int XS = GROUPS == 1 ? 2 : 1;                 // activations
+  static_assert(XL == 4, "activation tile / thread split");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char wq_gemm_direct_smem[];
-  unsigned char* const lds = wq_gemm_direct_smem;
 
   // XCD-aware tile order: consecutive workgroup ids land on different XCDs; regroup them so
   // that each XCD owns a contiguous range of activation row blocks (which then stay in its
@@ -82,12 +90,22 @@ __global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
   int bid = blockIdx.x;
   if ((nblocks & 7) == 0) bid = (bid & 7) * (nblocks >> 3) + (bid >> 3);
   const int tile_m = bid / tiles_n, tile_n = bid % tiles_n;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int m0 = tile_m * BM, n0 = tile_n * (WAVES * 64);
 
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = threadIdx.x & 63;
+  const int wave_id = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = GROUPS == 1 ? 0 : wave_id >> 2;  // K group of this wavefront
+  const int wave = wave_id & 3;                    // 64-column slice of the tile
+  const int tid = threadIdx.x & (NT - 1);          // thread index inside the K group
   const int fr = lane & 31, fh = lane >> 5;
+  unsigned char* const lds = wq_gemm_direct_smem + grp * (4 * STAGE);  // the group's four stages
+
+  // K range of this group, in 64-wide steps; both groups run the same number of steps and
+  // the shorter one reads zeros (out-of-range offsets) past its end.
+  const int ksteps = K / BK;
+  const int nloop = GROUPS == 1 ? ksteps : 4 * ((ksteps / 4 + 1) / 2);
+  const int kbase = grp * nloop;
+  const int kend = GROUPS == 1 ? ksteps : (grp == 0 ? nloop : ksteps);
 
   const uint32_t row_bytes = (uint32_t)K * BITS / 8;
   const uint32_t groups_per_row = ((uint32_t)K / CH) >> group_shift;
@@ -121,11 +139,10 @@ __global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
     a_rd[kk] = (uint32_t)fr * 128u + (uint32_t)(((fh * 4 + kk) ^ (fr & 7)) << 4);
 
   const Q4Consts qc = make_q4_consts(zero_point);
-  const int ksteps = K / BK;
 
   auto load_x = [&](u32x4 (&xr)[XL], int kt, auto ic) {
     constexpr int i = decltype(ic)::value;
-    const uint32_t xk = kt < ksteps ? (uint32_t)kt * BK * 2u : kStepOobD;
+    const uint32_t xk = kt < kend ? (uint32_t)kt * BK * 2u : kStepOobD;
     xr[i] = load_b128(rx, xg[i] + xk);
   };
   auto store_x = [&](const u32x4 (&xr)[XL], uint32_t stage_base, auto ic) {
@@ -136,7 +153,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
   auto load_b = [&](RawB<BITS>& b, int kt, auto cc) {
     constexpr int c = decltype(cc)::value, j = c / NV, v = c % NV;
     const uint32_t k0 = (uint32_t)kt * BK;
-    b.w[j][v] = load_b128(rw, wg[j] + (kt < ksteps ? k0 * BITS / 8 : kStepOobD) + v * 16u);
+    b.w[j][v] = load_b128(rw, wg[j] + (kt < kend ? k0 * BITS / 8 : kStepOobD) + v * 16u);
   };
   constexpr int PBL = 2 * NV;  // packed-weight load pieces per step
 
@@ -147,10 +164,10 @@ __global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
   uint32_t sc_cur[2][SW], sc_nxt[2][SW];
   auto load_scales = [&](uint32_t (&sc)[2][SW], int kt0) {
     // kt0: first step of the macro step (a multiple of 4)
-    const bool ok = kt0 < ksteps;
+    const bool ok = kt0 < kend;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const uint32_t off = ok ? sg[j] + (uint32_t)kt0 * (BK / (BITS == 4 ? 32 : 128)) * 2u : kStepOobD;
+      const uint32_t off = ok ? sg[j] + (uint32_t)kt0 * BK / (BITS == 4 ? 32 : 128) * 2u : kStepOobD;
       if constexpr (BITS == 4) {
         const u32x4 v = load_b128(rs, off);
 #pragma unroll
@@ -211,25 +228,39 @@ __global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  // ---- prologue: rings of four register sets and four LDS stages, everything modulo 4 -----
-  // activations of step T: global -> registers during step T-4, registers -> LDS stage T%4
-  // during step T-2, multiplied in step T;  packed weights of step T: loaded during step T-3.
-  u32x4 xr[4][XL];
-  RawB<BITS> rb[4];
-  static_for_d<0, 3>([&](auto tc) {
+  // ---- prologue ---------------------------------------------------------------------------
+  // activations of step T: global -> register set T%2 late in step T-4 (one set: in step
+  // T-3), registers -> LDS stage T%4 early in step T-2, multiplied in step T;  packed weights of step T: loaded
+  // into set T%RB three steps ahead (int4), or late in step T-2 (int8, two sets).  (Step numbers below are relative to the group's first.)
+  u32x4 xr[XS][XL];
+  RawB<BITS> rb[RB];
+  static_for_d<0, (RB == 2 ? 2 : RB - 1)>([&](auto tc) {
     constexpr int T = decltype(tc)::value;
-    static_for_d<0, PBL>([&](auto cc) { load_b(rb[T], T, cc); });
+    static_for_d<0, PBL>([&](auto cc) { load_b(rb[T], kbase + T, cc); });
   });
-  load_scales(sc_cur, 0);
-  load_scales(sc_nxt, 4);
-  static_for_d<0, 4>([&](auto tc) {
-    constexpr int T = decltype(tc)::value;
-    static_for_d<0, XL>([&](auto ic) { load_x(xr[T], T, ic); });
-  });
-  static_for_d<0, 2>([&](auto tc) {
-    constexpr int T = decltype(tc)::value;
-    static_for_d<0, XL>([&](auto ic) { store_x(xr[T], (uint32_t)(T * STAGE), ic); });
-  });
+  load_scales(sc_cur, kbase);
+  load_scales(sc_nxt, kbase + 4);
+  if constexpr (XS == 2) {
+    static_for_d<0, 2>([&](auto tc) {
+      constexpr int T = decltype(tc)::value;
+      static_for_d<0, XL>([&](auto ic) { load_x(xr[T], kbase + T, ic); });
+    });
+    static_for_d<0, 2>([&](auto tc) {
+      constexpr int T = decltype(tc)::value;
+      static_for_d<0, XL>([&](auto ic) { store_x(xr[T], (uint32_t)(T * STAGE), ic); });
+    });
+    static_for_d<0, 2>([&](auto tc) {
+      constexpr int T = decltype(tc)::value;
+      static_for_d<0, XL>([&](auto ic) { load_x(xr[T], kbase + 2 + T, ic); });
+    });
+  } else {
+    static_for_d<0, 2>([&](auto tc) {
+      constexpr int T = decltype(tc)::value;
+      static_for_d<0, XL>([&](auto ic) { load_x(xr[0], kbase + T, ic); });
+      static_for_d<0, XL>([&](auto ic) { store_x(xr[0], (uint32_t)(T * STAGE), ic); });
+    });
+    static_for_d<0, XL>([&](auto ic) { load_x(xr[0], kbase + 2, ic); });
+  }
   __syncthreads();
   static_for_d<0, TM>([&](auto ic) { read_a(0, a_rd[0], ic); });
 #pragma unroll
@@ -243,13 +274,14 @@ __global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
   t_bits = stage_bits(stage_perm(rb[0], std::integral_constant<int, 6>{}));
   t_perm = stage_perm(rb[0], std::integral_constant<int, 7>{});
 
-  // One K step, P = kt % 4 fixes every register set and LDS stage at compile time.
+  // One K step, P = (step number in the group) % 4 fixes every register set and LDS stage at
+  // compile time.
   constexpr int NMFMA = TM * 2 * 4;
   auto step = [&](auto pc, int kt) {
     constexpr int P = decltype(pc)::value;
-    RawB<BITS>& bcur = rb[P];
-    RawB<BITS>& bnxt = rb[(P + 1) & 3];
-    RawB<BITS>& bload = rb[(P + 3) & 3];   // receives step kt+3
+    RawB<BITS>& bcur = rb[P % RB];
+    RawB<BITS>& bnxt = rb[(P + 1) % RB];
+    RawB<BITS>& bload = rb[(P + RB - 1) % RB];   // receives step kt + RB - 1
     constexpr uint32_t st_rd = (uint32_t)(P * STAGE), st_next = (uint32_t)(((P + 1) & 3) * STAGE);
     constexpr uint32_t st_wr = (uint32_t)(((P + 2) & 3) * STAGE);
     // scales of the next step (its first pairs are converted at the end of this one)
@@ -278,23 +310,26 @@ __global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
       // A fragments of the next slice (slice 0 of the next stage at the end), one per slot
       if constexpr (j == 0)
         read_a((kk + 1) & 1, a_rd[(kk + 1) & 3] + (kk == 3 ? st_next : st_rd), std::integral_constant<int, i>{});
-      // packed weights of step kt+3
-      if constexpr (s < PBL) load_b(bload, kt + 3, std::integral_constant<int, s>{});
-      // activations: global -> registers (step kt+4), registers -> LDS (step kt+2)
-      if constexpr (j == 1 && kk < 2) {
-        if constexpr (kk * TM + i < XL) load_x(xr[P], kt + 4, std::integral_constant<int, kk * TM + i>{});
+      // activations: registers -> LDS (step kt+2), then the same registers <- global (step kt+4)
+      if constexpr (kk == 0 && j == 1) store_x(xr[P % XS], st_wr, std::integral_constant<int, i>{});
+      if constexpr (XS == 2) {
+        if constexpr (kk == 2 && j == 1) load_x(xr[P & 1], kt + 4, std::integral_constant<int, i>{});
+      } else {
+        if constexpr (kk == 1 && j == 1) load_x(xr[0], kt + 3, std::integral_constant<int, i>{});
       }
-      if constexpr (j == 1 && kk >= 2) {
-        if constexpr ((kk - 2) * TM + i < XL)
-          store_x(xr[(P + 2) & 3], st_wr, std::integral_constant<int, (kk - 2) * TM + i>{});
+      // packed weights of step kt + RB - 1, into the set whose last use has passed
+      if constexpr (RB == 4) {
+        if constexpr (kk == 1 && j == 1 && i < PBL) load_b(bload, kt + 3, std::integral_constant<int, i>{});
+      } else {
+        // two sets: the current step's set is free once its last pair has entered the pipeline
+        if constexpr (kk == 3 && j == 1 && i < PBL) load_b(bcur, kt + 2, std::integral_constant<int, i>{});
       }
       __builtin_amdgcn_sched_barrier(0);
     });
     __syncthreads();
   };
 
-  const int ksteps4 = (ksteps + 3) & ~3;  // padded steps load zeros (out-of-range offsets)
-  for (int kt = 0; kt < ksteps4; kt += 4) {
+  for (int kt = kbase; kt < kbase + nloop; kt += 4) {
     step(std::integral_constant<int, 0>{}, kt);
     step(std::integral_constant<int, 1>{}, kt + 1);
     step(std::integral_constant<int, 2>{}, kt + 2);
@@ -304,6 +339,42 @@ __global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
 #pragma unroll
       for (int q = 0; q < SW; ++q) sc_cur[j][q] = sc_nxt[j][q];
     load_scales(sc_nxt, kt + 8);
+  }
+
+  // ---- K groups: the second group hands its partial sums over through LDS -----------------
+  // Two rounds of 64 KB (row blocks i = 0,1 then 2,3); a wavefront and its partner hold the
+  // same elements in the same lanes, so the exchange is lane-contiguous 16-byte vectors.
+  if constexpr (GROUPS == 2) {
+    float4_t* const xch = reinterpret_cast<float4_t*>(wq_gemm_direct_smem) + wave * (16 * 64) + lane;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      if (grp == 1) {
+#pragma unroll
+        for (int il = 0; il < 2; ++il)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v4 = 0; v4 < 4; ++v4) {
+              const float16_t& a = acc[h * 2 + il][j];
+              xch[((il * 2 + j) * 4 + v4) * 64] = float4_t{a[v4 * 4], a[v4 * 4 + 1], a[v4 * 4 + 2], a[v4 * 4 + 3]};
+            }
+      }
+      __syncthreads();
+      if (grp == 0) {
+#pragma unroll
+        for (int il = 0; il < 2; ++il)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v4 = 0; v4 < 4; ++v4) {
+              const float4_t o = xch[((il * 2 + j) * 4 + v4) * 64];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[h * 2 + il][j][v4 * 4 + e] += o[e];
+            }
+      }
+      __syncthreads();
+    }
+    if (grp == 1) return;
   }
 
   // ---- epilogue: lane holds column (lane % 32) and rows 8*(v/4) + 4*(lane/32) + v%4 ------
@@ -322,14 +393,19 @@ __global__ __launch_bounds__(WAVES * 64, 1) void wq_gemm_direct_kernel(
 
 namespace {
 
-template <int BITS, int TM, int WAVES>
+template <int BITS, int GROUPS>
 void launch_direct(const Problem& p, int group_shift) {
-  constexpr int BM = TM * 32, BN = WAVES * 64;
+  constexpr int BM = 128, BN = 256;
   const int tiles_m = (int)((p.m + BM - 1) / BM);
   const int tiles_n = (int)((p.n + BN - 1) / BN);
-  dim3 grid(tiles_m * tiles_n), block(WAVES * 64);
-  constexpr size_t lds_bytes = 4 * (size_t)BM * 128;
-  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, TM, WAVES>), grid, block, lds_bytes, p.stream,
+  dim3 grid(tiles_m * tiles_n), block(GROUPS * 256);
+  constexpr size_t lds_bytes = (size_t)GROUPS * 4 * BM * 128;  // four activation stages per K group
+  static const bool attr_set = [] {
+    return hipFuncSetAttribute((const void*)wq_gemm_direct_kernel<BITS, GROUPS>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) == hipSuccess;
+  }();
+  (void)attr_set;
+  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
                      tiles_n);
@@ -337,15 +413,21 @@ void launch_direct(const Problem& p, int group_shift) {
 
 }  // namespace
 
-// variant: 1 = 128 x 256 tile (four wavefronts of 128 x 64)
+// 128 x 256 tile; variant 1: four wavefronts (one per SIMD), variant 2: eight wavefronts in
+// two K groups (two per SIMD), each group accumulating half of K
 bool launch_gemm_direct(const Problem& p, int group_shift, int variant) {
   if (!gemm_pipe_applicable(p)) return false;
   // scales are fetched per 256 k: the kernel is laid out for the two benchmark quantizations
   if (p.k % 256 != 0 || p.group != (p.bits == 4 ? 32 : 128)) return false;
   switch (variant) {
     case 1:
-      if (p.bits == 4) launch_direct<4, 4, 4>(p, group_shift);
-      else launch_direct<8, 4, 4>(p, group_shift);
+      if (p.bits == 4) launch_direct<4, 1>(p, group_shift);
+      else launch_direct<8, 1>(p, group_shift);
+      return true;
+    case 2:
+      if (p.k < 512) return false;
+      if (p.bits == 4) launch_direct<4, 2>(p, group_shift);
+      else launch_direct<8, 2>(p, group_shift);
       return true;
     default: return false;
   }

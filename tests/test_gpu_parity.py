@@ -190,6 +190,35 @@ def test_gemm_kernel_matches_oracle(bits, m, n, k):
     assert_close(got, want, (bits, m, n, k))
 
 
+@pytest.mark.parametrize("variant,bits,m,n,k", [
+    (21, 4, 300, 200, 256), (21, 4, 129, 520, 1280), (21, 8, 129, 72, 256), (21, 8, 513, 260, 1024),
+    (22, 4, 300, 200, 512), (22, 4, 129, 520, 1280), (22, 4, 70, 136, 768), (22, 8, 513, 260, 1024),
+    (22, 8, 65, 300, 1792)])
+def test_gemm_direct_weight_variants_match_oracle(variant, bits, m, n, k):
+    """Direct-weight kernel with one (21) and two (22) K groups: ragged M and N, K of one macro step,
+    an even and an odd number of 256-wide macro steps (the second K group is then the shorter one)."""
+    from relax_amd import lib
+
+    x, wq, s, g = O.make_case(500 + m + n, m, n, k, bits)
+    got = run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_GEMM, variant=variant)
+    want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
+    assert_close(got, want, (variant, bits, m, n, k))
+
+
+def test_gemm_direct_weight_variant_refuses_other_layouts():
+    """K not a multiple of 256 or a non-default group size: the variant refuses, the default dispatch
+    falls back to another GEMM kernel with the same result."""
+    from relax_amd import lib
+
+    for bits, m, n, k, group in [(4, 200, 96, 320, 32), (4, 200, 96, 512, 64), (8, 200, 96, 512, 64)]:
+        x, wq, s, g = O.make_case(9, m, n, k, bits, group)
+        for variant in (21, 22):
+            with pytest.raises(lib.WqError, match="does not apply"):
+                run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_GEMM, variant=variant)
+        assert_close(run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_GEMM),
+                     c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=8), (bits, m, n, k, group))
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 11, 12, 13])
 @pytest.mark.parametrize("bits,m,n,k", [(4, 300, 200, 128), (4, 70, 136, 448), (4, 513, 72, 320),
                                          (8, 129, 72, 256), (8, 513, 260, 1024)])
