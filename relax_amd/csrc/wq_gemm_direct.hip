@@ -83,13 +83,21 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
 
   extern __shared__ __attribute__((aligned(16))) unsigned char wq_gemm_direct_smem[];
 
-  // XCD-aware tile order: consecutive workgroup ids land on different XCDs; regroup them so
-  // that each XCD owns a contiguous range of activation row blocks (which then stay in its
-  // L2) and streams the much smaller packed weights once.
+  // XCD-aware tile order.  Consecutive workgroup ids land on different XCDs; regroup them so
+  // that each XCD owns a contiguous range of the tile list, and order the list in column
+  // panels of eight tiles, row-major inside a panel: the 32 workgroups an XCD runs at a time
+  // then cover 4 activation row blocks x 8 weight column tiles and walk K together, so its L2
+  // serves every activation block eight times and every weight tile four times per fetch.
   const int nblocks = tiles_m * tiles_n;
   int bid = blockIdx.x;
   if ((nblocks & 7) == 0) bid = (bid & 7) * (nblocks >> 3) + (bid >> 3);
-  const int tile_m = bid / tiles_n, tile_n = bid % tiles_n;
+  constexpr int PANEL = 8;
+  const int full = tiles_n / PANEL;                 // panels of full width
+  const int in_full = bid / (tiles_m * PANEL);      // panel index if inside the full ones
+  const int panel = min(in_full, full);
+  const int width = panel < full ? PANEL : tiles_n - full * PANEL;
+  const int rest = bid - panel * tiles_m * PANEL;
+  const int tile_m = rest / width, tile_n = panel * PANEL + rest % width;
   const int m0 = tile_m * BM, n0 = tile_n * (WAVES * 64);
 
   const int lane = threadIdx.x & 63;
