@@ -67,6 +67,40 @@ MI355X_WQ_API int mi355x_wq_matmul(const mi355x_wq_desc* desc, const void* x, co
 MI355X_WQ_API int mi355x_wq_matmul_ex(const mi355x_wq_desc* desc, const void* x, const void* wq,
                         const void* scales, void* y, int64_t m, void* stream, int kernel);
 
+/* Element-wise operations fused behind the matmul, in the order a composite applies them to
+ * t0 = f16(accumulator): t1 = t0 + bias[n]; t2 = act(t1); y = t2 + residual[m,n].  Every
+ * step is one float16 operation with one rounding, as the CPU path executes `relax.add` /
+ * `relax.nn.relu` on float16 tensors (python/tvm/relax/transform/legalize_ops.py:632;
+ * relu = max(t, 0): python/tvm/topi/nn/elemwise.py:26-39, lowered to select(t > 0, t, 0):
+ * src/target/llvm/codegen_llvm.cc:1500-1504).  This is the
+ * `matmul_bias` / `matmul_bias_relu` family of the reference's pattern helpers
+ * (python/tvm/relax/dpl/pattern.py:1049-1095) and of its CUTLASS epilogues
+ * (python/tvm/contrib/cutlass/gen_tensor_op.py:377-380), plus the residual add that follows
+ * the O and down projections of a decoder layer.  `relax.nn.gelu` is not offered: the CPU
+ * path cannot lower erf on float16 (src/target/intrin_rule.h:39-48), so there is nothing to match. */
+enum {
+  MI355X_WQ_ACT_NONE = 0,
+  MI355X_WQ_ACT_RELU = 1
+};
+typedef struct mi355x_wq_epilogue {
+  const void* bias;     /* float16 [N] (device), or NULL */
+  const void* residual; /* float16 [M,N] (device, compact), or NULL; may be `y` itself */
+  int32_t activation;   /* MI355X_WQ_ACT_* */
+  int32_t reserved;     /* must be 0 */
+} mi355x_wq_epilogue;
+
+/* y[M,N] = epilogue( f16( x @ dequant(wq, scales)^T ) ); `ep` NULL or all-empty = plain matmul.
+ * Same kernels as mi355x_wq_matmul; the epilogue runs on the accumulator registers, so the
+ * matmul result makes no extra trip through HBM. */
+MI355X_WQ_API int mi355x_wq_matmul_fused(const mi355x_wq_desc* desc, const void* x, const void* wq,
+                           const void* scales, const mi355x_wq_epilogue* ep, void* y, int64_t m,
+                           void* stream);
+
+/* Same, with the kernel family forced (tests and benchmarks). */
+MI355X_WQ_API int mi355x_wq_matmul_fused_ex(const mi355x_wq_desc* desc, const void* x, const void* wq,
+                              const void* scales, const mi355x_wq_epilogue* ep, void* y, int64_t m,
+                              void* stream, int kernel);
+
 /* wd[N,K] = dequant(wq, scales), bit-exact with the float16 arithmetic of the
  * `decode` PrimFunc as the llvm target lowers it
  * (src/target/llvm/codegen_llvm.cc:820-852, 1271-1285). */

@@ -68,6 +68,8 @@ enum {
  * the reference backend (src/relay/backend/contrib/codegen_c/codegen_c.h:101-121,
  * 163-235).  Arguments, all tensors (type code 7 or 13):
  *   matmul     : x[M,K] f16, wq[N,K*bits/32] u32, scales[N,K/group] f16, y[M,N] f16 (output, last)
+ *   matmul_bias / matmul_bias_relu : x, wq, scales, bias[N] f16, y
+ *   matmul_residual                : x, wq, scales, residual[M,N] f16, y
  *   dequantize : wq, scales, wd[N,K] f16 (output, last)
  * group is K / scales.shape[1]; the zero point is 7 (q4f16) or 0 (q8f16).
  * Return 0, or -1 after recording the message with TVMAPISetLastError (when the
@@ -78,6 +80,22 @@ MI355X_WQ_API int mi355x_q4f16_matmul(mi355x_tvm_value* args, int* type_codes, i
                         mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
 MI355X_WQ_API int mi355x_q8f16_matmul(mi355x_tvm_value* args, int* type_codes, int num_args,
                         mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
+MI355X_WQ_API int mi355x_q4f16_matmul_bias(mi355x_tvm_value* args, int* type_codes, int num_args,
+                             mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
+MI355X_WQ_API int mi355x_q4f16_matmul_bias_relu(mi355x_tvm_value* args, int* type_codes, int num_args,
+                                  mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
+                                  void* resource_handle);
+MI355X_WQ_API int mi355x_q4f16_matmul_residual(mi355x_tvm_value* args, int* type_codes, int num_args,
+                                 mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
+                                 void* resource_handle);
+MI355X_WQ_API int mi355x_q8f16_matmul_bias(mi355x_tvm_value* args, int* type_codes, int num_args,
+                             mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
+MI355X_WQ_API int mi355x_q8f16_matmul_bias_relu(mi355x_tvm_value* args, int* type_codes, int num_args,
+                                  mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
+                                  void* resource_handle);
+MI355X_WQ_API int mi355x_q8f16_matmul_residual(mi355x_tvm_value* args, int* type_codes, int num_args,
+                                 mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
+                                 void* resource_handle);
 MI355X_WQ_API int mi355x_q4f16_dequantize(mi355x_tvm_value* args, int* type_codes, int num_args,
                             mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
                             void* resource_handle);
@@ -102,7 +120,11 @@ typedef struct mi355x_wq_callspec {
   int32_t arg_wq;
   int32_t arg_scales;
   int32_t arg_out;
-  int32_t num_args;   /* expected argument count */
+  int32_t num_args;   /* expected argument count: 4 (matmul) / 3 (dequantize) + fused operands */
+  /* fused epilogue of a matmul composite (mi355x_wq_epilogue in mi355x_wq.h) */
+  int32_t arg_bias;     /* argument index of bias [N] or [1,N] float16, or -1 */
+  int32_t arg_residual; /* argument index of residual [M,N] float16, or -1 */
+  int32_t activation;   /* MI355X_WQ_ACT_* */
 } mi355x_wq_callspec;
 
 /* The body every entry (fixed-name or generated trampoline) forwards to. */
@@ -115,8 +137,9 @@ MI355X_WQ_API void mi355x_wq_packed_set_stream(void* stream);
 MI355X_WQ_API void* mi355x_wq_packed_get_stream(void);
 
 /*
- * Registers "mi355x.q4f16_matmul", "mi355x.q8f16_matmul", "mi355x.q4f16_dequantize"
- * and "mi355x.q8f16_dequantize" in TVM's global function table through the C API
+ * Registers every fixed-name entry above as "mi355x.<name without the mi355x_ prefix>"
+ * ("mi355x.q4f16_matmul", "mi355x.q4f16_matmul_bias", ..., "mi355x.q8f16_dequantize") in TVM's
+ * global function table through the C API
  * (TVMFuncCreateFromCFunc + TVMFuncRegisterGlobal,
  * include/tvm/runtime/c_runtime_api.h:362-405), resolved from the already loaded
  * TVM runtime with dlsym -- the same effect as TVM_REGISTER_GLOBAL

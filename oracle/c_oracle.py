@@ -37,6 +37,8 @@ def lib() -> C.CDLL:
         L.wq_oracle_matmul_f32acc.argtypes = [p, p, i64, i64, i64, p, C.c_int]
         L.wq_oracle_cast_f16.argtypes = [p, i64, p]
         L.wq_oracle_wq_matmul.argtypes = [C.c_int, i64, p, p, p, i64, i64, i64, p, p, p, C.c_int]
+        L.wq_oracle_epilogue.argtypes = [p, i64, i64, p, C.c_int, p]
+        L.wq_oracle_epilogue.restype = None
         _lib = L
     return _lib
 
@@ -112,6 +114,30 @@ def wq_matmul(x, wq, s, bits: int, group: int, nthreads: int = 1) -> np.ndarray:
     if rc != 0:
         raise ValueError("wq_oracle_wq_matmul rejected the arguments")
     return y
+
+
+def epilogue(y, bias=None, activation=None, residual=None) -> np.ndarray:
+    """Fused tail on a copy of y [M,N] float16: + bias[N], relu, + residual[M,N]."""
+    L = lib()
+    out = np.array(y, dtype=np.float16, order="C", copy=True)
+    m, n = out.shape
+    if activation not in (None, "none", "relu", "relax.nn.relu"):
+        raise ValueError(f"unsupported activation {activation!r}")
+    b = None if bias is None else np.ascontiguousarray(np.asarray(bias, dtype=np.float16).reshape(-1))
+    r = None if residual is None else np.ascontiguousarray(residual, dtype=np.float16)
+    if b is not None and b.shape != (n,):
+        raise ValueError("bias must have N elements")
+    if r is not None and r.shape != (m, n):
+        raise ValueError("residual must be [M, N]")
+    L.wq_oracle_epilogue(_ptr(out), m, n, None if b is None else _ptr(b),
+                         1 if activation in ("relu", "relax.nn.relu") else 0,
+                         None if r is None else _ptr(r))
+    return out
+
+
+def wq_matmul_fused(x, wq, s, bits: int, group: int, bias=None, activation=None, residual=None,
+                    nthreads: int = 1) -> np.ndarray:
+    return epilogue(wq_matmul(x, wq, s, bits, group, nthreads=nthreads), bias, activation, residual)
 
 
 def max_threads() -> int:

@@ -165,6 +165,24 @@ int wq_oracle_wq_matmul(int bits, int64_t group, const uint16_t* x, const uint32
   return 0;
 }
 
+/* ---- fused tail: y[m,n] = (relu?)(y[m,n] + bias[n]) + residual[m,n], each add one float16
+ * rounding (float32 sum of two float16 values, rounded to float16: the double rounding is
+ * innocuous because float32 carries 24 >= 2*11 + 2 significand bits); relu is
+ * select(t > 0, t, 0) -- src/target/llvm/codegen_llvm.cc:1500-1504.  bias / residual may be
+ * NULL. ---- */
+void wq_oracle_epilogue(uint16_t* y, int64_t m_rows, int64_t n_rows, const uint16_t* bias, int relu,
+                        const uint16_t* residual) {
+  for (int64_t m = 0; m < m_rows; ++m)
+    for (int64_t n = 0; n < n_rows; ++n) {
+      uint16_t h = y[m * n_rows + n];
+      if (bias) h = wq_oracle_f32_to_f16(wq_oracle_f16_to_f32(h) + wq_oracle_f16_to_f32(bias[n]));
+      if (relu) h = (wq_oracle_f16_to_f32(h) > 0.0f) ? h : (uint16_t)0;
+      if (residual)
+        h = wq_oracle_f32_to_f16(wq_oracle_f16_to_f32(h) + wq_oracle_f16_to_f32(residual[m * n_rows + n]));
+      y[m * n_rows + n] = h;
+    }
+}
+
 int wq_oracle_max_threads(void) {
 #if defined(_OPENMP)
   return omp_get_max_threads();

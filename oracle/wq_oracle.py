@@ -27,6 +27,13 @@ Reference semantics followed (file:line under the reference tree):
   python/tvm/relax/transform/legalize_ops.py:157-162,
   src/target/llvm/codegen_llvm.cc:849-850.
 
+* fused tail (composites with `relax.add` / `relax.nn.relu` behind the cast): each op is
+  legalized to its own element-wise PrimFunc on float16 tensors
+  (python/tvm/relax/transform/legalize_ops.py:632 and the binary-op table above it), so every
+  add rounds once to float16; relu is max(t, 0) (python/tvm/topi/nn/elemwise.py:26-39),
+  emitted as select(t > 0, t, 0) with an ordered compare
+  (src/target/llvm/codegen_llvm.cc:1500-1504): -0 and NaN both give +0.
+
 Layout decisions frozen by this build (the reference holds no quantized path):
 element k of a row lives in word k // per_word at bit offset
 (k % per_word) * bits, least-significant field first.
@@ -35,7 +42,9 @@ Pinning (see tests/test_oracle.py): unpack against an independent pure-Python
 bit walk over every field value and position; dequantize exhaustively against a
 float64 closed form for all 16 x 65536 (q4) and 256 x 65536 (q8) operand pairs;
 matmul against exact integer arithmetic, one-hot readback, a float64 bound and an
-order-sensitive hand-computed case.
+order-sensitive hand-computed case; the float16 add of the fused tail against exact
+rational arithmetic (fractions) with an independent nearest-even search over all float16
+values, and tie / overflow / signed-zero known answers; relu on the special values.
 """
 from __future__ import annotations
 
@@ -162,6 +171,46 @@ def wq_matmul(x, wq, s, bits: int, group: int) -> np.ndarray:
 # ----------------------------------------------------------------------------
 # synthetic inputs of the benchmark's distributions
 # ----------------------------------------------------------------------------
+def add_f16(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """IEEE binary16 addition, one rounding (broadcasting like `relax.add`).
+
+    The exact sum of two float16 values is computed in float64 (exact: both operands are
+    multiples of 2^-24 below 2^16, so the sum has at most 41 significant bits) and rounded
+    once to float16."""
+    a = np.asarray(a, dtype=np.float16)
+    b = np.asarray(b, dtype=np.float16)
+    with np.errstate(over="ignore", invalid="ignore"):
+        return (a.astype(np.float64) + b.astype(np.float64)).astype(np.float16)
+
+
+def relu_f16(t: np.ndarray) -> np.ndarray:
+    """select(t > 0, t, 0): negative values, -0 and NaN become +0."""
+    t = np.asarray(t, dtype=np.float16)
+    with np.errstate(invalid="ignore"):
+        return np.where(t > np.float16(0), t, np.float16(0)).astype(np.float16)
+
+
+def epilogue(y: np.ndarray, bias=None, activation: str | None = None, residual=None) -> np.ndarray:
+    """The fused tail of a composite applied to y = f16(accumulator):
+    + bias[N], then relu, then + residual[M,N]; every step absent or one float16 op."""
+    t = np.asarray(y, dtype=np.float16)
+    if bias is not None:
+        t = add_f16(t, np.asarray(bias, dtype=np.float16).reshape(1, -1))
+    if activation in ("relu", "relax.nn.relu"):
+        t = relu_f16(t)
+    elif activation not in (None, "none"):
+        raise ValueError(f"unsupported activation {activation!r}")
+    if residual is not None:
+        t = add_f16(t, residual)
+    return t
+
+
+def wq_matmul_fused(x, wq, s, bits: int, group: int, bias=None, activation: str | None = None,
+                    residual=None) -> np.ndarray:
+    """y = epilogue(f16(x @ dequant(Wq, S)^T))."""
+    return epilogue(wq_matmul(x, wq, s, bits, group), bias, activation, residual)
+
+
 def make_case(seed: int, m: int, n: int, k: int, bits: int, group: int | None = None):
     """x ~ N(0,1) f16; q4: w ~ U{0..15}, S ~ U(0.005,0.02); q8: w ~ U{-127..127}, S ~ U(0.002,0.01)."""
     rng = np.random.default_rng(seed)

@@ -109,10 +109,21 @@ int mi355x_wq_select_kernel(const mi355x_wq_desc* desc, int64_t m) {
   return wq::select_kernel(desc, m);
 }
 
-int mi355x_wq_matmul_ex(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
-                        void* y, int64_t m, void* stream, int kernel) {
+int mi355x_wq_matmul_fused_ex(const mi355x_wq_desc* desc, const void* x, const void* wq_,
+                              const void* scales, const mi355x_wq_epilogue* ep, void* y, int64_t m,
+                              void* stream, int kernel) {
   using namespace wq;
   if (!check_desc(desc, m)) return -1;
+  if (ep != nullptr) {
+    if (ep->reserved != 0) {
+      set_error("epilogue.reserved must be 0, got %d", ep->reserved);
+      return -1;
+    }
+    if (ep->activation != MI355X_WQ_ACT_NONE && ep->activation != MI355X_WQ_ACT_RELU) {
+      set_error("unknown epilogue activation %d", ep->activation);
+      return -1;
+    }
+  }
   if (m == 0 || desc->n == 0) return 0;  // empty output
   if (desc->k == 0) {
     set_error("K = 0 is not supported (the output would be all zeros)");
@@ -121,9 +132,16 @@ int mi355x_wq_matmul_ex(const mi355x_wq_desc* desc, const void* x, const void* w
   if (!check_ptr(x, "x", 16) || !check_ptr(wq_, "wq", 16) || !check_ptr(scales, "scales", 2) ||
       !check_ptr(y, "y", 2))
     return -1;
+  if (ep != nullptr && ep->bias != nullptr && !check_ptr(ep->bias, "bias", 2)) return -1;
+  if (ep != nullptr && ep->residual != nullptr && !check_ptr(ep->residual, "residual", 2)) return -1;
   const int family = kernel & 0xFF, variant = (kernel >> 8) & 0xFF;
   Problem p{x, wq_, scales, y, m, desc->n, desc->k, desc->bits, desc->group, desc->zero_point,
             static_cast<hipStream_t>(stream)};
+  if (ep != nullptr) {
+    p.bias = ep->bias;
+    p.residual = ep->residual;
+    p.activation = ep->activation;
+  }
   int chosen = family == MI355X_WQ_KERNEL_AUTO ? select_kernel(desc, m) : family;
   switch (chosen) {
     case MI355X_WQ_KERNEL_GEMV: return launch_gemv(p, variant);
@@ -133,9 +151,20 @@ int mi355x_wq_matmul_ex(const mi355x_wq_desc* desc, const void* x, const void* w
   }
 }
 
+int mi355x_wq_matmul_fused(const mi355x_wq_desc* desc, const void* x, const void* wq_,
+                           const void* scales, const mi355x_wq_epilogue* ep, void* y, int64_t m,
+                           void* stream) {
+  return mi355x_wq_matmul_fused_ex(desc, x, wq_, scales, ep, y, m, stream, MI355X_WQ_KERNEL_AUTO);
+}
+
+int mi355x_wq_matmul_ex(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
+                        void* y, int64_t m, void* stream, int kernel) {
+  return mi355x_wq_matmul_fused_ex(desc, x, wq_, scales, nullptr, y, m, stream, kernel);
+}
+
 int mi355x_wq_matmul(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
                      void* y, int64_t m, void* stream) {
-  return mi355x_wq_matmul_ex(desc, x, wq_, scales, y, m, stream, MI355X_WQ_KERNEL_AUTO);
+  return mi355x_wq_matmul_fused_ex(desc, x, wq_, scales, nullptr, y, m, stream, MI355X_WQ_KERNEL_AUTO);
 }
 
 int mi355x_wq_dequantize(const mi355x_wq_desc* desc, const void* wq_, const void* scales, void* wd,

@@ -124,4 +124,22 @@ __device__ __forceinline__ half8_t pack_h8(half2_t a, half2_t b, half2_t c, half
   return half8_t{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 }
 
+// Operations fused behind the float16 cast of the accumulator, in the order the composite
+// applies them: bias add, activation, residual add -- each a single float16 operation with
+// one rounding, as the CPU path executes them on float16 tensors.
+struct Epilogue {
+  const half_t* bias;      // [N], or nullptr
+  const half_t* residual;  // [M,N], or nullptr; may be the output buffer itself
+  int activation;          // 0 none, 1 relu
+};
+
+__device__ __forceinline__ void store_out(const Epilogue& ep, half_t* y, int m, int n, int N, float acc) {
+  half_t h = (half_t)acc;
+  const size_t idx = (size_t)m * N + n;
+  if (ep.bias != nullptr) h = h + ep.bias[n];
+  if (ep.activation == 1) h = h > (half_t)0 ? h : (half_t)0;  // max(h, 0) as select(h > 0, h, 0)
+  if (ep.residual != nullptr) h = h + ep.residual[idx];
+  y[idx] = h;
+}
+
 }  // namespace wq

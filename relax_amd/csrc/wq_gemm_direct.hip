@@ -66,8 +66,8 @@ struct RawB {
 template <int BITS, int GROUPS>
 __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
-    half_t* __restrict__ y, int M, int N, int K, int group_shift, int zero_point, int tiles_m,
-    int tiles_n) {
+    half_t* y, int M, int N, int K, int group_shift, int zero_point, int tiles_m, int tiles_n,
+    const Epilogue ep) {
   constexpr int BK = 64, TM = 4, WAVES = 4;
   constexpr int BM = TM * 32;
   constexpr int NT = WAVES * 64;   // threads of one K group
@@ -394,7 +394,7 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int m = m0 + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
-        if (m < M && n < N) y[(size_t)m * N + n] = (half_t)acc[i][j][v];
+        if (m < M && n < N) store_out(ep, y, m, n, N, acc[i][j][v]);
       }
     }
 }
@@ -416,7 +416,7 @@ void launch_direct(const Problem& p, int group_shift) {
   hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
-                     tiles_n);
+                     tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
 }
 
 }  // namespace

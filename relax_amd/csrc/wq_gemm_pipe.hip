@@ -56,8 +56,8 @@ struct GemmStage {
 template <int BITS, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM * WN * 64, 1) void wq_gemm_pipe_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
-    half_t* __restrict__ y, int M, int N, int K, int group_shift, int zero_point, int tiles_m,
-    int tiles_n) {
+    half_t* y, int M, int N, int K, int group_shift, int zero_point, int tiles_m, int tiles_n,
+    const Epilogue ep) {
   constexpr int BK = 64;
   constexpr int NT = WM * WN * 64;
   constexpr int CH = 128 / BITS;          // k per 16-byte packed chunk: 32 / 16
@@ -275,7 +275,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void wq_gemm_pipe_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int m = m0 + wm * (BM / WM) + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
-        if (m < M && n < N) y[(size_t)m * N + n] = (half_t)acc[i][j][v];
+        if (m < M && n < N) store_out(ep, y, m, n, N, acc[i][j][v]);
       }
     }
 }
@@ -298,7 +298,7 @@ void launch_pipe(const Problem& p, int group_shift) {
   hipLaunchKernelGGL((wq_gemm_pipe_kernel<BITS, BM, BN, WM, WN>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
-                     tiles_n);
+                     tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
 }
 
 }  // namespace

@@ -53,6 +53,7 @@ struct GemvArgs {
   int tiles;         // ceil(N / 16)
   int max_tiles;     // tiles per workgroup, upper bound (slot array extent)
   int phase_chunks;  // chunks per K phase (multiple of 4*D)
+  Epilogue ep;
 };
 
 template <int BITS, int WAVES, int D, int SPL>
@@ -251,7 +252,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(const GemvArgs a) {
       float sum = 0.f;
 #pragma unroll
       for (int w = 0; w < WAVES; ++w) sum += slots[((size_t)(i * WAVES + w) * 4 + r) * 64 + l];
-      a.y[(size_t)m * N + n] = (half_t)sum;
+      store_out(a.ep, a.y, m, n, N, sum);
     }
   }
 }
@@ -324,6 +325,7 @@ void launch_one(const Problem& p, int group_shift, const Plan& plan) {
   a.tiles = (int)((p.n + 15) / 16);
   a.max_tiles = plan.max_tiles;
   a.phase_chunks = plan.phase_chunks;
+  a.ep = Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation};
   static bool attr_set = false;  // idempotent; a race only repeats the same call
   if (!attr_set) {
     (void)hipFuncSetAttribute((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL>,

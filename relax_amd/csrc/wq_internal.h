@@ -13,6 +13,10 @@ struct Problem {
   int64_t m, n, k;
   int bits, group, zero_point;
   hipStream_t stream;
+  // fused epilogue (all optional): y = f16add(act(f16add(f16(acc), bias[n])), residual[m,n])
+  const void* bias = nullptr;
+  const void* residual = nullptr;
+  int activation = 0;  // 0 none, 1 relu
 };
 
 // Tuning variant: 0 = library default for the shape, >0 = explicit choice

@@ -32,8 +32,10 @@ constexpr Dtype kF16{2, 16, "float16"};
 constexpr Dtype kU32{1, 32, "uint32"};
 
 // Checks one tensor argument; on success stores the (byte_offset adjusted) pointer.
+// `vector_ok`: the tensor may be 1-d [N] (reported as rows = 1, cols = N).
 bool take_tensor(mi355x_tvm_value* args, int* type_codes, int idx, const char* role, Dtype want,
-                 int device_id_expected, const mi355x_dl_tensor** out, void** ptr) {
+                 int device_id_expected, const mi355x_dl_tensor** out, void** ptr,
+                 bool vector_ok = false, int64_t* rows = nullptr, int64_t* cols = nullptr) {
   const int tc = type_codes[idx];
   if (tc != MI355X_TVM_DLTENSOR_HANDLE && tc != MI355X_TVM_NDARRAY_HANDLE) {
     wq::set_error("argument %d (%s): expected a tensor (type code 7 or 13), got type code %d", idx,
@@ -44,6 +46,29 @@ bool take_tensor(mi355x_tvm_value* args, int* type_codes, int idx, const char* r
   if (t == nullptr) {
     wq::set_error("argument %d (%s): NULL tensor handle", idx, role);
     return false;
+  }
+  if (vector_ok && t->ndim == 1 && t->shape != nullptr) {
+    if (t->dtype.code != want.code || t->dtype.bits != want.bits || t->dtype.lanes != 1) {
+      wq::set_error("argument %d (%s): expected dtype %s, got code=%d bits=%d lanes=%d", idx, role,
+                    want.name, t->dtype.code, t->dtype.bits, t->dtype.lanes);
+      return false;
+    }
+    if (t->device.device_type != MI355X_DL_ROCM ||
+        (device_id_expected >= 0 && t->device.device_id != device_id_expected)) {
+      wq::set_error("argument %d (%s): expected a ROCm tensor on device %d, got device type %d id %d",
+                    idx, role, device_id_expected, t->device.device_type, t->device.device_id);
+      return false;
+    }
+    if (t->shape[0] < 0 || (t->strides != nullptr && t->shape[0] > 1 && t->strides[0] != 1) ||
+        (t->data == nullptr && t->shape[0] != 0)) {
+      wq::set_error("argument %d (%s): a 1-d tensor must be compact with a data pointer", idx, role);
+      return false;
+    }
+    *out = t;
+    *ptr = static_cast<char*>(t->data) + t->byte_offset;
+    if (rows != nullptr) *rows = 1;
+    if (cols != nullptr) *cols = t->shape[0];
+    return true;
   }
   if (t->ndim != 2 || t->shape == nullptr) {
     wq::set_error("argument %d (%s): expected a 2-d tensor, got ndim=%d", idx, role, t->ndim);
@@ -85,6 +110,8 @@ bool take_tensor(mi355x_tvm_value* args, int* type_codes, int idx, const char* r
   }
   *out = t;
   *ptr = static_cast<char*>(t->data) + t->byte_offset;
+  if (rows != nullptr) *rows = t->shape[0];
+  if (cols != nullptr) *cols = t->shape[1];
   return true;
 }
 
@@ -106,7 +133,13 @@ int mi355x_wq_packed_call(const mi355x_wq_callspec* spec, mi355x_tvm_value* args
     wq::set_error("call spec: unknown op %d", spec->op);
     return fail();
   }
-  const int expect = is_matmul ? 4 : 3;
+  const bool has_bias = is_matmul && spec->arg_bias >= 0;
+  const bool has_res = is_matmul && spec->arg_residual >= 0;
+  if (!is_matmul && (spec->arg_bias >= 0 || spec->arg_residual >= 0 || spec->activation != 0)) {
+    wq::set_error("call spec: dequantize takes no fused operands");
+    return fail();
+  }
+  const int expect = (is_matmul ? 4 : 3) + (has_bias ? 1 : 0) + (has_res ? 1 : 0);
   if (num_args != expect || spec->num_args != expect) {
     wq::set_error("%s expects %d arguments, got %d", is_matmul ? "matmul" : "dequantize", expect,
                   num_args);
@@ -117,9 +150,13 @@ int mi355x_wq_packed_call(const mi355x_wq_callspec* spec, mi355x_tvm_value* args
     return fail();
   }
   // role indices must be a permutation of 0..expect-1
-  int roles[4] = {spec->arg_wq, spec->arg_scales, spec->arg_out, spec->arg_x};
+  int roles[6] = {spec->arg_wq, spec->arg_scales, spec->arg_out, 0, 0, 0};
+  int nroles = 3;
+  if (is_matmul) roles[nroles++] = spec->arg_x;
+  if (has_bias) roles[nroles++] = spec->arg_bias;
+  if (has_res) roles[nroles++] = spec->arg_residual;
   unsigned seen = 0;
-  for (int i = 0; i < expect; ++i) {
+  for (int i = 0; i < nroles; ++i) {
     if (roles[i] < 0 || roles[i] >= expect || (seen & (1u << roles[i]))) {
       wq::set_error("call spec: argument roles are not a permutation of 0..%d", expect - 1);
       return fail();
@@ -181,6 +218,33 @@ int mi355x_wq_packed_call(const mi355x_wq_callspec* spec, mi355x_tvm_value* args
                   (long long)to->shape[1], (long long)d.n, (long long)d.k);
     return fail();
   }
+  mi355x_wq_epilogue ep;
+  memset(&ep, 0, sizeof(ep));
+  ep.activation = spec->activation;
+  if (has_bias) {
+    const mi355x_dl_tensor* tb = nullptr;
+    void* pb = nullptr;
+    int64_t br = 0, bc = 0;
+    if (!take_tensor(args, type_codes, spec->arg_bias, "bias", kF16, dev, &tb, &pb, true, &br, &bc))
+      return fail();
+    if (br != 1 || bc != d.n) {
+      wq::set_error("bias has shape (%lld, %lld), expected (%lld) or (1, %lld)", (long long)br,
+                    (long long)bc, (long long)d.n, (long long)d.n);
+      return fail();
+    }
+    ep.bias = pb;
+  }
+  if (has_res) {
+    const mi355x_dl_tensor* tr = nullptr;
+    void* pr = nullptr;
+    if (!take_tensor(args, type_codes, spec->arg_residual, "residual", kF16, dev, &tr, &pr)) return fail();
+    if (tr->shape[0] != m || tr->shape[1] != d.n) {
+      wq::set_error("residual has shape (%lld, %lld), expected (%lld, %lld)", (long long)tr->shape[0],
+                    (long long)tr->shape[1], (long long)m, (long long)d.n);
+      return fail();
+    }
+    ep.residual = pr;
+  }
   if (mi355x_wq_check(&d, m) != 0) return fail();
   if (d.n == 0 || (is_matmul && m == 0)) return 0;  // nothing to compute
 
@@ -194,21 +258,30 @@ int mi355x_wq_packed_call(const mi355x_wq_callspec* spec, mi355x_tvm_value* args
     wq::set_error("tensors live on ROCm device %d but the current HIP device is %d", dev, cur);
     return fail();
   }
-  const int rc = is_matmul ? mi355x_wq_matmul(&d, px, pw, ps, po, m, g_stream)
+  const int rc = is_matmul ? mi355x_wq_matmul_fused(&d, px, pw, ps, &ep, po, m, g_stream)
                            : mi355x_wq_dequantize(&d, pw, ps, po, g_stream);
   return rc == 0 ? 0 : fail();
 }
 
-#define MI355X_FIXED_ENTRY(NAME, OP, BITS, ZP)                                                    \
+// Fixed-name entries: arguments in the canonical order x, wq, scales, [bias | residual], out.
+#define MI355X_FIXED_ENTRY(NAME, OP, BITS, ZP, BIAS, RES, ACT)                                      \
   int NAME(mi355x_tvm_value* args, int* type_codes, int num_args, mi355x_tvm_value*, int*, void*) { \
-    static const mi355x_wq_callspec spec = {OP, BITS, 0, ZP, 0, (OP) == 0 ? 1 : 0, (OP) == 0 ? 2 : 1, \
-                                            (OP) == 0 ? 3 : 2, (OP) == 0 ? 4 : 3};                \
-    return mi355x_wq_packed_call(&spec, args, type_codes, num_args);                              \
+    static const mi355x_wq_callspec spec = {                                                        \
+        OP, BITS, 0, ZP, 0, (OP) == 0 ? 1 : 0, (OP) == 0 ? 2 : 1,                                   \
+        ((OP) == 0 ? 3 : 2) + (BIAS) + (RES), ((OP) == 0 ? 4 : 3) + (BIAS) + (RES),                 \
+        (BIAS) ? 3 : -1, (RES) ? 3 : -1, ACT};                                                      \
+    return mi355x_wq_packed_call(&spec, args, type_codes, num_args);                                \
   }
-MI355X_FIXED_ENTRY(mi355x_q4f16_matmul, 0, 4, 7)
-MI355X_FIXED_ENTRY(mi355x_q8f16_matmul, 0, 8, 0)
-MI355X_FIXED_ENTRY(mi355x_q4f16_dequantize, 1, 4, 7)
-MI355X_FIXED_ENTRY(mi355x_q8f16_dequantize, 1, 8, 0)
+MI355X_FIXED_ENTRY(mi355x_q4f16_matmul, 0, 4, 7, 0, 0, 0)
+MI355X_FIXED_ENTRY(mi355x_q8f16_matmul, 0, 8, 0, 0, 0, 0)
+MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_bias, 0, 4, 7, 1, 0, 0)
+MI355X_FIXED_ENTRY(mi355x_q8f16_matmul_bias, 0, 8, 0, 1, 0, 0)
+MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_bias_relu, 0, 4, 7, 1, 0, MI355X_WQ_ACT_RELU)
+MI355X_FIXED_ENTRY(mi355x_q8f16_matmul_bias_relu, 0, 8, 0, 1, 0, MI355X_WQ_ACT_RELU)
+MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_residual, 0, 4, 7, 0, 1, 0)
+MI355X_FIXED_ENTRY(mi355x_q8f16_matmul_residual, 0, 8, 0, 0, 1, 0)
+MI355X_FIXED_ENTRY(mi355x_q4f16_dequantize, 1, 4, 7, 0, 0, 0)
+MI355X_FIXED_ENTRY(mi355x_q8f16_dequantize, 1, 8, 0, 0, 0, 0)
 #undef MI355X_FIXED_ENTRY
 
 // ---- registration in TVM's global table through its C API -----------------------
@@ -238,6 +311,12 @@ int mi355x_wq_register_tvm_globals(int allow_override) {
   };
   const Entry entries[] = {{"mi355x.q4f16_matmul", mi355x_q4f16_matmul},
                            {"mi355x.q8f16_matmul", mi355x_q8f16_matmul},
+                           {"mi355x.q4f16_matmul_bias", mi355x_q4f16_matmul_bias},
+                           {"mi355x.q8f16_matmul_bias", mi355x_q8f16_matmul_bias},
+                           {"mi355x.q4f16_matmul_bias_relu", mi355x_q4f16_matmul_bias_relu},
+                           {"mi355x.q8f16_matmul_bias_relu", mi355x_q8f16_matmul_bias_relu},
+                           {"mi355x.q4f16_matmul_residual", mi355x_q4f16_matmul_residual},
+                           {"mi355x.q8f16_matmul_residual", mi355x_q8f16_matmul_residual},
                            {"mi355x.q4f16_dequantize", mi355x_q4f16_dequantize},
                            {"mi355x.q8f16_dequantize", mi355x_q8f16_dequantize}};
   int count = 0;

@@ -32,7 +32,7 @@ struct SkinnyBatch {
 template <int BITS, int R, int MT, int WAVES, int U>
 __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
-    half_t* __restrict__ y, int M, int N, int K, int group_shift, int zero_point) {
+    half_t* y, int M, int N, int K, int group_shift, int zero_point, const Epilogue ep) {
   constexpr int CH = 128 / BITS;  // k covered by one 16-byte lane load: 32 / 16
   constexpr int NJ = CH / 8;      // MFMAs fed by one lane load: 4 / 2
   const int lane = threadIdx.x & 63;
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
     const int r = t / MT, mt = t % MT;
     const int m = mt * 16 + 4 * (l >> 4) + i;
     const int n = (blockIdx.x * R + r) * 16 + (l & 15);
-    if (m < M && n < N) y[(size_t)m * N + n] = (half_t)sum;
+    if (m < M && n < N) store_out(ep, y, m, n, N, sum);
   }
 }
 
@@ -188,7 +188,8 @@ void launch_one(const Problem& p, int group_shift) {
   dim3 grid((tiles + R - 1) / R), block(WAVES * 64);
   hipLaunchKernelGGL((wq_skinny_kernel<BITS, R, MT, WAVES, U>), grid, block, 0, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
-                     (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point);
+                     (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point,
+                     Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
 }
 
 template <int BITS, int MT>

@@ -9,21 +9,33 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 SO_PATH = os.path.join(CSRC, "libmi355x_wq.so")
 
 KERNEL_AUTO, KERNEL_GEMV, KERNEL_GEMM, KERNEL_SKINNY = 0, 1, 2, 3
+ACT_NONE, ACT_RELU = 0, 1
+ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "relax.nn.relu": ACT_RELU}
 
 # every symbol include/mi355x_wq.h and include/mi355x_wq_packed.h declare
 EXPORTED_SYMBOLS = (
-    "mi355x_wq_matmul", "mi355x_wq_matmul_ex", "mi355x_wq_dequantize", "mi355x_wq_check",
+    "mi355x_wq_matmul", "mi355x_wq_matmul_ex", "mi355x_wq_matmul_fused", "mi355x_wq_matmul_fused_ex",
+    "mi355x_wq_dequantize", "mi355x_wq_check",
     "mi355x_wq_select_kernel", "mi355x_wq_last_error", "mi355x_wq_version",
-    "mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_dequantize",
+    "mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_matmul_bias", "mi355x_q8f16_matmul_bias",
+    "mi355x_q4f16_matmul_bias_relu", "mi355x_q8f16_matmul_bias_relu", "mi355x_q4f16_matmul_residual",
+    "mi355x_q8f16_matmul_residual", "mi355x_q4f16_dequantize",
     "mi355x_q8f16_dequantize", "mi355x_wq_packed_call", "mi355x_wq_packed_set_stream",
     "mi355x_wq_packed_get_stream", "mi355x_wq_register_tvm_globals",
 )
+PACKED_ENTRIES = tuple(s for s in EXPORTED_SYMBOLS if s.startswith(("mi355x_q4f16_", "mi355x_q8f16_")))
 
 
 class WqDesc(C.Structure):
     """mi355x_wq_desc"""
     _fields_ = [("bits", C.c_int32), ("group", C.c_int32), ("zero_point", C.c_int32),
                 ("reserved", C.c_int32), ("n", C.c_int64), ("k", C.c_int64)]
+
+
+class WqEpilogue(C.Structure):
+    """mi355x_wq_epilogue"""
+    _fields_ = [("bias", C.c_void_p), ("residual", C.c_void_p), ("activation", C.c_int32),
+                ("reserved", C.c_int32)]
 
 
 class WqError(RuntimeError):
@@ -57,6 +69,9 @@ def load() -> C.CDLL:
     dp = C.POINTER(WqDesc)
     L.mi355x_wq_matmul.argtypes = [dp, vp, vp, vp, vp, i64, vp]
     L.mi355x_wq_matmul_ex.argtypes = [dp, vp, vp, vp, vp, i64, vp, ci]
+    ep = C.POINTER(WqEpilogue)
+    L.mi355x_wq_matmul_fused.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp]
+    L.mi355x_wq_matmul_fused_ex.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp, ci]
     L.mi355x_wq_dequantize.argtypes = [dp, vp, vp, vp, vp]
     L.mi355x_wq_check.argtypes = [dp, i64]
     L.mi355x_wq_select_kernel.argtypes = [dp, i64]
@@ -64,8 +79,7 @@ def load() -> C.CDLL:
     L.mi355x_wq_packed_set_stream.argtypes = [vp]
     L.mi355x_wq_packed_get_stream.restype = vp
     L.mi355x_wq_register_tvm_globals.argtypes = [ci]
-    for name in ("mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_dequantize",
-                 "mi355x_q8f16_dequantize"):
+    for name in PACKED_ENTRIES:
         getattr(L, name).argtypes = [vp, C.POINTER(ci), ci, vp, C.POINTER(ci), vp]
     L.mi355x_wq_packed_call.argtypes = [vp, vp, C.POINTER(ci), ci]
     _lib = L

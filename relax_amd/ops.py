@@ -20,8 +20,12 @@ def _as_u32_storage(wq: torch.Tensor) -> torch.Tensor:
 
 def wq_matmul(x: torch.Tensor, wq: torch.Tensor, scales: torch.Tensor, bits: int, group: int,
               zero_point: int | None = None, out: torch.Tensor | None = None, kernel: int = 0,
-              variant: int = 0, stream=None) -> torch.Tensor:
-    """y[M,N] = f16(x[M,K] @ dequant(wq, scales)^T) on the current HIP device (asynchronous)."""
+              variant: int = 0, stream=None, bias: torch.Tensor | None = None,
+              activation: str | None = None, residual: torch.Tensor | None = None) -> torch.Tensor:
+    """y[M,N] = f16(x[M,K] @ dequant(wq, scales)^T) on the current HIP device (asynchronous).
+
+    Optional fused epilogue, each step one float16 operation: ``+ bias[N]``, then ``activation``
+    ("relu"), then ``+ residual[M,N]`` (``residual`` may be ``out`` itself)."""
     L = _lib.load()
     wq = _as_u32_storage(wq)
     if not (x.is_cuda and wq.is_cuda and scales.is_cuda):
@@ -41,8 +45,26 @@ def wq_matmul(x: torch.Tensor, wq: torch.Tensor, scales: torch.Tensor, bits: int
     elif tuple(out.shape) != (m, n) or out.dtype != torch.float16 or not out.is_contiguous():
         raise ValueError("out must be a compact float16 [M, N] tensor")
     desc = _lib.make_desc(bits, group, n, k, zero_point)
-    rc = L.mi355x_wq_matmul_ex(desc, x.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(),
-                               m, _stream_ptr(stream), kernel | (variant << 8))
+    if bias is None and residual is None and activation is None:
+        rc = L.mi355x_wq_matmul_ex(desc, x.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(),
+                                   m, _stream_ptr(stream), kernel | (variant << 8))
+        _lib.check(rc)
+        return out
+    if activation not in _lib.ACTIVATIONS:
+        raise ValueError(f"unsupported activation {activation!r}")
+    if bias is not None:
+        if not bias.is_cuda or bias.dtype != torch.float16 or not bias.is_contiguous() or \
+                tuple(bias.shape) not in ((n,), (1, n)):
+            raise ValueError(f"bias must be a compact float16 device tensor of shape ({n},) or (1, {n})")
+    if residual is not None:
+        if not residual.is_cuda or residual.dtype != torch.float16 or not residual.is_contiguous() or \
+                tuple(residual.shape) != (m, n):
+            raise ValueError(f"residual must be a compact float16 device tensor of shape ({m}, {n})")
+    ep = _lib.WqEpilogue(bias.data_ptr() if bias is not None else None,
+                         residual.data_ptr() if residual is not None else None,
+                         _lib.ACTIVATIONS[activation], 0)
+    rc = L.mi355x_wq_matmul_fused_ex(desc, x.data_ptr(), wq.data_ptr(), scales.data_ptr(), ep,
+                                     out.data_ptr(), m, _stream_ptr(stream), kernel | (variant << 8))
     _lib.check(rc)
     return out
 

@@ -7,6 +7,14 @@ The composite the backend takes over is the idiomatic weight-only-quantized line
     y32 = R.matmul(x, R.permute_dims(Wd), out_dtype="float32")
     y   = R.astype(y32, "float16")
 
+optionally followed by the element-wise tail the reference's `make_matmul_pattern(with_bias,
+activation)` describes for its CUTLASS backend (python/tvm/relax/dpl/pattern.py:1049-1095:
+`add`, then `relax.nn.relu`), and by the residual add of a decoder layer:
+
+    y = R.add(y, bias)            # bias [N] or [1, N]
+    y = R.nn.relu(y)
+    y = R.add(y, residual)        # residual [M, N]
+
 `matmul(x, permute_dims(W))` is what `relax.op.linear` expands to
 (python/tvm/relax/op/linear_algebra.py:54-90).  The pattern name's prefix before the
 first "." becomes the `Codegen` attribute, i.e. the backend name
@@ -30,12 +38,25 @@ def patterns():
     """[(name, DFPattern)] for FuseOpsByPattern(patterns, annotate_codegen=True)."""
     from tvm.relax.dpl import is_call_tir, is_op, wildcard  # python/tvm/relax/dpl/pattern.py:678-837
 
-    table = []
-    for fn_name, q in DECODE_FUNCS.items():
+    def core(fn_name):
         decoded = is_call_tir(fn_name, [wildcard(), wildcard()])
         weight_t = is_op("relax.permute_dims")(decoded)
         mm = is_op("relax.matmul")(wildcard(), weight_t)
-        table.append((f"{BACKEND}.q{q['bits']}f16_matmul", is_op("relax.astype")(mm)))
+        return is_op("relax.astype")(mm)
+
+    # Longest tail first: earlier entries have priority (transform.py:337-339).  A pattern cannot
+    # tell a [N] bias from a [M, N] residual (no shape predicate without concrete extents); the
+    # codegen hook decides from the operand's shape and rejects what the epilogue cannot express.
+    table = []
+    for fn_name, q in DECODE_FUNCS.items():
+        base = f"{BACKEND}.q{q['bits']}f16_matmul"
+        add1 = lambda: is_op("relax.add")(core(fn_name), wildcard())  # noqa: E731
+        relu = lambda: is_op("relax.nn.relu")(add1())                 # noqa: E731
+        table.append((base + "_add_relu_add", is_op("relax.add")(relu(), wildcard())))
+        table.append((base + "_add_add", is_op("relax.add")(add1(), wildcard())))
+        table.append((base + "_add_relu", relu()))
+        table.append((base + "_add", add1()))
+        table.append((base, core(fn_name)))
     return table
 
 

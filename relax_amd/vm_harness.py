@@ -46,9 +46,17 @@ class TVMValue(C.Union):
 
 
 class CallSpec(C.Structure):
-    """mi355x_wq_callspec"""
+    """mi355x_wq_callspec; the fused-operand roles default to "absent" (-1)."""
     _fields_ = [(n, C.c_int32) for n in ("op", "bits", "group", "zero_point", "arg_x", "arg_wq",
-                                         "arg_scales", "arg_out", "num_args")]
+                                         "arg_scales", "arg_out", "num_args", "arg_bias",
+                                         "arg_residual", "activation")]
+
+    def __init__(self, *args, **kw):
+        if len(args) < 10:
+            kw.setdefault("arg_bias", -1)
+        if len(args) < 11:
+            kw.setdefault("arg_residual", -1)
+        super().__init__(*args, **kw)
 
 
 _DTYPES = {

@@ -23,8 +23,38 @@ CASES = [  # name, seed, M, N, K, bits, group
     ("q8f16_m66_n24_k384", 15, 66, 24, 384, 8, 128),
 ]
 
+FUSED_CASES = [  # name, seed, M, N, K, bits, group, bias?, activation, residual?
+    ("fused_q4f16_m4_n48_k128_bias_relu_res", 21, 4, 48, 128, 4, 32, True, "relu", True),
+    ("fused_q4f16_m1_n80_k256_res", 22, 1, 80, 256, 4, 32, False, None, True),
+    ("fused_q8f16_m70_n24_k256_bias", 23, 70, 24, 256, 8, 128, True, None, False),
+]
+
+
+def fused_operands(seed, m, n, with_bias, with_residual):
+    """bias ~ N(0, 0.5), residual ~ N(0, 1), float16, from their own seeded stream."""
+    rng = np.random.default_rng(1000 + seed)
+    bias = (0.5 * rng.standard_normal(n, dtype=np.float32)).astype(np.float16) if with_bias else None
+    res = rng.standard_normal((m, n), dtype=np.float32).astype(np.float16) if with_residual else None
+    return bias, res
+
+
 if __name__ == "__main__":
     here = os.path.dirname(os.path.abspath(__file__))
+    for name, seed, m, n, k, bits, group, wb, act, wr in FUSED_CASES:
+        x, wq, s, g = O.make_case(seed, m, n, k, bits, group)
+        bias, res = fused_operands(seed, m, n, wb, wr)
+        y = O.wq_matmul_fused(x, wq, s, bits, g, bias, act, res)
+        extra = {}
+        if bias is not None:
+            extra["bias"] = bias
+        if res is not None:
+            extra["residual"] = res
+        np.savez_compressed(os.path.join(here, name + ".npz"), x=x, wq=wq, scales=s, y=y,
+                            y_plain=O.wq_matmul(x, wq, s, bits, g), bits=np.int32(bits), group=np.int32(g),
+                            activation=np.array(act or "none"), **extra)
+        print(name, y.shape, float(np.abs(y).max()))
+    if "--fused-only" in sys.argv:
+        sys.exit(0)
     for name, seed, m, n, k, bits, group in CASES:
         x, wq, s, g = O.make_case(seed, m, n, k, bits, group)
         wd = O.dequant(wq, s, bits, g)

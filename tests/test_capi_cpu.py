@@ -27,7 +27,7 @@ def declared_symbols():
 def test_library_exports_every_declared_symbol():
     L = lib.load()
     names = declared_symbols()
-    assert len(names) == 15 and set(names) == set(lib.EXPORTED_SYMBOLS)
+    assert len(names) == 23 and set(names) == set(lib.EXPORTED_SYMBOLS)
     for n in names:
         assert hasattr(L, n), n
     assert L.mi355x_wq_version() >= 100
@@ -183,6 +183,64 @@ def test_generic_entry_checks_the_call_spec():
             vm_harness.call_packed(None, permuted, spec=spec)
 
 
+def test_fused_entries_check_their_extra_operand():
+    x, wq, s, y = _cpu_case()
+    dev = dict(device_type=10)
+    a = _args(x, wq, s, y, **dev)
+    bias = vm_harness.TensorArg(torch.zeros(16, dtype=torch.float16), **dev)
+    bias2d = vm_harness.TensorArg(torch.zeros((1, 16), dtype=torch.float16), **dev)
+    res = vm_harness.TensorArg(torch.zeros((2, 16), dtype=torch.float16), **dev)
+    for sym in ("mi355x_q4f16_matmul_bias", "mi355x_q4f16_matmul_bias_relu", "mi355x_q4f16_matmul_residual"):
+        with pytest.raises(vm_harness.PackedError, match="expects 5 arguments, got 4"):
+            vm_harness.call_packed(sym, a)
+    with pytest.raises(vm_harness.PackedError, match=r"bias has shape \(1, 8\), expected \(16\) or \(1, 16\)"):
+        vm_harness.call_packed("mi355x_q4f16_matmul_bias", a[:3] + [
+            vm_harness.TensorArg(torch.zeros(8, dtype=torch.float16), **dev), a[3]])
+    with pytest.raises(vm_harness.PackedError, match=r"bias has shape \(2, 16\)"):
+        vm_harness.call_packed("mi355x_q4f16_matmul_bias", a[:3] + [res, a[3]])
+    with pytest.raises(vm_harness.PackedError, match=r"argument 3 \(bias\): expected dtype float16"):
+        vm_harness.call_packed("mi355x_q4f16_matmul_bias_relu", a[:3] + [
+            vm_harness.TensorArg(torch.zeros(16, dtype=torch.float32), **dev), a[3]])
+    with pytest.raises(vm_harness.PackedError, match=r"residual has shape \(1, 16\), expected \(2, 16\)"):
+        vm_harness.call_packed("mi355x_q4f16_matmul_residual", a[:3] + [bias2d, a[3]])
+    with pytest.raises(vm_harness.PackedError, match=r"argument 3 \(residual\): expected a 2-d tensor"):
+        vm_harness.call_packed("mi355x_q4f16_matmul_residual", a[:3] + [bias, a[3]])
+    if not torch.cuda.is_available():  # every check passes; only the missing device stops the calls
+        for sym, extra in (("mi355x_q4f16_matmul_bias", bias), ("mi355x_q4f16_matmul_bias", bias2d),
+                           ("mi355x_q4f16_matmul_bias_relu", bias), ("mi355x_q4f16_matmul_residual", res)):
+            with pytest.raises(vm_harness.PackedError, match="no usable HIP device"):
+                vm_harness.call_packed(sym, a[:3] + [extra, a[3]])
+    # generic entry: bias and residual together, roles permuted; bad activation / roles rejected
+    spec = vm_harness.CallSpec(0, 4, 0, 7, 2, 0, 1, 5, 6, 3, 4, 1)
+    order = [a[1], a[2], a[0], bias, res, a[3]]
+    if not torch.cuda.is_available():
+        with pytest.raises(vm_harness.PackedError, match="no usable HIP device"):
+            vm_harness.call_packed(None, order, spec=spec)
+    with pytest.raises(vm_harness.PackedError, match="not a permutation"):
+        vm_harness.call_packed(None, order, spec=vm_harness.CallSpec(0, 4, 0, 7, 2, 0, 1, 5, 6, 3, 3, 0))
+    with pytest.raises(vm_harness.PackedError, match="dequantize takes no fused operands"):
+        vm_harness.call_packed(None, a[1:], spec=vm_harness.CallSpec(1, 4, 0, 7, 0, 0, 1, 2, 3, 1, -1, 0))
+
+
+def test_fused_c_entry_validates_the_epilogue():
+    L = lib.load()
+    d = lib.make_desc(4, 32, 16, 64)
+    ep = lib.WqEpilogue(None, None, 7, 0)
+    assert L.mi355x_wq_matmul_fused(d, 16, 16, 16, ep, 16, 2, None) == -1
+    assert "unknown epilogue activation 7" in lib.last_error()
+    ep = lib.WqEpilogue(None, None, 0, 1)
+    assert L.mi355x_wq_matmul_fused(d, 16, 16, 16, ep, 16, 2, None) == -1
+    assert "epilogue.reserved must be 0" in lib.last_error()
+    ep = lib.WqEpilogue(3, None, 1, 0)  # odd bias pointer
+    assert L.mi355x_wq_matmul_fused(d, 16, 16, 16, ep, 16, 2, None) == -1
+    assert "bias" in lib.last_error() and "aligned" in lib.last_error()
+    ep = lib.WqEpilogue(None, 5, 0, 0)
+    assert L.mi355x_wq_matmul_fused(d, 16, 16, 16, ep, 16, 2, None) == -1
+    assert "residual" in lib.last_error() and "aligned" in lib.last_error()
+    # an empty output is a no-op whatever the epilogue
+    assert L.mi355x_wq_matmul_fused(d, None, None, None, lib.WqEpilogue(None, None, 1, 0), None, 0, None) == 0
+
+
 def test_stream_setter_round_trip():
     L = lib.load()
     L.mi355x_wq_packed_set_stream(0x1230)
@@ -202,13 +260,12 @@ assert L.mi355x_wq_register_tvm_globals(0) == -1 and "no TVM runtime" in lib.las
 fake = C.CDLL({fake!r}, mode=C.RTLD_GLOBAL)
 fake.fake_tvm_name.restype = C.c_char_p
 fake.fake_tvm_last_error.restype = C.c_char_p
-assert L.mi355x_wq_register_tvm_globals(0) == 4
+assert L.mi355x_wq_register_tvm_globals(0) == 10
 names = sorted(fake.fake_tvm_name(i).decode() for i in range(fake.fake_tvm_count()))
-assert names == ["mi355x.q4f16_dequantize", "mi355x.q4f16_matmul", "mi355x.q8f16_dequantize",
-                 "mi355x.q8f16_matmul"], names
+assert names == sorted("mi355x." + s[len("mi355x_"):] for s in lib.PACKED_ENTRIES), names
 # call a registered function the way the registry would, with host tensors: it must fail and the
 # message must arrive in the host's last-error slot (what LOG(FATAL) << TVMGetLastError() prints)
-idx = [fake.fake_tvm_name(i).decode() for i in range(4)].index("mi355x.q4f16_matmul")
+idx = [fake.fake_tvm_name(i).decode() for i in range(10)].index("mi355x.q4f16_matmul")
 x = torch.zeros((1, 64), dtype=torch.float16); wq = torch.zeros((16, 8), dtype=torch.int32)
 s = torch.zeros((16, 2), dtype=torch.float16); y = torch.zeros((1, 16), dtype=torch.float16)
 ta = [vm_harness.TensorArg(x), vm_harness.TensorArg(wq, as_uint32=True), vm_harness.TensorArg(s),

@@ -9,12 +9,16 @@ from oracle import c_oracle, wq_oracle as O
 FILES = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
 
 
+PLAIN = [f for f in FILES if not os.path.basename(f).startswith("fused_")]
+FUSED = [f for f in FILES if os.path.basename(f).startswith("fused_")]
+
+
 def test_fixtures_exist():
-    assert len(FILES) >= 5
+    assert len(PLAIN) >= 5 and len(FUSED) >= 3
 
 
 def test_fixtures_match_both_oracles():
-    for f in FILES:
+    for f in PLAIN:
         z = np.load(f)
         bits, g = int(z["bits"]), int(z["group"])
         for impl in (O, c_oracle):
@@ -22,6 +26,43 @@ def test_fixtures_match_both_oracles():
             y = impl.wq_matmul(z["x"], z["wq"], z["scales"], bits, g)
             assert np.array_equal(wd.view(np.uint16), z["wd"].view(np.uint16)), f
             assert np.array_equal(y.view(np.uint16), z["y"].view(np.uint16)), f
+
+
+def fused_operands(z):
+    act = str(z["activation"])
+    return (z["bias"] if "bias" in z.files else None, None if act == "none" else act,
+            z["residual"] if "residual" in z.files else None)
+
+
+def test_fused_fixtures_match_both_oracles():
+    for f in FUSED:
+        z = np.load(f)
+        bits, g = int(z["bits"]), int(z["group"])
+        bias, act, res = fused_operands(z)
+        for impl in (O, c_oracle):
+            y = impl.wq_matmul_fused(z["x"], z["wq"], z["scales"], bits, g, bias, act, res)
+            assert np.array_equal(y.view(np.uint16), z["y"].view(np.uint16)), f
+            assert np.array_equal(impl.epilogue(z["y_plain"], bias, act, res).view(np.uint16),
+                                  z["y"].view(np.uint16)), f
+
+
+def test_fused_fixture_by_hand():
+    """One element of the bias + relu + residual fixture, recomputed with Python fractions."""
+    from fractions import Fraction
+
+    z = np.load([f for f in FUSED if "bias_relu_res" in f][0])
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16)
+    finite = halves[np.isfinite(halves)]
+
+    def nearest(fr):  # round-to-nearest-even among all finite float16 values, by exhaustive search
+        best = min(finite, key=lambda h: (abs(Fraction(float(h)) - fr), int(h.view(np.uint16)) & 1))
+        return best
+
+    for (m, n) in [(0, 0), (3, 47), (2, 17)]:
+        t = nearest(Fraction(float(z["y_plain"][m, n])) + Fraction(float(z["bias"][n])))
+        t = t if t > 0 else np.float16(0)
+        want = nearest(Fraction(float(t)) + Fraction(float(z["residual"][m, n])))
+        assert want.view(np.uint16) == z["y"][m, n].view(np.uint16)
 
 
 def test_fixture_known_fields():

@@ -122,3 +122,106 @@ def test_config5_decoder_layer_chain(m):
     err = np.abs(got.astype(np.float64) - want.astype(np.float64))
     assert np.all(np.isfinite(got)) and np.all(err <= 4 * (ATOL + RTOL * np.abs(want.astype(np.float64)))), float(err.max())
     assert float(np.mean(err)) < 2e-3
+
+
+def test_fused_fixed_name_entries_called_vm_style():
+    """matmul_bias / matmul_bias_relu / matmul_residual as DPS externs: same bits as the tensor front end."""
+    import relax_amd
+    from relax_amd import vm_harness
+
+    vm_harness.set_stream()
+    for bits, m, n, k in [(4, 1, 4096, 4096), (4, 40, 136, 256), (8, 300, 520, 1024)]:
+        x, wq, s, g = O.make_case(31, m, n, k, bits)
+        rng = np.random.default_rng(m)
+        bias = rng.standard_normal(n).astype(np.float16)
+        res = rng.standard_normal((m, n)).astype(np.float16)
+        xd, wd, sd, bd, rd = _dev(x), _dev(wq), _dev(s), _dev(bias), _dev(res)
+        for sym, extra, kw in (("matmul_bias", bd, dict(bias=bd)),
+                               ("matmul_bias", bd.reshape(1, n), dict(bias=bd)),
+                               ("matmul_bias_relu", bd, dict(bias=bd, activation="relu")),
+                               ("matmul_residual", rd, dict(residual=rd))):
+            y = vm_harness.call_dps("mi355x_q%df16_%s" % (bits, sym), [xd, wd, sd, extra], (m, n))
+            ref = relax_amd.wq_matmul(xd, wd, sd, bits, g, **kw)
+            torch.cuda.synchronize()
+            assert np.array_equal(y.cpu().numpy().view(np.uint16), ref.cpu().numpy().view(np.uint16)), (sym, bits, m)
+        want = c_oracle.wq_matmul_fused(x, wq, s, bits, g, bias, "relu", None, nthreads=16)
+        got = relax_amd.wq_matmul(xd, wd, sd, bits, g, bias=bd, activation="relu").cpu().numpy()
+        err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+        assert np.all(err <= 2 * ATOL + RTOL * np.abs(want.astype(np.float64)))
+
+
+def test_generated_entry_with_bias_relu_and_residual(tmp_path):
+    import relax_amd
+    from relax_amd import vm_harness
+    from relax_amd.tvm_glue import CallSpec
+    from tests.test_tvm_glue_cpu import build_entries, call_entry
+
+    L = build_entries(tmp_path, [("fused_tail_mi355x", CallSpec(0, 4, 0, 7, 2, 0, 1, 5, 3, 4, 1))])
+    vm_harness.set_stream()
+    m, n, k = 8, 4096, 4096
+    x, wq, s, g = O.make_case(33, m, n, k, 4)
+    rng = np.random.default_rng(3)
+    bias, res = rng.standard_normal(n).astype(np.float16), rng.standard_normal((m, n)).astype(np.float16)
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    xd, wd, sd, bd, rd = _dev(x), _dev(wq), _dev(s), _dev(bias), _dev(res)
+    t = [vm_harness.TensorArg(wd, as_uint32=True), vm_harness.TensorArg(sd), vm_harness.TensorArg(xd),
+         vm_harness.TensorArg(bd), vm_harness.TensorArg(rd), vm_harness.TensorArg(y)]
+    rc, code = call_entry(L, "fused_tail_mi355x", t)
+    torch.cuda.synchronize()
+    assert rc == 0 and code == vm_harness.K_TVM_NULLPTR
+    ref = relax_amd.wq_matmul(xd, wd, sd, 4, g, bias=bd, activation="relu", residual=rd)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy().view(np.uint16), ref.cpu().numpy().view(np.uint16))
+
+
+@pytest.mark.parametrize("m", [4, 1024])
+def test_decoder_layer_chain_with_fused_residuals(m):
+    """The layer chain with the two residual adds fused into the O and down projections:
+        a   = stand-in(qkv) / 1024;   h   = x + a Wo^T        (residual fused)
+        z   = stand-in(gu)  / 32;     out = h + z Wd^T        (residual fused)
+    Bit-equal to the same chain with separate float16 adds on the GPU, and within tolerance of the
+    oracle on a sample of rows."""
+    import relax_amd
+
+    shapes = {"qkv": (12288, 4096), "o": (4096, 4096), "gu": (22016, 4096), "down": (4096, 11008)}
+    rng = np.random.default_rng(56)
+    x = (rng.standard_normal((m, 4096)) * 0.5).astype(np.float16)
+    W = {}
+    for i, (name, (n, k)) in enumerate(shapes.items()):
+        _, wq, s, g = O.make_case(70 + i, 1, n, k, 4)
+        W[name] = (wq, s)
+
+    def layer(xh, matmul, f16):
+        qkv = matmul(xh, "qkv", None)
+        a = f16(f16(f16(qkv[:, :4096] * f16(0.5)) + f16(qkv[:, 4096:8192] * f16(0.25))) + f16(qkv[:, 8192:] * f16(0.25)))
+        a = f16(a * f16(1 / 1024))
+        h = matmul(a, "o", xh)
+        gu = matmul(h, "gu", None)
+        z = f16(f16(gu[:, :11008] * f16(1 / 32)) * f16(gu[:, 11008:] * f16(1 / 32)))
+        z = f16(z * f16(1 / 32))
+        return matmul(z, "down", h)
+
+    dW = {k: (_dev(v[0]), _dev(v[1])) for k, v in W.items()}
+    tf16 = lambda v: v if torch.is_tensor(v) else torch.tensor(v, dtype=torch.float16, device="cuda")  # noqa: E731
+
+    def gpu_fused(t, name, res):
+        return relax_amd.wq_matmul(t.contiguous(), dW[name][0], dW[name][1], 4, 32, residual=res)
+
+    def gpu_separate(t, name, res):
+        y = relax_amd.wq_matmul(t.contiguous(), dW[name][0], dW[name][1], 4, 32)
+        return y if res is None else y + res
+
+    fused = layer(_dev(x), gpu_fused, tf16)
+    separate = layer(_dev(x), gpu_separate, tf16)
+    torch.cuda.synchronize()
+    assert np.array_equal(fused.cpu().numpy().view(np.uint16), separate.cpu().numpy().view(np.uint16))
+    rows = np.arange(m) if m <= 4 else np.random.default_rng(5).choice(m, size=4, replace=False)
+
+    def cpu_matmul(t, name, res):
+        return c_oracle.wq_matmul_fused(np.ascontiguousarray(t), W[name][0], W[name][1], 4, 32,
+                                        residual=None if res is None else np.ascontiguousarray(res), nthreads=16)
+
+    want = layer(x[rows], cpu_matmul, lambda v: np.asarray(v, dtype=np.float16))
+    got = fused.cpu().numpy()[rows]
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    assert np.all(np.isfinite(got)) and np.all(err <= 4 * (ATOL + RTOL * np.abs(want.astype(np.float64)))), float(err.max())

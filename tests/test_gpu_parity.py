@@ -294,7 +294,8 @@ def test_golden_fixtures():
     import glob
     import os
 
-    files = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
+    files = sorted(f for f in glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz"))
+                   if not os.path.basename(f).startswith("fused_"))
     assert files, "no golden fixtures found"
     import relax_amd
 
@@ -305,3 +306,143 @@ def test_golden_fixtures():
         assert_close(got, z["y"], f)
         wd = relax_amd.wq_dequantize(_dev(z["wq"]), _dev(z["scales"]), bits, g).cpu().numpy()
         assert np.array_equal(wd.view(np.uint16), z["wd"].view(np.uint16)), f
+
+
+# ------------------------------------------------------------------ fused tail: bias, relu, residual
+def _fused_operands(seed, m, n):
+    rng = np.random.default_rng(seed)
+    return ((0.5 * rng.standard_normal(n)).astype(np.float16), rng.standard_normal((m, n)).astype(np.float16))
+
+
+def run_fused(x, wq, s, bits, group, bias=None, activation=None, residual=None, kernel=0, variant=0, out=None):
+    import relax_amd
+
+    y = relax_amd.wq_matmul(_dev(x), _dev(wq), _dev(s), bits, group, kernel=kernel, variant=variant,
+                            bias=None if bias is None else _dev(bias), activation=activation,
+                            residual=None if residual is None else _dev(residual), out=out)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def assert_fused(got, got_plain, want_plain, bias, act, res, what):
+    """The fused output must be (a) bit for bit the float16 tail applied to the same kernel's plain
+    output, and (b) within the matmul tolerance -- taken on the value before the tail, where
+    cancellation has not yet shrunk the reference -- of the oracle's fused result."""
+    tail_of_plain = O.epilogue(got_plain, bias, act, res)
+    assert np.array_equal(got.view(np.uint16), tail_of_plain.view(np.uint16)), what
+    want = O.epilogue(want_plain, bias, act, res).astype(np.float64)
+    err = np.abs(got.astype(np.float64) - want)
+    pre = np.abs(want_plain.astype(np.float64)) + (0 if bias is None else np.abs(bias.astype(np.float64))[None, :])
+    bound = ATOL + RTOL * pre + 2.0**-10 * np.abs(want)
+    assert np.all(np.isfinite(got)) and np.all(err <= bound), (what, float(err.max()))
+
+
+FUSED_SHAPES = [  # bits, M, N, K -> kernel family under AUTO dispatch
+    (4, 1, 200, 1024), (4, 8, 96, 352), (8, 16, 40, 256),       # GEMV
+    (4, 33, 72, 256), (8, 64, 48, 384),                          # skinny
+    (4, 300, 520, 512), (8, 129, 260, 1024), (4, 2048, 256, 768),  # GEMM, direct-weight kernel
+    (4, 200, 96, 320), (4, 70, 32, 96),                          # GEMM, pipelined / generic fallbacks
+]
+
+
+@pytest.mark.parametrize("tail", ["bias", "bias_relu", "residual", "bias_relu_residual", "bias_residual"])
+@pytest.mark.parametrize("bits,m,n,k", FUSED_SHAPES)
+def test_fused_tail_every_kernel_family(bits, m, n, k, tail):
+    x, wq, s, g = O.make_case(700 + m + n, m, n, k, bits)
+    b, r = _fused_operands(m * 7 + n, m, n)
+    bias = b if "bias" in tail else None
+    res = r if "residual" in tail else None
+    act = "relu" if "relu" in tail else None
+    got_plain = run_matmul(x, wq, s, bits, g)
+    got = run_fused(x, wq, s, bits, g, bias, act, res)
+    want_plain = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
+    assert_fused(got, got_plain, want_plain, bias, act, res, (tail, bits, m, n, k))
+    if act:
+        assert got.min() >= 0 if res is None else True
+
+
+@pytest.mark.parametrize("kernel,variant,bits,m,n,k", [
+    ("GEMV", 14, 4, 3, 40, 352), ("GEMV", 25, 4, 1, 64, 1024), ("GEMV", 11, 8, 16, 24, 128),
+    ("SKINNY", 1, 4, 20, 40, 256), ("SKINNY", 6, 8, 48, 24, 256),
+    ("GEMM", 1, 4, 70, 136, 448), ("GEMM", 4, 8, 129, 72, 256), ("GEMM", 11, 4, 300, 200, 128),
+    ("GEMM", 13, 8, 513, 260, 1024), ("GEMM", 21, 4, 129, 520, 1280), ("GEMM", 22, 8, 65, 300, 1792),
+])
+def test_fused_tail_explicit_kernel_variants(kernel, variant, bits, m, n, k):
+    from relax_amd import lib
+
+    fam = getattr(lib, "KERNEL_" + kernel)
+    x, wq, s, g = O.make_case(800 + m + n, m, n, k, bits)
+    bias, res = _fused_operands(m + 3 * n, m, n)
+    got_plain = run_matmul(x, wq, s, bits, g, kernel=fam, variant=variant)
+    got = run_fused(x, wq, s, bits, g, bias, "relu", res, kernel=fam, variant=variant)
+    want_plain = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
+    assert_fused(got, got_plain, want_plain, bias, "relu", res, (kernel, variant, bits, m, n, k))
+
+
+@pytest.mark.parametrize("bits,m,n,k", [(4, 1, 4096, 4096), (4, 8, 200, 1024), (4, 40, 72, 256), (4, 256, 512, 512)])
+def test_fused_residual_in_place(bits, m, n, k):
+    """h += x W^T: the residual is the output buffer itself (each element is read, then written,
+    by the one thread that owns it)."""
+    import relax_amd
+
+    x, wq, s, g = O.make_case(900 + m, m, n, k, bits)
+    _, res = _fused_operands(m + n, m, n)
+    separate = run_fused(x, wq, s, bits, g, residual=res)
+    h = _dev(res.copy())
+    out = relax_amd.wq_matmul(_dev(x), _dev(wq), _dev(s), bits, g, residual=h, out=h)
+    torch.cuda.synchronize()
+    assert out.data_ptr() == h.data_ptr()
+    assert np.array_equal(h.cpu().numpy().view(np.uint16), separate.view(np.uint16))
+
+
+def test_fused_special_values_follow_the_cpu_rules():
+    """relu(-0) = +0, an overflowing bias add gives inf, inf + (-inf) residual gives NaN."""
+    m, n, k = 2, 32, 64
+    w = np.full((n, k), 7, dtype=np.int64)          # dequantizes to 0: the matmul result is +0 everywhere
+    w[:, 0] = 8                                     # ... except x[:, 0] * scale
+    wq = O.pack_q4(w)
+    s = np.full((n, k // 32), 1.0, dtype=np.float16)
+    x = np.zeros((m, k), dtype=np.float16)
+    x[0, 0], x[1, 0] = -0.0, 60000.0                # row 0: -0 * 1 = -0 accumulates to +0 (sum starts at +0)
+    bias = np.zeros(n, dtype=np.float16)
+    bias[0], bias[1], bias[2] = -0.0, 60000.0, -1.0
+    res = np.zeros((m, n), dtype=np.float16)
+    res[1, 3] = -np.inf
+    got = run_fused(x, wq, s, 4, 32, bias, "relu", res)
+    want = c_oracle.wq_matmul_fused(x, wq, s, 4, 32, bias, "relu", res)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+    assert got[0, 0].view(np.uint16) == 0 and np.isinf(got[1, 1]) and got[0, 2] == 0 and got[1, 3] == -np.inf
+
+
+def test_fused_golden_fixtures():
+    import glob
+    import os
+
+    from tests.test_golden_cpu import fused_operands
+
+    files = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "fused_*.npz")))
+    assert len(files) >= 3
+    for f in files:
+        z = np.load(f)
+        bits, g = int(z["bits"]), int(z["group"])
+        bias, act, res = fused_operands(z)
+        got_plain = run_matmul(z["x"], z["wq"], z["scales"], bits, g)
+        got = run_fused(z["x"], z["wq"], z["scales"], bits, g, bias, act, res)
+        assert_fused(got, got_plain, z["y_plain"], bias, act, res, f)
+
+
+def test_fused_argument_checks():
+    import relax_amd
+
+    x, wq, s, g = O.make_case(1, 2, 32, 64, 4)
+    xd, wd, sd = _dev(x), _dev(wq), _dev(s)
+    with pytest.raises(ValueError, match="unsupported activation"):
+        relax_amd.wq_matmul(xd, wd, sd, 4, g, activation="gelu")
+    with pytest.raises(ValueError, match="bias must be"):
+        relax_amd.wq_matmul(xd, wd, sd, 4, g, bias=torch.zeros(31, dtype=torch.float16, device="cuda"))
+    with pytest.raises(ValueError, match="residual must be"):
+        relax_amd.wq_matmul(xd, wd, sd, 4, g, residual=torch.zeros((1, 32), dtype=torch.float16, device="cuda"))
+    with pytest.raises(ValueError, match="bias must be"):
+        relax_amd.wq_matmul(xd, wd, sd, 4, g, bias=torch.zeros(32, dtype=torch.float32, device="cuda"))

@@ -219,3 +219,134 @@ def test_make_case_distributions():
     w = O.unpack_q8(wq)
     assert g == 128 and w.min() == -127 and w.max() == 127
     assert 0.00199 <= float(s.min()) and float(s.max()) <= 0.01001
+
+
+# ------------------------------------------------------------------ fused tail: float16 add, relu
+def _f16(bits):
+    return np.array(bits, dtype=np.uint16).view(np.float16)
+
+
+def _add_both(a, b):
+    """a + b through both restatements (the C one via its epilogue with a as y and b as bias)."""
+    a = np.asarray(a, dtype=np.float16).reshape(1, -1)
+    b = np.asarray(b, dtype=np.float16).reshape(-1)
+    got_np = O.add_f16(a, b.reshape(1, -1))
+    got_c = c_oracle.epilogue(a, bias=b)
+    return got_np.reshape(-1), got_c.reshape(-1)
+
+
+def test_f16_add_known_answers():
+    """Ties go to even, sums past 65504 + 16 overflow, signed zeros and infinities follow IEEE 754."""
+    cases = [
+        (2048.0, 1.0, 2048.0),            # tie: 2049 lies between 2048 (even) and 2050
+        (2048.0, 3.0, 2052.0),            # tie: 2051 -> 2052 (even significand)
+        (1.0, 2.0**-11, 1.0),             # half an ulp above 1: tie to even
+        (1.0, 3 * 2.0**-11, 1.0 + 2.0**-9),
+        (1.0, 2.0**-11 + 2.0**-21, 1.0 + 2.0**-10),   # the next float16 above 2^-11: just past the tie
+        (65504.0, 8.0, 65504.0),
+        (65504.0, 16.0, np.inf),          # tie at 65520 rounds to the even neighbour 2^16 = overflow
+        (-65504.0, -16.0, -np.inf),
+        (6.0e-8, 6.0e-8, 1.2e-7),         # subnormal + subnormal is exact (both are 2^-24)
+        (1024.0, -1023.5, 0.5),           # exact cancellation
+        (0.1, 0.2, 0.2998046875),         # f16(0.1) + f16(0.2) = 0.29998779296875 -> 0.2998046875
+    ]
+    a = np.array([c[0] for c in cases], dtype=np.float16)
+    b = np.array([c[1] for c in cases], dtype=np.float16)
+    want = np.array([c[2] for c in cases], dtype=np.float16)
+    for got in _add_both(a, b):
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), (got, want)
+    # signed zeros: (+0) + (-0) = +0, (-0) + (-0) = -0, x + (-x) = +0; inf - inf is NaN
+    a = _f16([0x0000, 0x8000, 0x3C00, 0x7C00])
+    b = _f16([0x8000, 0x8000, 0xBC00, 0xFC00])
+    for got in _add_both(a, b):
+        assert list(got.view(np.uint16)[:3]) == [0x0000, 0x8000, 0x0000] and np.isnan(got[3])
+
+
+def test_f16_add_against_exact_rationals():
+    """Independent check of the rounding: exact sums as fractions, nearest-even by search in the
+    sorted table of all finite float16 values (no floating-point arithmetic on the checking side)."""
+    import bisect
+    from fractions import Fraction
+
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16)
+    finite = halves[np.isfinite(halves) & ~((halves == 0) & np.signbit(halves))]  # drop -0: one zero in the table
+    order = np.argsort(finite.astype(np.float64), kind="stable")
+    table = finite[order]
+    fracs = [Fraction(float(h)) for h in table]
+    big = Fraction(65520)  # halfway between 65504 and 2^16
+
+    def nearest(fr):
+        if fr >= big:
+            return np.float16(np.inf)
+        if fr <= -big:
+            return np.float16(-np.inf)
+        i = bisect.bisect_left(fracs, fr)
+        cands = [j for j in (i - 1, i) if 0 <= j < len(fracs)]
+        dist = [abs(fracs[j] - fr) for j in cands]
+        if len(cands) == 2 and dist[0] == dist[1]:
+            j = cands[0] if (int(table[cands[0]].view(np.uint16)) & 1) == 0 else cands[1]
+        else:
+            j = cands[int(np.argmin(dist))]
+        return table[j]
+
+    rng = np.random.default_rng(42)
+    bits_a = rng.integers(0, 65536, size=3000).astype(np.uint16)
+    bits_b = rng.integers(0, 65536, size=3000).astype(np.uint16)
+    # add pairs with nearby exponents (where rounding ties actually occur) and opposite signs
+    near = rng.integers(0x3000, 0x4800, size=3000).astype(np.uint16)
+    bits_a = np.concatenate([bits_a, near, near])
+    bits_b = np.concatenate([bits_b, near + rng.integers(0, 64, size=3000).astype(np.uint16),
+                             (near ^ 0x8000) + rng.integers(0, 3, size=3000).astype(np.uint16)])
+    a, b = bits_a.view(np.float16), bits_b.view(np.float16)
+    ok = np.isfinite(a) & np.isfinite(b)
+    a, b = a[ok], b[ok]
+    got_np, got_c = _add_both(a, b)
+    for i in range(a.size):
+        exact = Fraction(float(a[i])) + Fraction(float(b[i]))
+        want = nearest(exact)
+        if exact == 0:
+            assert got_np[i] == 0 and got_c[i] == 0
+            continue
+        assert got_np[i].view(np.uint16) == want.view(np.uint16), (a[i], b[i])
+        assert got_c[i].view(np.uint16) == want.view(np.uint16), (a[i], b[i])
+
+
+def test_relu_special_values_and_epilogue_order():
+    t = _f16([0x8000, 0x0000, 0x0001, 0x8001, 0x7C00, 0xFC00, 0x7E00, 0xFE00, 0x3C00, 0xBC00])
+    want = [0x0000, 0x0000, 0x0001, 0x0000, 0x7C00, 0x0000, 0x0000, 0x0000, 0x3C00, 0x0000]
+    assert list(O.relu_f16(t).view(np.uint16)) == want
+    assert list(c_oracle.epilogue(t.reshape(1, -1), activation="relu").view(np.uint16).reshape(-1)) == want
+    # order: bias before relu, residual after: y = -1, bias = +0.5 -> relu(-0.5) = 0 -> + residual 2 = 2;
+    # any other order gives 1.5 (relu last on -1+0.5+2) or 2.5 (relu first)
+    y = np.array([[-1.0]], dtype=np.float16)
+    for impl in (O, c_oracle):
+        out = impl.epilogue(y, bias=np.array([0.5], dtype=np.float16), activation="relu",
+                            residual=np.array([[2.0]], dtype=np.float16))
+        assert float(out[0, 0]) == 2.0
+    # bias broadcasts over rows, residual is element-wise
+    y = np.zeros((2, 3), dtype=np.float16)
+    b = np.array([1, 2, 3], dtype=np.float16)
+    r = np.array([[10, 20, 30], [40, 50, 60]], dtype=np.float16)
+    for impl in (O, c_oracle):
+        assert np.array_equal(impl.epilogue(y, bias=b, residual=r), r + b[None, :])
+    with pytest.raises(ValueError):
+        O.epilogue(y, activation="gelu")
+
+
+@pytest.mark.parametrize("bits,m,n,k", [(4, 3, 40, 128), (8, 5, 24, 256)])
+def test_fused_path_is_epilogue_of_plain_path(bits, m, n, k):
+    x, wq, s, g = O.make_case(8, m, n, k, bits)
+    rng = np.random.default_rng(3)
+    bias = rng.standard_normal(n).astype(np.float16)
+    res = rng.standard_normal((m, n)).astype(np.float16)
+    plain = O.wq_matmul(x, wq, s, bits, g)
+    for act in (None, "relu"):
+        a = O.wq_matmul_fused(x, wq, s, bits, g, bias, act, res)
+        c = c_oracle.wq_matmul_fused(x, wq, s, bits, g, bias, act, res)
+        assert np.array_equal(a.view(np.uint16), c.view(np.uint16))
+        t = plain.astype(np.float64) + bias.astype(np.float64)[None, :]
+        t = t.astype(np.float16)
+        if act:
+            t = np.maximum(t, np.float16(0))
+        want = (t.astype(np.float64) + res.astype(np.float64)).astype(np.float16)
+        assert np.array_equal(a.view(np.uint16), want.view(np.uint16))

@@ -103,3 +103,83 @@ def test_quantize_helpers_round_trip():
     assert np.abs(O.dequant_q8f16(wq, s).astype(np.float32) - w).max() <= 0.51 * float(s.max()) + 1e-3
     with pytest.raises(ValueError):
         pack_q4(np.full((1, 8), 16))
+
+
+# ---------------------------------------------------------------- role derivation on a stand-in IR
+@pytest.fixture
+def fake_tvm(monkeypatch):
+    import sys
+
+    from tests.support import fake_relax
+
+    tvm, relax = fake_relax.as_module()
+    monkeypatch.setitem(sys.modules, "tvm", tvm)
+    monkeypatch.setitem(sys.modules, "tvm.relax", relax)
+    return fake_relax
+
+
+def test_roles_of_plain_and_fused_composites(fake_tvm):
+    from relax_amd.tvm_glue.codegen import ACT_NONE, ACT_RELU, spec_from_function
+
+    m, n = 4, 48
+    s = spec_from_function(fake_tvm.quantized_linear())
+    assert (s.arg_wq, s.arg_scales, s.arg_x, s.arg_out, s.num_args) == (0, 1, 2, 3, 4)
+    assert (s.arg_bias, s.arg_residual, s.activation, s.bits, s.zero_point) == (-1, -1, ACT_NONE, 4, 7)
+    s = spec_from_function(fake_tvm.quantized_linear("decode_q8f16", tail=[("add", [n])]))
+    assert (s.bits, s.zero_point, s.arg_bias, s.arg_residual, s.arg_out, s.num_args) == (8, 0, 3, -1, 4, 5)
+    s = spec_from_function(fake_tvm.quantized_linear(tail=[("add", [1, n]), ("relu",)]))
+    assert (s.arg_bias, s.arg_residual, s.activation) == (3, -1, ACT_RELU)
+    s = spec_from_function(fake_tvm.quantized_linear(tail=[("add", [m, n])]))
+    assert (s.arg_bias, s.arg_residual, s.activation, s.arg_out) == (-1, 3, ACT_NONE, 4)
+    # add(residual, y): the operand order of the add does not matter
+    s = spec_from_function(fake_tvm.quantized_linear(tail=[("add", [m, n], True)]))
+    assert (s.arg_bias, s.arg_residual) == (-1, 3)
+    s = spec_from_function(fake_tvm.quantized_linear(tail=[("add", [n]), ("relu",), ("add", [m, n])]))
+    assert (s.arg_bias, s.arg_residual, s.activation, s.arg_out, s.num_args) == (3, 4, ACT_RELU, 5, 6)
+    s.validate()
+    # outer parameters in another order: roles follow the call arguments, not the positions
+    s = spec_from_function(fake_tvm.quantized_linear(tail=[("add", [n])], outer_order=[2, 3, 0, 1]))
+    assert (s.arg_x, s.arg_bias, s.arg_wq, s.arg_scales, s.arg_out) == (0, 1, 2, 3, 4)
+
+
+def test_role_derivation_rejects_tails_the_epilogue_cannot_express(fake_tvm):
+    from relax_amd.tvm_glue.codegen import spec_from_function
+
+    m, n = 4, 48
+    with pytest.raises(ValueError, match="in this order"):  # relu after a [M,N] add
+        spec_from_function(fake_tvm.quantized_linear(tail=[("add", [m, n]), ("add", [m, n])]))
+    with pytest.raises(ValueError, match="only fused between"):
+        spec_from_function(fake_tvm.quantized_linear(tail=[("add", [m, n]), ("relu",)]))
+    with pytest.raises(ValueError, match="only fused between"):
+        spec_from_function(fake_tvm.quantized_linear(tail=[("relu",), ("relu",)]))
+    f = fake_tvm.quantized_linear()
+    f.body.blocks[0].bindings[0].value.attrs["Composite"] = "cutlass.matmul"
+    with pytest.raises(ValueError, match="does not belong to backend"):
+        spec_from_function(f)
+
+
+def test_generated_fused_entry_forwards_all_roles(tmp_path):
+    # (wq, scales, x, bias, residual, y) with relu between the adds
+    spec = CallSpec(0, 4, 0, 7, 2, 0, 1, 5, 3, 4, 1)
+    L = build_entries(tmp_path, [("fused_tail_mi355x", spec)])
+    dev = dict(device_type=10)
+    x = torch.zeros((2, 64), dtype=torch.float16)
+    wq = torch.zeros((16, 8), dtype=torch.int32)
+    s = torch.zeros((16, 2), dtype=torch.float16)
+    y = torch.zeros((2, 16), dtype=torch.float16)
+    bias = torch.zeros(16, dtype=torch.float16)
+    res = torch.zeros((2, 16), dtype=torch.float16)
+    t = [vm_harness.TensorArg(wq, as_uint32=True, **dev), vm_harness.TensorArg(s, **dev),
+         vm_harness.TensorArg(x, **dev), vm_harness.TensorArg(bias, **dev),
+         vm_harness.TensorArg(res, **dev), vm_harness.TensorArg(y, **dev)]
+    rc, _ = call_entry(L, "fused_tail_mi355x", [t[0], t[1], t[2], t[4], t[3], t[5]])  # bias and residual swapped
+    assert rc == -1 and "bias has shape (2, 16)" in lib.last_error()
+    rc, _ = call_entry(L, "fused_tail_mi355x", t[:5])
+    assert rc == -1 and "expects 6 arguments, got 5" in lib.last_error()
+    if not torch.cuda.is_available():
+        rc, _ = call_entry(L, "fused_tail_mi355x", t)
+        assert rc == -1 and "no usable HIP device" in lib.last_error()
+    with pytest.raises(ValueError, match="activation"):
+        trampoline_source([("f", CallSpec(0, 4, 0, 7, 0, 1, 2, 3, -1, -1, 9))])
+    with pytest.raises(ValueError, match="no fused operands"):
+        trampoline_source([("f", CallSpec(1, 4, 0, 7, 0, 0, 1, 3, 2, -1, 0))])
