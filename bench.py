@@ -85,6 +85,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=N_LAYERS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
+    ap.add_argument("--no-epilogue", action="store_true", help="skip the fused-residual leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times (a kernel of known HBM "
                          "traffic, used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
@@ -188,10 +189,11 @@ def main() -> int:
 
         flops = sum(2 * PREFILL_M * n * k for _, n, k in LLAMA7B) * len(use)
         with torch.cuda.stream(stream):
-            prefill_pass()
+            for _ in range(1 + min(args.warmup, 3)):
+                prefill_pass()
             torch.cuda.synchronize()
             g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            reps = max(2, args.steps // 4)
+            reps = max(2, args.steps // 2)
             g0.record(stream)
             for _ in range(reps):
                 prefill_pass()
@@ -217,7 +219,8 @@ def main() -> int:
                     torch.matmul(xg[k], wd.t(), out=yg[n])
 
         with torch.cuda.stream(stream):
-            library_pass()
+            for _ in range(1 + min(args.warmup, 3)):
+                library_pass()
             torch.cuda.synchronize()
             g0.record(stream)
             for _ in range(reps):
@@ -229,6 +232,47 @@ def main() -> int:
         result["gemm"]["library_f16_gemm_note"] = ("torch.matmul (hipBLASLt) on float16 weights dequantized "
                                                    "beforehand, same shapes and data")
         del wds
+
+    # ---- fused residual add: O and down projections of every layer, batch 1 and 8 -------------
+    # h = h + x W^T as one launch against the matmul followed by a separate float16 add kernel.
+    if not args.no_epilogue:
+        hs = {m: torch.randn((m, 4096), device=dev).to(torch.float16) for m in DECODE_BATCHES}
+        tmp = {m: torch.empty((m, 4096), dtype=torch.float16, device=dev) for m in DECODE_BATCHES}
+
+        def residual_pass(fused):
+            for m in DECODE_BATCHES:
+                for mats in layers:
+                    for wq, s, n, k in (mats[1], mats[3]):  # O (4096x4096) and down (4096x11008)
+                        if fused:
+                            relax_amd.wq_matmul(xs[(m, k)], wq, s, 4, 32, residual=hs[m], out=hs[m])
+                        else:
+                            relax_amd.wq_matmul(xs[(m, k)], wq, s, 4, 32, out=tmp[m])
+                            hs[m].add_(tmp[m])
+
+        times = {}
+        with torch.cuda.stream(stream):
+            for fused in (False, True):
+                residual_pass(fused)
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=stream):
+                    residual_pass(fused)
+                gr.replay()
+                torch.cuda.synchronize()
+                r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                r0.record(stream)
+                for _ in range(args.steps):
+                    gr.replay()
+                r1.record(stream)
+                torch.cuda.synchronize()
+                times[fused] = r0.elapsed_time(r1) / args.steps
+        pairs = len(DECODE_BATCHES) * args.layers * 2
+        result["epilogue"] = {
+            "workload": "O and down projections of %d layers at batch 1 and 8, each followed by the "
+                        "residual add h += y (one HIP graph)" % args.layers,
+            "us_per_projection_separate_add": round(times[False] * 1e3 / pairs, 3),
+            "us_per_projection_fused": round(times[True] * 1e3 / pairs, 3),
+            "speedup": round(times[False] / times[True], 3)}
 
     if not args.no_cpu:
         one, omp = cpu_baseline(quick=False)
