@@ -87,7 +87,13 @@ bool check_ptr(const void* p, const char* name, size_t align) {
 
 int select_kernel(const mi355x_wq_desc* d, int64_t m) {
   Problem p{nullptr, nullptr, nullptr, nullptr, m, d->n, d->k, d->bits, d->group, d->zero_point, nullptr};
-  if (gemv_applicable(p)) return MI355X_WQ_KERNEL_GEMV;
+  if (gemv_applicable(p)) {
+    // The GEMV kernel stages the activations in LDS.  Measured on MI355X: once they
+    // are large (more than 64 KB, one workgroup per CU) and there is at most one row tile per CU
+    // to amortise the staging, the register-activation kernel is faster.
+    const int64_t x_bytes = m * d->k * 2, tiles = (d->n + 15) / 16;
+    if (!(x_bytes > 64 * 1024 && tiles <= 256)) return MI355X_WQ_KERNEL_GEMV;
+  }
   return m <= kSkinnyMaxM ? MI355X_WQ_KERNEL_SKINNY : MI355X_WQ_KERNEL_GEMM;
 }
 

@@ -204,7 +204,14 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(const GemvArgs a) {
       __builtin_amdgcn_sched_barrier(0);
       x_store(tid, x0);
       x_store(tid + NT, x1);
-      for (int idx = tid + 2 * NT; idx < total; idx += NT) x_store(idx, x_load(idx));
+      // the rest four vectors at a time: all four requests are in flight before the first store
+      for (int idx = tid + 2 * NT; idx < total; idx += 4 * NT) {
+        const u32x4 v0 = x_load(idx), v1 = x_load(idx + NT), v2 = x_load(idx + 2 * NT), v3 = x_load(idx + 3 * NT);
+        x_store(idx, v0);
+        x_store(idx + NT, v1);
+        x_store(idx + 2 * NT, v2);
+        x_store(idx + 3 * NT, v3);
+      }
     }
     __syncthreads();
 

@@ -224,7 +224,17 @@ int launch_skinny(const Problem& p, int variant) {
     return -1;
   }
   const int mt = (int)((p.m + 15) / 16);
-  if (variant == 0) variant = mt >= 3 ? 1 : 2;
+  if (variant == 0) {
+    // Measured on MI355X (q4f16, Llama-2-7B shapes, M = 4 .. 64): the number of workgroups is what
+    // matters.  At most one row tile per CU: one tile per 4-wave workgroup; a few more: two
+    // tiles per workgroup (a second, mostly empty round of workgroups costs more); more: four
+    // tiles per workgroup; many: two tiles per 8-wave workgroup for one row block, else four.
+    const int64_t tiles = (p.n + 15) / 16;
+    if (tiles <= 256) variant = 1;
+    else if (tiles <= 384) variant = mt >= 3 ? 1 : 2;
+    else if (tiles <= 1024) variant = 7;
+    else variant = mt == 1 ? 5 : (mt == 2 ? 7 : 9);
+  }
   bool ok;
   if (p.bits == 4) {
     ok = mt <= 1   ? dispatch_variant<4, 1>(p, group_shift, variant)
