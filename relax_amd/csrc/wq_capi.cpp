@@ -19,6 +19,43 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+int current_device_slot() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return dev >= 0 && dev < kMaxDevices ? dev : kMaxDevices - 1;
+}
+
+bool ensure_dynamic_lds(const void* kernel, int bytes, bool* done) {
+  const int slot = current_device_slot();
+  if (done[slot]) return true;  // a race only repeats the same idempotent call
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    set_error("cannot reserve %d bytes of LDS for a kernel on this device: %s", bytes, hipGetErrorString(e));
+    return false;
+  }
+  done[slot] = true;
+  return true;
+}
+
+int cu_count() {
+  static int cached[kMaxDevices] = {0};  // same value for every caller of a device
+  const int slot = current_device_slot();
+  if (cached[slot] == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+        prop.multiProcessorCount > 0)
+      cached[slot] = prop.multiProcessorCount;
+    else
+      return 256;
+  }
+  return cached[slot];
+}
+
 namespace {
 
 constexpr int64_t kMaxBufferBytes = 0x7FFFFFF0ll;  // kernels address buffers with 32-bit offsets

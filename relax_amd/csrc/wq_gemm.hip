@@ -185,21 +185,18 @@ __global__ __launch_bounds__(WM * WN * 64) void wq_gemm_kernel(
 namespace {
 
 template <int BITS, int BM, int BN, int WM, int WN>
-void launch_one(const Problem& p, int group_shift) {
+bool launch_one(const Problem& p, int group_shift) {
   const int tiles_m = (int)((p.m + BM - 1) / BM);
   const int tiles_n = (int)((p.n + BN - 1) / BN);
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * (64 + 8) * sizeof(half_t);
-  static bool attr_set = false;  // idempotent; a race only repeats the same call
-  if (!attr_set) {
-    (void)hipFuncSetAttribute((const void*)wq_gemm_kernel<BITS, BM, BN, WM, WN>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    attr_set = true;
-  }
+  static bool lds_ok[kMaxDevices] = {false};
+  if (!ensure_dynamic_lds((const void*)wq_gemm_kernel<BITS, BM, BN, WM, WN>, (int)lds_bytes, lds_ok)) return false;
   hipLaunchKernelGGL((wq_gemm_kernel<BITS, BM, BN, WM, WN>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
                      tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
+  return true;
 }
 
 }  // namespace
@@ -237,10 +234,11 @@ int launch_gemm(const Problem& p, int variant) {
     variant = -1;
   }
   if (variant == 0) variant = 1;
+  bool launched = true;
 #define WQ_GEMM_CASE(ID, BM, BN, WM, WN)                                  \
   case ID:                                                                \
-    if (p.bits == 4) launch_one<4, BM, BN, WM, WN>(p, group_shift);       \
-    else launch_one<8, BM, BN, WM, WN>(p, group_shift);                   \
+    launched = p.bits == 4 ? launch_one<4, BM, BN, WM, WN>(p, group_shift) \
+                           : launch_one<8, BM, BN, WM, WN>(p, group_shift); \
     break;
   switch (variant) {
     case -1: break;  // already launched above
@@ -255,6 +253,7 @@ int launch_gemm(const Problem& p, int variant) {
       return -1;
   }
 #undef WQ_GEMM_CASE
+  if (!launched) return -1;  // the error is already set
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("gemm kernel launch failed: %s", hipGetErrorString(e));

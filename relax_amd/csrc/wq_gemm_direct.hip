@@ -402,21 +402,19 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
 namespace {
 
 template <int BITS, int GROUPS>
-void launch_direct(const Problem& p, int group_shift) {
+bool launch_direct(const Problem& p, int group_shift) {
   constexpr int BM = 128, BN = 256;
   const int tiles_m = (int)((p.m + BM - 1) / BM);
   const int tiles_n = (int)((p.n + BN - 1) / BN);
   dim3 grid(tiles_m * tiles_n), block(GROUPS * 256);
   constexpr size_t lds_bytes = (size_t)GROUPS * 4 * BM * 128;  // four activation stages per K group
-  static const bool attr_set = [] {
-    return hipFuncSetAttribute((const void*)wq_gemm_direct_kernel<BITS, GROUPS>,
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) == hipSuccess;
-  }();
-  (void)attr_set;
+  static bool lds_ok[kMaxDevices] = {false};
+  if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS>, (int)lds_bytes, lds_ok)) return false;
   hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
                      tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
+  return true;
 }
 
 }  // namespace
@@ -429,14 +427,10 @@ bool launch_gemm_direct(const Problem& p, int group_shift, int variant) {
   if (p.k % 256 != 0 || p.group != (p.bits == 4 ? 32 : 128)) return false;
   switch (variant) {
     case 1:
-      if (p.bits == 4) launch_direct<4, 1>(p, group_shift);
-      else launch_direct<8, 1>(p, group_shift);
-      return true;
+      return p.bits == 4 ? launch_direct<4, 1>(p, group_shift) : launch_direct<8, 1>(p, group_shift);
     case 2:
       if (p.k < 512) return false;
-      if (p.bits == 4) launch_direct<4, 2>(p, group_shift);
-      else launch_direct<8, 2>(p, group_shift);
-      return true;
+      return p.bits == 4 ? launch_direct<4, 2>(p, group_shift) : launch_direct<8, 2>(p, group_shift);
     default: return false;
   }
 }

@@ -283,22 +283,19 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void wq_gemm_pipe_kernel(
 namespace {
 
 template <int BITS, int BM, int BN, int WM, int WN>
-void launch_pipe(const Problem& p, int group_shift) {
+bool launch_pipe(const Problem& p, int group_shift) {
   const int tiles_m = (int)((p.m + BM - 1) / BM);
   const int tiles_n = (int)((p.n + BN - 1) / BN);
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   constexpr size_t lds_bytes = 3 * (size_t)(BM + BN) * 128;
   static_assert(lds_bytes <= 160 * 1024, "three stages must fit the 160 KB LDS");
-  static bool attr_set = false;  // idempotent; a race only repeats the same call
-  if (!attr_set) {
-    (void)hipFuncSetAttribute((const void*)wq_gemm_pipe_kernel<BITS, BM, BN, WM, WN>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    attr_set = true;
-  }
+  static bool lds_ok[kMaxDevices] = {false};
+  if (!ensure_dynamic_lds((const void*)wq_gemm_pipe_kernel<BITS, BM, BN, WM, WN>, (int)lds_bytes, lds_ok)) return false;
   hipLaunchKernelGGL((wq_gemm_pipe_kernel<BITS, BM, BN, WM, WN>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
                      tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
+  return true;
 }
 
 }  // namespace
@@ -313,9 +310,8 @@ bool launch_gemm_pipe(const Problem& p, int group_shift, int variant) {
   if (!gemm_pipe_applicable(p)) return false;
 #define WQ_PIPE_CASE(ID, BM, BN, WM, WN)                             \
   case ID:                                                           \
-    if (p.bits == 4) launch_pipe<4, BM, BN, WM, WN>(p, group_shift); \
-    else launch_pipe<8, BM, BN, WM, WN>(p, group_shift);             \
-    return true;
+    return p.bits == 4 ? launch_pipe<4, BM, BN, WM, WN>(p, group_shift) \
+                       : launch_pipe<8, BM, BN, WM, WN>(p, group_shift);
   switch (variant) {
     WQ_PIPE_CASE(1, 256, 128, 2, 2)
     WQ_PIPE_CASE(2, 128, 128, 2, 2)

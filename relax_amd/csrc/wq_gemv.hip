@@ -274,20 +274,6 @@ struct Plan {
   size_t lds_bytes;
 };
 
-int cu_count() {
-  static int cached = 0;  // same value for every caller; a race only repeats the query
-  if (cached == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-        prop.multiProcessorCount > 0)
-      cached = prop.multiProcessorCount;
-    else
-      return 256;
-  }
-  return cached;
-}
-
 // Chooses the grid (workgroups per CU), the tiles per workgroup and the K phase so
 // that partial-tile slots + staged activations fit in LDS.
 template <int BITS, int WAVES, int D>
@@ -316,8 +302,12 @@ bool make_plan(const Problem& p, int wgs_per_cu, Plan* out) {
   return out->lds_bytes <= budget;
 }
 
+// Launch results of the helpers below: the variant does not fit the problem (try another),
+// the kernel was launched, or a runtime call failed (error already set).
+enum { kNotApplicable = 0, kLaunched = 1, kFailed = -1 };
+
 template <int BITS, int WAVES, int D, int SPL>
-void launch_one(const Problem& p, int group_shift, const Plan& plan) {
+int launch_one(const Problem& p, int group_shift, const Plan& plan) {
   GemvArgs a;
   a.x = (const half_t*)p.x;
   a.wq = (const uint32_t*)p.wq;
@@ -333,40 +323,32 @@ void launch_one(const Problem& p, int group_shift, const Plan& plan) {
   a.max_tiles = plan.max_tiles;
   a.phase_chunks = plan.phase_chunks;
   a.ep = Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation};
-  static bool attr_set = false;  // idempotent; a race only repeats the same call
-  if (!attr_set) {
-    (void)hipFuncSetAttribute((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWgMax);
-    attr_set = true;
-  }
+  static bool lds_ok[kMaxDevices] = {false};
+  if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL>, (int)kLdsPerWgMax, lds_ok))
+    return kFailed;
   hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL>), dim3(plan.grid), dim3(WAVES * 64),
                      plan.lds_bytes, p.stream, a);
+  return kLaunched;
 }
 
 // D chunks per lane need K to be a multiple of 4*D chunks, and the lane's D
 // chunks to share one scale (SPL = 1) or to have one each (SPL = D).
 template <int BITS, int WAVES, int D>
-bool try_launch(const Problem& p, int group_shift, int wgs_per_cu) {
+int try_launch(const Problem& p, int group_shift, int wgs_per_cu) {
   constexpr int ch = 128 / BITS;
-  if (D > 1 && p.k % (4 * D * ch) != 0) return false;
+  if (D > 1 && p.k % (4 * D * ch) != 0) return kNotApplicable;
   Plan plan;
-  if (!make_plan<BITS, WAVES, D>(p, wgs_per_cu, &plan)) return false;
-  if (group_shift == 0) {
-    launch_one<BITS, WAVES, D, D>(p, group_shift, plan);
-    return true;
-  }
-  if ((1 << group_shift) >= D) {
-    launch_one<BITS, WAVES, D, 1>(p, group_shift, plan);
-    return true;
-  }
-  return false;
+  if (!make_plan<BITS, WAVES, D>(p, wgs_per_cu, &plan)) return kNotApplicable;
+  if (group_shift == 0) return launch_one<BITS, WAVES, D, D>(p, group_shift, plan);
+  if ((1 << group_shift) >= D) return launch_one<BITS, WAVES, D, 1>(p, group_shift, plan);
+  return kNotApplicable;
 }
 
 // variant = 10 * workgroups-per-CU + shape index
 template <int BITS>
-bool dispatch(const Problem& p, int gs, int variant) {
+int dispatch(const Problem& p, int gs, int variant) {
   const int wpc = variant / 10, shape = variant % 10;
-  if (wpc < 1 || wpc > 8) return false;
+  if (wpc < 1 || wpc > 8) return kNotApplicable;
   switch (shape) {
     case 1: return try_launch<BITS, 4, 1>(p, gs, wpc);
     case 2: return try_launch<BITS, 4, 2>(p, gs, wpc);
@@ -376,7 +358,7 @@ bool dispatch(const Problem& p, int gs, int variant) {
     case 6: return try_launch<BITS, 8, 4>(p, gs, wpc);
     case 7: return try_launch<BITS, 16, 1>(p, gs, wpc);
     case 8: return try_launch<BITS, 16, 2>(p, gs, wpc);
-    default: return false;
+    default: return kNotApplicable;
   }
 }
 
@@ -396,7 +378,7 @@ int launch_gemv(const Problem& p, int variant) {
     set_error("gemv kernel: M=%lld is outside 1..16", (long long)p.m);
     return -1;
   }
-  bool ok = false;
+  int ok = kNotApplicable;
   if (variant == 0) {
     // Measured on MI355X (Llama-2-7B shapes): up to 4 rows run best with two 8-wave
     // workgroups per CU, larger batches (more LDS per workgroup) with one.  Two-chunk
@@ -406,12 +388,13 @@ int launch_gemv(const Problem& p, int variant) {
     for (int q = 0; q < 4; ++q) {
       const int v = order[q];
       ok = p.bits == 4 ? dispatch<4>(p, gs, v) : dispatch<8>(p, gs, v);
-      if (ok) break;
+      if (ok != kNotApplicable) break;
     }
   } else {
     ok = p.bits == 4 ? dispatch<4>(p, gs, variant) : dispatch<8>(p, gs, variant);
   }
-  if (!ok) {
+  if (ok == kFailed) return -1;
+  if (ok == kNotApplicable) {
     set_error("gemv kernel: variant %d does not apply to M=%lld K=%lld group=%d", variant,
               (long long)p.m, (long long)p.k, p.group);
     return -1;

@@ -35,4 +35,16 @@ constexpr int64_t kSkinnyMaxM = 64;
 
 void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 
+// Index of the current HIP device, clamped to the size of the per-device caches below.
+constexpr int kMaxDevices = 64;
+int current_device_slot();
+
+// Raises a kernel's dynamic-LDS limit on the current device, once per device and kernel
+// (the attribute is per device; `done` is the kernel's own flag array of kMaxDevices
+// entries).  Returns false with the error set if the runtime refuses.
+bool ensure_dynamic_lds(const void* kernel, int bytes, bool* done);
+
+// Compute units of the current device (cached per device).
+int cu_count();
+
 }  // namespace wq
