@@ -2,8 +2,8 @@
 // y[M,N] = x[M,K] @ dequant(Wq,S)^T.
 //
 // Bound: dense float16 MFMA; the design goal is to keep LDS traffic (128 B/clk/CU on
-// gfx950) well below the matrix pipe's appetite.  A workgroup owns a BM x (64*WAVES)
-// output tile; all wavefronts share the same BM activation rows (staged in LDS) and
+// gfx950) well below the matrix pipe's appetite.  A workgroup owns a BM x 256 output tile
+// (BM = 128, or 64 when M is too small to give every CU a 128-row tile); all wavefronts share the same BM activation rows (staged in LDS) and
 // each owns 64 distinct weight rows, i.e. a BM x 64 sub-tile of 32x32x16 MFMAs.  The
 // MFMA B operand of lane (col = lane % 32, kh = lane / 32) for 16-wide k slice kk is
 // the 8 weights k = k0 + (kh*4 + kk)*8 .. +8 of row `col` -- exactly one packed int4
@@ -63,12 +63,13 @@ struct RawB {
   u32x4 w[2][NV];                               // [column tile][load]
 };
 
-template <int BITS, int GROUPS>
+template <int BITS, int GROUPS, int TM>
 __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
     half_t* y, int M, int N, int K, int group_shift, int zero_point, int tiles_m, int tiles_n,
     const Epilogue ep) {
-  constexpr int BK = 64, TM = 4, WAVES = 4;
+  constexpr int BK = 64, WAVES = 4;
+  static_assert(TM == 4 || TM == 2, "row blocks of 32 per wavefront: 128- or 64-row tile");
   constexpr int BM = TM * 32;
   constexpr int NT = WAVES * 64;   // threads of one K group
   constexpr int CH = 128 / BITS;   // k per 16-byte packed chunk
@@ -76,10 +77,11 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
   constexpr int XL = BM * 8 / NT;  // 16-byte activation chunks per thread per step
   constexpr int STAGE = BM * 128;  // bytes per LDS stage
   // register sets: two wavefronts per SIMD leave 128 VGPRs beside the accumulators and hide
-  // latency by themselves, so the K-group variant prefetches only one step deep
+  // latency by themselves, so the K-group variants prefetch only one step deep (deeper rings
+  // were measured with the 64-row tile, where registers would allow them: no gain)
   constexpr int RB = (BITS == 4 && GROUPS == 1) ? 4 : 2;  // packed weights
   constexpr int XS = GROUPS == 1 ? 2 : 1;                 // activations
-  static_assert(XL == 4, "activation tile / thread split");
+  static_assert(XL == TM, "activation tile / thread split: one 16-byte chunk per thread and row block");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char wq_gemm_direct_smem[];
 
@@ -219,10 +221,14 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
     return as_u32(v * bcast_h2(__builtin_bit_cast(half_t, (uint16_t)s_step[parity][j])));
   };
 
+  // A B fragment (four pairs) feeds TM MFMAs, so PPS = 4 / TM pairs enter and leave the
+  // conversion pipeline per MFMA slot; a pair leaves LEAD slots before its fragment's first use.
+  constexpr int PPS = 4 / TM;
+  constexpr int LEAD = TM == 4 ? 5 : 3;
   half8_t fa[2][TM];
   u32x4 fbq[4];  // ring of B fragments (fragment q of a step lives in fbq[q % 4])
-  uint32_t t_perm, t_bits;  // pipeline registers of the pair conversion
-  half2_t t_center;
+  uint32_t t_perm[PPS], t_bits[PPS];  // pipeline registers of the pair conversion
+  half2_t t_center[PPS];
   auto read_a = [&](int buf, uint32_t base, auto ic) {
     constexpr int i = decltype(ic)::value;
     fa[buf][i] = *reinterpret_cast<const half8_t*>(lds + base + (uint32_t)i * 4096u);
@@ -273,14 +279,18 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
   static_for_d<0, TM>([&](auto ic) { read_a(0, a_rd[0], ic); });
 #pragma unroll
   for (int j = 0; j < 2; ++j) s_step[0][j] = pick_scale(sc_cur, j, 0);
-  // prime the conversion pipeline: pairs 0..4 complete, 5 / 6 / 7 three / two / one stage in
-  static_for_d<0, 5>([&](auto gc) {
+  // prime the conversion pipeline: the first PPS * LEAD pairs complete, then PPS pairs each
+  // three, two and one stage in
+  static_for_d<0, PPS * LEAD>([&](auto gc) {
     constexpr int g = decltype(gc)::value;
     fbq[g / 4][g & 3] = stage_scale(0, stage_center(stage_bits(stage_perm(rb[0], gc))), gc);
   });
-  t_center = stage_center(stage_bits(stage_perm(rb[0], std::integral_constant<int, 5>{})));
-  t_bits = stage_bits(stage_perm(rb[0], std::integral_constant<int, 6>{}));
-  t_perm = stage_perm(rb[0], std::integral_constant<int, 7>{});
+  static_for_d<0, PPS>([&](auto pc) {
+    constexpr int pp = decltype(pc)::value;
+    t_center[pp] = stage_center(stage_bits(stage_perm(rb[0], std::integral_constant<int, PPS * LEAD + pp>{})));
+    t_bits[pp] = stage_bits(stage_perm(rb[0], std::integral_constant<int, PPS * (LEAD + 1) + pp>{}));
+    t_perm[pp] = stage_perm(rb[0], std::integral_constant<int, PPS * (LEAD + 2) + pp>{});
+  });
 
   // One K step, P = (step number in the group) % 4 fixes every register set and LDS stage at
   // compile time.
@@ -304,17 +314,18 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
       const half8_t bm = __builtin_bit_cast(half8_t, fbq[q & 3]);
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk & 1][i], bm, acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-      // pair conversion pipeline: slot s finishes pair s+5 and starts pair s+8 (pairs 32..
-      // belong to the next step's packed weights)
-      {
-        constexpr int gd = s + 5, ga = s + 8;
-        fbq[(gd / 4) & 3][gd & 3] = stage_scale(gd < 32 ? (P & 1) : ((P + 1) & 1), t_center,
+      // pair conversion pipeline: slot s finishes pairs PPS*(s+LEAD).. and starts the pairs three
+      // slots behind them (pairs 32.. belong to the next step's packed weights)
+      static_for_d<0, PPS>([&](auto pc) {
+        constexpr int pp = decltype(pc)::value;
+        constexpr int gd = PPS * (s + LEAD) + pp, ga = gd + 3 * PPS;
+        fbq[(gd / 4) & 3][gd & 3] = stage_scale(gd < 32 ? (P & 1) : ((P + 1) & 1), t_center[pp],
                                                 std::integral_constant<int, gd & 31>{});
-        t_center = stage_center(t_bits);
-        t_bits = stage_bits(t_perm);
-        t_perm = ga < 32 ? stage_perm(bcur, std::integral_constant<int, ga & 31>{})
-                         : stage_perm(bnxt, std::integral_constant<int, ga & 31>{});
-      }
+        t_center[pp] = stage_center(t_bits[pp]);
+        t_bits[pp] = stage_bits(t_perm[pp]);
+        t_perm[pp] = ga < 32 ? stage_perm(bcur, std::integral_constant<int, ga & 31>{})
+                             : stage_perm(bnxt, std::integral_constant<int, ga & 31>{});
+      });
       // A fragments of the next slice (slice 0 of the next stage at the end), one per slot
       if constexpr (j == 0)
         read_a((kk + 1) & 1, a_rd[(kk + 1) & 3] + (kk == 3 ? st_next : st_rd), std::integral_constant<int, i>{});
@@ -327,10 +338,11 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
       }
       // packed weights of step kt + RB - 1, into the set whose last use has passed
       if constexpr (RB == 4) {
-        if constexpr (kk == 1 && j == 1 && i < PBL) load_b(bload, kt + 3, std::integral_constant<int, i>{});
+        if constexpr (kk == 1 && j * TM + i < PBL) load_b(bload, kt + 3, std::integral_constant<int, j * TM + i>{});
       } else {
         // two sets: the current step's set is free once its last pair has entered the pipeline
-        if constexpr (kk == 3 && j == 1 && i < PBL) load_b(bcur, kt + 2, std::integral_constant<int, i>{});
+        // (slot NMFMA - LEAD - 3 - 1 at the latest, i.e. before the last slice)
+        if constexpr (kk == 3 && j * TM + i < PBL) load_b(bcur, kt + 2, std::integral_constant<int, j * TM + i>{});
       }
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -350,12 +362,12 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
   }
 
   // ---- K groups: the second group hands its partial sums over through LDS -----------------
-  // Two rounds of 64 KB (row blocks i = 0,1 then 2,3); a wavefront and its partner hold the
+  // Rounds of 64 KB (two row blocks each); a wavefront and its partner hold the
   // same elements in the same lanes, so the exchange is lane-contiguous 16-byte vectors.
   if constexpr (GROUPS == 2) {
     float4_t* const xch = reinterpret_cast<float4_t*>(wq_gemm_direct_smem) + wave * (16 * 64) + lane;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < TM / 2; ++h) {
       if (grp == 1) {
 #pragma unroll
         for (int il = 0; il < 2; ++il)
@@ -401,36 +413,44 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
 
 namespace {
 
-template <int BITS, int GROUPS>
+template <int BITS, int GROUPS, int TM>
 bool launch_direct(const Problem& p, int group_shift) {
-  constexpr int BM = 128, BN = 256;
+  constexpr int BM = TM * 32, BN = 256;
   const int tiles_m = (int)((p.m + BM - 1) / BM);
   const int tiles_n = (int)((p.n + BN - 1) / BN);
   dim3 grid(tiles_m * tiles_n), block(GROUPS * 256);
-  constexpr size_t lds_bytes = (size_t)GROUPS * 4 * BM * 128;  // four activation stages per K group
+  // four activation stages per K group; the K-group exchange needs 64 KB
+  constexpr size_t lds_bytes = GROUPS == 2 && TM == 2 ? 65536 : (size_t)GROUPS * 4 * BM * 128;
   static bool lds_ok[kMaxDevices] = {false};
-  if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS>, (int)lds_bytes, lds_ok)) return false;
-  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS>), grid, block, lds_bytes, p.stream,
+  if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS, TM>, (int)lds_bytes, lds_ok)) return false;
+  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
                      tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
   return true;
 }
 
+template <int GROUPS, int TM>
+bool launch_bits(const Problem& p, int group_shift) {
+  return p.bits == 4 ? launch_direct<4, GROUPS, TM>(p, group_shift) : launch_direct<8, GROUPS, TM>(p, group_shift);
+}
+
 }  // namespace
 
-// 128 x 256 tile; variant 1: four wavefronts (one per SIMD), variant 2: eight wavefronts in
-// two K groups (two per SIMD), each group accumulating half of K
+// 256 output columns per workgroup.  variant 1: 128 rows, four wavefronts (one per SIMD);
+// variant 2: 128 rows, eight wavefronts in two K groups (two per SIMD), each group accumulating
+// half of K; variants 3 / 4: the same with 64 rows per workgroup -- twice the tiles and about
+// half the time per K step, for M too small to give every CU a 128-row tile.
 bool launch_gemm_direct(const Problem& p, int group_shift, int variant) {
   if (!gemm_pipe_applicable(p)) return false;
   // scales are fetched per 256 k: the kernel is laid out for the two benchmark quantizations
   if (p.k % 256 != 0 || p.group != (p.bits == 4 ? 32 : 128)) return false;
+  if ((variant == 2 || variant == 4) && p.k < 512) return false;
   switch (variant) {
-    case 1:
-      return p.bits == 4 ? launch_direct<4, 1>(p, group_shift) : launch_direct<8, 1>(p, group_shift);
-    case 2:
-      if (p.k < 512) return false;
-      return p.bits == 4 ? launch_direct<4, 2>(p, group_shift) : launch_direct<8, 2>(p, group_shift);
+    case 1: return launch_bits<1, 4>(p, group_shift);
+    case 2: return launch_bits<2, 4>(p, group_shift);
+    case 3: return launch_bits<1, 2>(p, group_shift);
+    case 4: return launch_bits<2, 2>(p, group_shift);
     default: return false;
   }
 }
