@@ -170,7 +170,7 @@ def main() -> int:
                    "launches_per_step": launches_per_step, "bytes_per_step": bytes_per_step},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "wq::wq_gemv_kernel (all decode launches)",
+                     "kernel": "wq::wq_gemv_kernel (7 of the 8 shape/batch cases; batch 8 on 4096x11008 runs wq::wq_skinny_kernel)",
                      "bytes_per_launch": bytes_per_step // launches_per_step,
                      "avg_launch_us": round(avg_launch_us, 3)},
     }

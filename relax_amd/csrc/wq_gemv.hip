@@ -384,7 +384,10 @@ int launch_gemv(const Problem& p, int variant) {
     // workgroups per CU, larger batches (more LDS per workgroup) with one.  Two-chunk
     // super steps first, single chunks (any K) as the fallback.
     const int small[] = {25, 15, 24, 14}, large[] = {15, 14, 15, 14};
-    const int* order = p.m <= 4 ? small : large;
+    // (rows of more than 4 KB -- int8 weights, long K -- already give one workgroup per CU
+    // enough bytes in flight: two per CU measured 8-10 % slower there)
+    const int64_t row_bytes = p.k * p.bits / 8;
+    const int* order = (p.m <= 4 && row_bytes <= 4096) ? small : large;
     for (int q = 0; q < 4; ++q) {
       const int v = order[q];
       ok = p.bits == 4 ? dispatch<4>(p, gs, v) : dispatch<8>(p, gs, v);
