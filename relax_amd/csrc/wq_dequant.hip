@@ -1,50 +1,63 @@
 // Bit-exact dequantization kernel: wd[N,K] float16 from packed int4/int8 + group
-// scales.  HBM-bound (write dominated: 2 bytes out per 0.5 or 1 byte in); every
-// lane converts one 16-byte packed chunk and issues 16-byte stores.
+// scales.  HBM-bound (write dominated: 2 bytes out per 0.5 or 1 byte in).
 #include "wq_device.h"
 #include "wq_internal.h"
 
 namespace wq {
 
+// One lane converts 8 weights -- one packed int4 word or two int8 words -- per round:
+// consecutive lanes read consecutive words and write consecutive 16-byte pieces, so every
+// load and every store instruction of a wavefront covers one contiguous span.  (K is a
+// multiple of the group size, at least 16, so 8 weights never straddle a row or a group.)
 template <int BITS>
 __global__ __launch_bounds__(256) void wq_dequant_kernel(const uint32_t* __restrict__ wq,
                                                          const half_t* __restrict__ scales,
                                                          half_t* __restrict__ wd, uint32_t n_rows,
                                                          uint32_t k, uint32_t group, int zero_point) {
-  constexpr uint32_t CH = 128 / BITS;  // k per 16-byte chunk: 32 (int4) / 16 (int8)
-  const uint32_t chunks_per_row = k / CH;
-  const uint64_t total = (uint64_t)n_rows * chunks_per_row;
-  const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= total) return;
-  const uint32_t n = (uint32_t)(idx / chunks_per_row);
-  const uint32_t c = (uint32_t)(idx - (uint64_t)n * chunks_per_row);
-  const u32x4 w = *reinterpret_cast<const u32x4*>(wq + idx * 4);
-  const half_t s = scales[(uint64_t)n * (k / group) + (c * CH) / group];
-  const half2_t s2 = bcast_h2(s);
-  u32x4* out = reinterpret_cast<u32x4*>(wd + ((uint64_t)n * k + (uint64_t)c * CH));
-  if constexpr (BITS == 4) {
-    const Q4Consts cs = make_q4_consts(zero_point);
+  constexpr int WPL = BITS / 4;  // packed words per lane and round: 1 (int4), 2 (int8)
+  constexpr int ROUNDS = 4;
+  const uint32_t units_per_row = k / 8;  // 8 weights = 16 bytes of output
+  const uint64_t total = (uint64_t)n_rows * units_per_row;
+  const uint32_t groups_per_row = k / group;
+  const Q4Consts cs = make_q4_consts(zero_point);
+  const uint64_t base = (uint64_t)blockIdx.x * (256 * ROUNDS) + threadIdx.x;
+  uint32_t w[ROUNDS][WPL];
+  half_t s[ROUNDS];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      half2_t h[4];
-      q4_word_natural(w[j], s2, cs, h);
-      out[j] = u32x4{as_u32(h[0]), as_u32(h[1]), as_u32(h[2]), as_u32(h[3])};
+  for (int r = 0; r < ROUNDS; ++r) {
+    const uint64_t idx = base + (uint64_t)r * 256;
+    if (idx < total) {
+      const uint32_t n = (uint32_t)(idx / units_per_row);
+      const uint32_t c = (uint32_t)(idx - (uint64_t)n * units_per_row);
+      if constexpr (WPL == 1) {
+        w[r][0] = wq[idx];
+      } else {
+        const u32x2 v = reinterpret_cast<const u32x2*>(wq)[idx];
+        w[r][0] = v[0];
+        w[r][1] = v[1];
+      }
+      s[r] = scales[(uint64_t)n * groups_per_row + (c * 8) / group];
     }
-  } else {
+  }
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      half2_t a[2], b[2];
-      q8_word_natural(w[2 * j], s2, a);
-      q8_word_natural(w[2 * j + 1], s2, b);
-      out[j] = u32x4{as_u32(a[0]), as_u32(a[1]), as_u32(b[0]), as_u32(b[1])};
+  for (int r = 0; r < ROUNDS; ++r) {
+    const uint64_t idx = base + (uint64_t)r * 256;
+    if (idx >= total) continue;
+    const half2_t s2 = bcast_h2(s[r]);
+    half2_t h[4];
+    if constexpr (BITS == 4) {
+      q4_word_natural(w[r][0], s2, cs, h);
+    } else {
+      q8_word_natural(w[r][0], s2, h);
+      q8_word_natural(w[r][WPL - 1], s2, h + 2);
     }
+    reinterpret_cast<u32x4*>(wd)[idx] = u32x4{as_u32(h[0]), as_u32(h[1]), as_u32(h[2]), as_u32(h[3])};
   }
 }
 
 int launch_dequant(const Problem& p, void* wd) {
-  const uint32_t ch = 128 / p.bits;
-  const uint64_t total = (uint64_t)p.n * (p.k / ch);
-  const uint64_t blocks = (total + 255) / 256;
+  const uint64_t total = (uint64_t)p.n * (p.k / 8);  // units of 8 weights
+  const uint64_t blocks = (total + 1023) / 1024;     // 256 threads x 4 units
   if (blocks == 0) return 0;
   if (blocks > 0x7FFFFFFFull) {
     set_error("dequantize: %lld x %lld is too large for one launch", (long long)p.n, (long long)p.k);
