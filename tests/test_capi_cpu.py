@@ -294,3 +294,42 @@ def test_registration_through_the_tvm_c_api(tmp_path):
     out = subprocess.run([sys.executable, "-c", REGISTRY_SCRIPT.format(root=ROOT, fake=fake)],
                          capture_output=True, text=True, timeout=300)
     assert out.returncode == 0 and "registry ok" in out.stdout, out.stdout + out.stderr
+
+
+# ---------------------------------------------------------------- the headers are plain C, usable without Python
+C_CLIENT = r"""
+#include <stdio.h>
+#include <string.h>
+#include "mi355x_wq.h"
+#include "mi355x_wq_packed.h"
+
+int main(void) {
+  mi355x_wq_desc d = {4, 32, 7, 0, 4096, 4096};
+  mi355x_wq_epilogue ep = {NULL, NULL, MI355X_WQ_ACT_RELU, 0};
+  mi355x_wq_callspec spec = {0, 4, 0, 7, 0, 1, 2, 3, 4, -1, -1, MI355X_WQ_ACT_NONE};
+  if (mi355x_wq_version() < 100) return 1;
+  if (mi355x_wq_check(&d, 8) != 0) return 2;
+  if (mi355x_wq_select_kernel(&d, 8) != MI355X_WQ_KERNEL_GEMV) return 3;
+  d.group = 48;
+  if (mi355x_wq_check(&d, 8) != -1 || strstr(mi355x_wq_last_error(), "group") == NULL) return 4;
+  d.group = 32;
+  /* a NULL operand is refused before anything touches the GPU */
+  if (mi355x_wq_matmul_fused(&d, NULL, NULL, NULL, &ep, NULL, 8, NULL) != -1) return 5;
+  if (strstr(mi355x_wq_last_error(), "x is NULL") == NULL) return 6;
+  if (mi355x_wq_packed_call(&spec, NULL, NULL, 4) != -1) return 7;
+  if (sizeof(mi355x_dl_tensor) != 48 || sizeof(mi355x_tvm_value) != 8) return 8;  /* DLPack / TVMValue ABI sizes */
+  puts("c client ok");
+  return 0;
+}
+"""
+
+
+def test_headers_compile_as_c99_and_link(tmp_path):
+    src = tmp_path / "client.c"
+    src.write_text(C_CLIENT)
+    exe = str(tmp_path / "client")
+    libdir = os.path.dirname(lib.SO_PATH)
+    subprocess.check_call(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"),
+                           "-o", exe, str(src), "-L" + libdir, "-lmi355x_wq", "-Wl,-rpath," + libdir])
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and "c client ok" in out.stdout, (out.returncode, out.stdout, out.stderr)
