@@ -210,10 +210,10 @@ int launch_gemm(const Problem& p, int variant) {
     return -1;
   }
   if (variant == 0 && gemm_pipe_applicable(p)) {
-    // measured on MI355X, M = 128 .. 4096 on the Llama shapes: the direct-weight kernel with
-    // two K groups wins everywhere it applies; next the same kernel with one group, then the
-    // LDS-staged pipeline (256x128 tile once M fills it a few times over, else 128x128)
-    // (64-row tiles while 128-row tiles would leave half of the CUs without one)
+    // Measured on MI355X, M = 128 .. 4096 on the Llama shapes: the direct-weight kernel with two
+    // K groups wins wherever it applies -- with 64-row tiles while 128-row tiles would leave
+    // half of the CUs without one; next the same kernel with one group (K below 512), then the
+    // LDS-staged pipeline (256x128 tile once M fills it a few times over, else 128x128).
     const int64_t tiles128 = ((p.m + 127) / 128) * ((p.n + 255) / 256);
     const int first = tiles128 <= cu_count() / 2 ? 4 : 2;
     if (launch_gemm_direct(p, group_shift, first) || launch_gemm_direct(p, group_shift, first - 1)) variant = -1;
