@@ -364,7 +364,61 @@ int dispatch(const Problem& p, int gs, int variant) {
 
 }  // namespace
 
-bool gemv_applicable(const Problem& p) { return p.m >= 1 && p.m <= 16; }
+namespace {
+
+// The variants the default dispatch tries, in order (see launch_gemv).
+const int* default_order(const Problem& p) {
+  // Measured on MI355X (Llama-2-7B shapes): up to 4 rows run best with two 8-wave
+  // workgroups per CU, larger batches (more LDS per workgroup) with one.  Two-chunk
+  // super steps first, single chunks (any K) as the fallback.
+  // (rows of more than 4 KB -- int8 weights, long K -- already give one workgroup per CU
+  // enough bytes in flight: two per CU measured 8-10 % slower there)
+  static const int small[] = {25, 15, 24, 14}, large[] = {15, 14, 15, 14};
+  const int64_t row_bytes = p.k * p.bits / 8;
+  return (p.m <= 4 && row_bytes <= 4096) ? small : large;
+}
+
+// Whether `variant` can be launched for p: K divisibility and an LDS plan (partial-tile slots of
+// the tiles a workgroup owns + staged activations).  Mirrors dispatch() without launching.
+template <int BITS>
+bool variant_has_plan(const Problem& p, int gs, int variant) {
+  const int wpc = variant / 10, shape = variant % 10;
+  constexpr int ch = 128 / BITS;
+  const int waves = shape <= 3 ? 4 : (shape <= 6 ? 8 : 16);
+  const int d = shape <= 6 ? (1 << ((shape - 1) % 3)) : (shape == 7 ? 1 : 2);
+  if (wpc < 1 || wpc > 8 || shape < 1 || shape > 8) return false;
+  if (d > 1 && p.k % (4 * d * ch) != 0) return false;
+  if (gs != 0 && (1 << gs) < d) return false;
+  Plan plan;
+  switch (waves * 10 + d) {
+    case 41: return make_plan<BITS, 4, 1>(p, wpc, &plan);
+    case 42: return make_plan<BITS, 4, 2>(p, wpc, &plan);
+    case 44: return make_plan<BITS, 4, 4>(p, wpc, &plan);
+    case 81: return make_plan<BITS, 8, 1>(p, wpc, &plan);
+    case 82: return make_plan<BITS, 8, 2>(p, wpc, &plan);
+    case 84: return make_plan<BITS, 8, 4>(p, wpc, &plan);
+    case 161: return make_plan<BITS, 16, 1>(p, wpc, &plan);
+    case 162: return make_plan<BITS, 16, 2>(p, wpc, &plan);
+    default: return false;
+  }
+}
+
+}  // namespace
+
+// M <= 16 and one of the default variants fits: with very many row tiles per workgroup (N in the
+// hundreds of thousands) the per-tile partial-sum slots outgrow LDS and the caller falls back to
+// the register-activation kernel.
+bool gemv_applicable(const Problem& p) {
+  if (p.m < 1 || p.m > 16) return false;
+  const int ch = 128 / p.bits;
+  int ratio = p.group / ch, gs = 0;
+  while ((1 << gs) < ratio) ++gs;
+  if (ratio < 1 || (1 << gs) != ratio) return false;
+  const int* order = default_order(p);
+  for (int q = 0; q < 4; ++q)
+    if (p.bits == 4 ? variant_has_plan<4>(p, gs, order[q]) : variant_has_plan<8>(p, gs, order[q])) return true;
+  return false;
+}
 
 int launch_gemv(const Problem& p, int variant) {
   const int ch = 128 / p.bits;
@@ -374,20 +428,13 @@ int launch_gemv(const Problem& p, int variant) {
     set_error("gemv kernel: group %d must be %d times a power of two", p.group, ch);
     return -1;
   }
-  if (!gemv_applicable(p)) {
+  if (p.m < 1 || p.m > 16) {
     set_error("gemv kernel: M=%lld is outside 1..16", (long long)p.m);
     return -1;
   }
   int ok = kNotApplicable;
   if (variant == 0) {
-    // Measured on MI355X (Llama-2-7B shapes): up to 4 rows run best with two 8-wave
-    // workgroups per CU, larger batches (more LDS per workgroup) with one.  Two-chunk
-    // super steps first, single chunks (any K) as the fallback.
-    const int small[] = {25, 15, 24, 14}, large[] = {15, 14, 15, 14};
-    // (rows of more than 4 KB -- int8 weights, long K -- already give one workgroup per CU
-    // enough bytes in flight: two per CU measured 8-10 % slower there)
-    const int64_t row_bytes = p.k * p.bits / 8;
-    const int* order = (p.m <= 4 && row_bytes <= 4096) ? small : large;
+    const int* order = default_order(p);
     for (int q = 0; q < 4; ++q) {
       const int v = order[q];
       ok = p.bits == 4 ? dispatch<4>(p, gs, v) : dispatch<8>(p, gs, v);

@@ -22,7 +22,7 @@ struct Problem {
 // Tuning variant: 0 = library default for the shape, >0 = explicit choice
 // (only reachable through mi355x_wq_matmul_ex; used by sweeps).
 int launch_gemv(const Problem& p, int variant);
-bool gemv_applicable(const Problem& p);  // M <= 16 and the activations fit the LDS staging area
+bool gemv_applicable(const Problem& p);  // M <= 16 and a default variant's LDS plan (slots + activations) fits
 int launch_skinny(const Problem& p, int variant);
 int launch_gemm(const Problem& p, int variant);
 bool gemm_pipe_applicable(const Problem& p);  // K % 64 == 0, operands below 1 GiB

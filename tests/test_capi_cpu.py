@@ -75,6 +75,9 @@ def test_kernel_selection_by_rows():
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 11008), 2) == lib.KERNEL_GEMV
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 11008), 8) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 22016, 11008), 8) == lib.KERNEL_GEMV
+    # a vocabulary-sized projection: too many row tiles per workgroup for the GEMV kernel's LDS slots
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 152064, 4096), 1) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 32000, 4096), 1) == lib.KERNEL_GEMV
     assert L.mi355x_wq_select_kernel(d, 17) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(d, 64) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(d, 65) == lib.KERNEL_GEMM

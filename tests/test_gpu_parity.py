@@ -121,6 +121,21 @@ def test_gemv_k_phases_when_activations_exceed_lds(bits, m, n, k):
     assert_close(got, want, (bits, m, n, k))
 
 
+@pytest.mark.parametrize("m", [1, 8])
+def test_vocabulary_sized_projection(m):
+    """N = 152064 (an lm_head): more row tiles per workgroup than the GEMV kernel's LDS slots hold, so the
+    default dispatch uses the register-activation kernel; forcing the GEMV family is refused."""
+    from relax_amd import lib
+
+    n, k = 152064, 1024
+    x, wq, s, g = O.make_case(19, m, n, k, 4)
+    got = run_matmul(x, wq, s, 4, g)
+    want = c_oracle.wq_matmul(x, wq, s, 4, g, nthreads=16)
+    assert_close(got, want, ("lm_head", m))
+    with pytest.raises(lib.WqError, match="does not apply"):
+        run_matmul(x, wq, s, 4, g, kernel=lib.KERNEL_GEMV)
+
+
 def test_gemv_refuses_more_than_16_rows():
     from relax_amd import lib
 
