@@ -466,3 +466,26 @@ def test_fused_argument_checks():
         relax_amd.wq_matmul(xd, wd, sd, 4, g, residual=torch.zeros((1, 32), dtype=torch.float16, device="cuda"))
     with pytest.raises(ValueError, match="bias must be"):
         relax_amd.wq_matmul(xd, wd, sd, 4, g, bias=torch.zeros(32, dtype=torch.float32, device="cuda"))
+
+
+# ------------------------------------------------------------------ int4 zero points other than 7
+@pytest.mark.parametrize("zero_point", [0, 8, 15])
+def test_int4_zero_points(zero_point):
+    """The descriptor carries the zero point (0..15 for int4); every kernel family must honour it:
+    dequantize bit for bit, the matmuls within tolerance of the NumPy oracle with that zero point."""
+    import relax_amd
+    from relax_amd import lib
+
+    for m, n, k, kernel, variant in [(1, 64, 256, lib.KERNEL_GEMV, 0), (8, 40, 352, lib.KERNEL_GEMV, 14),
+                                     (33, 48, 256, lib.KERNEL_SKINNY, 0), (129, 300, 512, lib.KERNEL_GEMM, 22),
+                                     (70, 136, 768, lib.KERNEL_GEMM, 24), (200, 96, 320, lib.KERNEL_GEMM, 12),
+                                     (70, 32, 96, lib.KERNEL_GEMM, 1)]:
+        x, wq, s, g = O.make_case(40 + zero_point + m, m, n, k, 4)
+        wd = O.dequant_q4f16(wq, s, g, zero_point)
+        want = O.cast_f16(O.matmul_f32acc(x, wd))
+        xd, wqd, sd = _dev(x), _dev(wq), _dev(s)
+        got_wd = relax_amd.wq_dequantize(wqd, sd, 4, g, zero_point=zero_point).cpu().numpy()
+        assert np.array_equal(got_wd.view(np.uint16), wd.view(np.uint16)), (zero_point, n, k)
+        got = relax_amd.wq_matmul(xd, wqd, sd, 4, g, zero_point=zero_point, kernel=kernel, variant=variant)
+        torch.cuda.synchronize()
+        assert_close(got.cpu().numpy(), want, (zero_point, m, n, k, kernel, variant))
