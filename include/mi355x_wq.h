@@ -16,7 +16,8 @@
  *   bits = 4: wd = (f16(field) - f16(zero_point)) * scale   (one float16 rounding)
  *   bits = 8: wd = f16(int8(field)) * scale                 (zero_point must be 0)
  *
- * Every pointer is device memory of the current HIP device.  All launches are
+ * Every pointer is device memory of the current HIP device; x, wq, scales and wd must be
+ * 16-byte aligned (y, bias and residual: 2 bytes).  All launches are
  * asynchronous on `stream` (a hipStream_t passed as void*; NULL = the null
  * stream); synchronisation is the caller's.  Functions return 0 on success and
  * -1 on failure, in which case nothing was launched and

@@ -172,7 +172,9 @@ int mi355x_wq_matmul_fused_ex(const mi355x_wq_desc* desc, const void* x, const v
     set_error("K = 0 is not supported (the output would be all zeros)");
     return -1;
   }
-  if (!check_ptr(x, "x", 16) || !check_ptr(wq_, "wq", 16) || !check_ptr(scales, "scales", 2) ||
+  // scales are fetched with up to 16-byte vector loads (rows of scales are 16-byte multiples
+  // whenever a kernel does so), hence the same alignment as the other operands
+  if (!check_ptr(x, "x", 16) || !check_ptr(wq_, "wq", 16) || !check_ptr(scales, "scales", 16) ||
       !check_ptr(y, "y", 2))
     return -1;
   if (ep != nullptr && ep->bias != nullptr && !check_ptr(ep->bias, "bias", 2)) return -1;
