@@ -215,8 +215,12 @@ int launch_gemm(const Problem& p, int variant) {
     // half of the CUs without one; next the same kernel with one group (K below 512), then the
     // LDS-staged pipeline (256x128 tile once M fills it a few times over, else 128x128).
     const int64_t tiles128 = ((p.m + 127) / 128) * ((p.n + 255) / 256);
+    const int64_t tiles64x128 = ((p.m + 63) / 64) * ((p.n + 127) / 128);
     const int first = tiles128 <= cu_count() / 2 ? 4 : 2;
-    if (launch_gemm_direct(p, group_shift, first) || launch_gemm_direct(p, group_shift, first - 1)) variant = -1;
+    // (and 64x128 tiles with four K groups while even those fit the CUs in one round)
+    if ((tiles64x128 <= cu_count() && launch_gemm_direct(p, group_shift, 5)) ||
+        launch_gemm_direct(p, group_shift, first) || launch_gemm_direct(p, group_shift, first - 1))
+      variant = -1;
     else variant = p.m >= 1024 ? 11 : 12;
   }
   if (variant == -1) {

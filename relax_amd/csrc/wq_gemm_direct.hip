@@ -63,13 +63,15 @@ struct RawB {
   u32x4 w[2][NV];                               // [column tile][load]
 };
 
-template <int BITS, int GROUPS, int TM>
-__global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
+template <int BITS, int GROUPS, int TM, int WAVES>
+__global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
     half_t* y, int M, int N, int K, int group_shift, int zero_point, int tiles_m, int tiles_n,
     const Epilogue ep) {
-  constexpr int BK = 64, WAVES = 4;
+  constexpr int BK = 64;
   static_assert(TM == 4 || TM == 2, "row blocks of 32 per wavefront: 128- or 64-row tile");
+  static_assert(WAVES == 4 || WAVES == 2, "wavefronts per K group: 256 or 128 output columns");
+  static_assert(GROUPS == 1 || GROUPS == 2 || GROUPS == 4, "K groups");
   constexpr int BM = TM * 32;
   constexpr int NT = WAVES * 64;   // threads of one K group
   constexpr int CH = 128 / BITS;   // k per 16-byte packed chunk
@@ -81,7 +83,7 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
   // were measured with the 64-row tile, where registers would allow them: no gain)
   constexpr int RB = (BITS == 4 && GROUPS == 1) ? 4 : 2;  // packed weights
   constexpr int XS = GROUPS == 1 ? 2 : 1;                 // activations
-  static_assert(XL == TM, "activation tile / thread split: one 16-byte chunk per thread and row block");
+  static_assert(XL >= 1 && XL <= 2 * TM, "activation chunks per thread must fit the MFMA slots of one k slice");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char wq_gemm_direct_smem[];
 
@@ -104,8 +106,8 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
 
   const int lane = threadIdx.x & 63;
   const int wave_id = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int grp = GROUPS == 1 ? 0 : wave_id >> 2;  // K group of this wavefront
-  const int wave = wave_id & 3;                    // 64-column slice of the tile
+  const int grp = GROUPS == 1 ? 0 : wave_id / WAVES;  // K group of this wavefront
+  const int wave = wave_id % WAVES;                   // 64-column slice of the tile
   const int tid = threadIdx.x & (NT - 1);          // thread index inside the K group
   const int fr = lane & 31, fh = lane >> 5;
   unsigned char* const lds = wq_gemm_direct_smem + grp * (4 * STAGE);  // the group's four stages
@@ -113,9 +115,9 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
   // K range of this group, in 64-wide steps; both groups run the same number of steps and
   // the shorter one reads zeros (out-of-range offsets) past its end.
   const int ksteps = K / BK;
-  const int nloop = GROUPS == 1 ? ksteps : 4 * ((ksteps / 4 + 1) / 2);
+  const int nloop = GROUPS == 1 ? ksteps : 4 * ((ksteps / 4 + GROUPS - 1) / GROUPS);
   const int kbase = grp * nloop;
-  const int kend = GROUPS == 1 ? ksteps : (grp == 0 ? nloop : ksteps);
+  const int kend = min(kbase + nloop, ksteps);
 
   const uint32_t row_bytes = (uint32_t)K * BITS / 8;
   const uint32_t groups_per_row = ((uint32_t)K / CH) >> group_shift;
@@ -330,11 +332,12 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
       if constexpr (j == 0)
         read_a((kk + 1) & 1, a_rd[(kk + 1) & 3] + (kk == 3 ? st_next : st_rd), std::integral_constant<int, i>{});
       // activations: registers -> LDS (step kt+2), then the same registers <- global (step kt+4)
-      if constexpr (kk == 0 && j == 1) store_x(xr[P % XS], st_wr, std::integral_constant<int, i>{});
+      constexpr int sq = 2 * TM - 1 - (j * TM + i);  // slot index inside the slice, from its end
+      if constexpr (kk == 0 && sq < XL) store_x(xr[P % XS], st_wr, std::integral_constant<int, sq>{});
       if constexpr (XS == 2) {
-        if constexpr (kk == 2 && j == 1) load_x(xr[P & 1], kt + 4, std::integral_constant<int, i>{});
+        if constexpr (kk == 2 && sq < XL) load_x(xr[P & 1], kt + 4, std::integral_constant<int, sq>{});
       } else {
-        if constexpr (kk == 1 && j == 1) load_x(xr[0], kt + 3, std::integral_constant<int, i>{});
+        if constexpr (kk == 1 && sq < XL) load_x(xr[0], kt + 3, std::integral_constant<int, sq>{});
       }
       // packed weights of step kt + RB - 1, into the set whose last use has passed
       if constexpr (RB == 4) {
@@ -361,40 +364,43 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
     load_scales(sc_nxt, kt + 8);
   }
 
-  // ---- K groups: the second group hands its partial sums over through LDS -----------------
-  // Rounds of 64 KB (two row blocks each); a wavefront and its partner hold the
+  // ---- K groups: the other groups hand their partial sums to the first through LDS ---------
+  // Rounds of 16 KB per wavefront (two row blocks each); a wavefront and its partners hold the
   // same elements in the same lanes, so the exchange is lane-contiguous 16-byte vectors.
-  if constexpr (GROUPS == 2) {
+  if constexpr (GROUPS > 1) {
     float4_t* const xch = reinterpret_cast<float4_t*>(wq_gemm_direct_smem) + wave * (16 * 64) + lane;
 #pragma unroll
-    for (int h = 0; h < TM / 2; ++h) {
-      if (grp == 1) {
+    for (int g = 1; g < GROUPS; ++g) {
 #pragma unroll
-        for (int il = 0; il < 2; ++il)
+      for (int h = 0; h < TM / 2; ++h) {
+        if (grp == g) {
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
+          for (int il = 0; il < 2; ++il)
 #pragma unroll
-            for (int v4 = 0; v4 < 4; ++v4) {
-              const float16_t& a = acc[h * 2 + il][j];
-              xch[((il * 2 + j) * 4 + v4) * 64] = float4_t{a[v4 * 4], a[v4 * 4 + 1], a[v4 * 4 + 2], a[v4 * 4 + 3]};
-            }
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+              for (int v4 = 0; v4 < 4; ++v4) {
+                const float16_t& a = acc[h * 2 + il][j];
+                xch[((il * 2 + j) * 4 + v4) * 64] = float4_t{a[v4 * 4], a[v4 * 4 + 1], a[v4 * 4 + 2], a[v4 * 4 + 3]};
+              }
+        }
+        __syncthreads();
+        if (grp == 0) {
+#pragma unroll
+          for (int il = 0; il < 2; ++il)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+              for (int v4 = 0; v4 < 4; ++v4) {
+                const float4_t o = xch[((il * 2 + j) * 4 + v4) * 64];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[h * 2 + il][j][v4 * 4 + e] += o[e];
+              }
+        }
+        __syncthreads();
       }
-      __syncthreads();
-      if (grp == 0) {
-#pragma unroll
-        for (int il = 0; il < 2; ++il)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v4 = 0; v4 < 4; ++v4) {
-              const float4_t o = xch[((il * 2 + j) * 4 + v4) * 64];
-#pragma unroll
-              for (int e = 0; e < 4; ++e) acc[h * 2 + il][j][v4 * 4 + e] += o[e];
-            }
-      }
-      __syncthreads();
     }
-    if (grp == 1) return;
+    if (grp != 0) return;
   }
 
   // ---- epilogue: lane holds column (lane % 32) and rows 8*(v/4) + 4*(lane/32) + v%4 ------
@@ -413,44 +419,51 @@ __global__ __launch_bounds__(GROUPS * 256, 1) void wq_gemm_direct_kernel(
 
 namespace {
 
-template <int BITS, int GROUPS, int TM>
+template <int BITS, int GROUPS, int TM, int WAVES>
 bool launch_direct(const Problem& p, int group_shift) {
-  constexpr int BM = TM * 32, BN = 256;
+  constexpr int BM = TM * 32, BN = WAVES * 64;
   const int tiles_m = (int)((p.m + BM - 1) / BM);
   const int tiles_n = (int)((p.n + BN - 1) / BN);
-  dim3 grid(tiles_m * tiles_n), block(GROUPS * 256);
-  // four activation stages per K group; the K-group exchange needs 64 KB
-  constexpr size_t lds_bytes = GROUPS == 2 && TM == 2 ? 65536 : (size_t)GROUPS * 4 * BM * 128;
+  dim3 grid(tiles_m * tiles_n), block(GROUPS * WAVES * 64);
+  // four activation stages per K group; the K-group exchange needs 16 KB per wavefront of a group
+  constexpr size_t stages = (size_t)GROUPS * 4 * BM * 128, exchange = GROUPS > 1 ? (size_t)WAVES * 16384 : 0;
+  constexpr size_t lds_bytes = stages > exchange ? stages : exchange;
+  static_assert(lds_bytes <= 160 * 1024, "LDS per workgroup");
   static bool lds_ok[kMaxDevices] = {false};
-  if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS, TM>, (int)lds_bytes, lds_ok)) return false;
-  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM>), grid, block, lds_bytes, p.stream,
+  if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES>, (int)lds_bytes, lds_ok))
+    return false;
+  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
                      tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
   return true;
 }
 
-template <int GROUPS, int TM>
+template <int GROUPS, int TM, int WAVES>
 bool launch_bits(const Problem& p, int group_shift) {
-  return p.bits == 4 ? launch_direct<4, GROUPS, TM>(p, group_shift) : launch_direct<8, GROUPS, TM>(p, group_shift);
+  return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES>(p, group_shift)
+                     : launch_direct<8, GROUPS, TM, WAVES>(p, group_shift);
 }
 
 }  // namespace
 
-// 256 output columns per workgroup.  variant 1: 128 rows, four wavefronts (one per SIMD);
-// variant 2: 128 rows, eight wavefronts in two K groups (two per SIMD), each group accumulating
-// half of K; variants 3 / 4: the same with 64 rows per workgroup -- twice the tiles and about
-// half the time per K step, for M too small to give every CU a 128-row tile.
+// variant 1: 128 x 256 tile, four wavefronts (one per SIMD); 2: the same tile, eight wavefronts in
+// two K groups (two per SIMD), each group accumulating half of K; 3 / 4: the same with 64 rows per
+// workgroup -- twice the tiles and about half the time per K step, for M too small to give every CU
+// a 128-row tile; 5: 64 x 128 tile, eight wavefronts in four K groups, for problems that leave CUs
+// idle even with 64 x 256 tiles.
 bool launch_gemm_direct(const Problem& p, int group_shift, int variant) {
   if (!gemm_pipe_applicable(p)) return false;
   // scales are fetched per 256 k: the kernel is laid out for the two benchmark quantizations
   if (p.k % 256 != 0 || p.group != (p.bits == 4 ? 32 : 128)) return false;
   if ((variant == 2 || variant == 4) && p.k < 512) return false;
+  if (variant == 5 && p.k < 1024) return false;
   switch (variant) {
-    case 1: return launch_bits<1, 4>(p, group_shift);
-    case 2: return launch_bits<2, 4>(p, group_shift);
-    case 3: return launch_bits<1, 2>(p, group_shift);
-    case 4: return launch_bits<2, 2>(p, group_shift);
+    case 1: return launch_bits<1, 4, 4>(p, group_shift);
+    case 2: return launch_bits<2, 4, 4>(p, group_shift);
+    case 3: return launch_bits<1, 2, 4>(p, group_shift);
+    case 4: return launch_bits<2, 2, 4>(p, group_shift);
+    case 5: return launch_bits<4, 2, 2>(p, group_shift);
     default: return false;
   }
 }

@@ -214,9 +214,12 @@ def test_gemm_kernel_matches_oracle(bits, m, n, k):
     (22, 8, 65, 300, 1792),
     (23, 4, 300, 200, 256), (23, 4, 65, 520, 1280), (23, 8, 129, 72, 256), (23, 8, 513, 260, 1024),
     (24, 4, 300, 200, 512), (24, 4, 65, 520, 1280), (24, 4, 70, 136, 768), (24, 8, 513, 260, 1024),
-    (24, 8, 100, 64, 1792)])
+    (24, 8, 100, 64, 1792),
+    (25, 4, 300, 200, 1024), (25, 4, 65, 520, 1280), (25, 4, 70, 136, 2304), (25, 8, 513, 260, 1024),
+    (25, 8, 100, 64, 1792)])
 def test_gemm_direct_weight_variants_match_oracle(variant, bits, m, n, k):
-    """Direct-weight kernel, 128-row tiles with one (21) and two (22) K groups and 64-row tiles (23, 24):
+    """Direct-weight kernel, 128-row tiles with one (21) and two (22) K groups, 64-row tiles (23, 24) and
+    64 x 128 tiles with four K groups (25):
     ragged M and N, K of one macro step, an even and an odd number of 256-wide macro steps (the second
     K group is then the shorter one)."""
     from relax_amd import lib
@@ -234,7 +237,7 @@ def test_gemm_direct_weight_variant_refuses_other_layouts():
 
     for bits, m, n, k, group in [(4, 200, 96, 320, 32), (4, 200, 96, 512, 64), (8, 200, 96, 512, 64)]:
         x, wq, s, g = O.make_case(9, m, n, k, bits, group)
-        for variant in (21, 22, 23, 24):
+        for variant in (21, 22, 23, 24, 25):
             with pytest.raises(lib.WqError, match="does not apply"):
                 run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_GEMM, variant=variant)
         assert_close(run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_GEMM),
@@ -388,7 +391,7 @@ def test_fused_tail_every_kernel_family(bits, m, n, k, tail):
     ("SKINNY", 1, 4, 20, 40, 256), ("SKINNY", 6, 8, 48, 24, 256),
     ("GEMM", 1, 4, 70, 136, 448), ("GEMM", 4, 8, 129, 72, 256), ("GEMM", 11, 4, 300, 200, 128),
     ("GEMM", 13, 8, 513, 260, 1024), ("GEMM", 21, 4, 129, 520, 1280), ("GEMM", 22, 8, 65, 300, 1792),
-    ("GEMM", 23, 8, 129, 72, 256), ("GEMM", 24, 4, 70, 136, 768),
+    ("GEMM", 23, 8, 129, 72, 256), ("GEMM", 24, 4, 70, 136, 768), ("GEMM", 25, 4, 129, 200, 1280),
 ])
 def test_fused_tail_explicit_kernel_variants(kernel, variant, bits, m, n, k):
     from relax_amd import lib
