@@ -513,3 +513,35 @@ def test_other_group_sizes_every_family(bits, group):
     _, wq, s, g = O.make_case(61, 1, 72, 2048, bits, group)
     wd = relax_amd.wq_dequantize(_dev(wq), _dev(s), bits, g).cpu().numpy()
     assert np.array_equal(wd.view(np.uint16), c_oracle.dequant(wq, s, bits, g).view(np.uint16))
+
+
+# ------------------------------------------------------------------ seeded random shapes, default dispatch
+def _random_shapes(seed, count):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for _ in range(count):
+        bits = int(rng.choice([4, 8]))
+        base = 32 if bits == 4 else 16
+        group = base * int(rng.choice([1, 1, 1, 2, 4] if bits == 4 else [8, 8, 8, 1, 2]))
+        k = group * int(rng.integers(1, 2048 // group + 1))
+        if rng.random() < 0.4:
+            k = 256 * int(rng.integers(1, 9))          # the direct-weight GEMM's K
+            group = 32 if bits == 4 else 128
+        m = int(rng.choice([1, 2, 3, 5, 8, 13, 16, 17, 31, 64, 65, 100, 129, 257, 300]))
+        n = int(rng.integers(1, 700))
+        shapes.append((bits, group, m, n, k))
+    return shapes
+
+
+@pytest.mark.parametrize("chunk", range(6))
+def test_seeded_random_shapes_default_dispatch(chunk):
+    """Ragged N (any value from 1), every M class, K any multiple of the group: the default dispatch against
+    the oracle, plain and with the full fused tail."""
+    for bits, group, m, n, k in _random_shapes(1000 + chunk, 12):
+        x, wq, s, g = O.make_case(chunk * 100 + m + n, m, n, k, bits, group)
+        want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
+        got = run_matmul(x, wq, s, bits, g)
+        assert_close(got, want, (bits, group, m, n, k))
+        bias, res = _fused_operands(m + n + k, m, n)
+        fused = run_fused(x, wq, s, bits, g, bias, "relu", res)
+        assert_fused(fused, got, want, bias, "relu", res, ("fused", bits, group, m, n, k))
