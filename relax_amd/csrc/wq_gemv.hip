@@ -57,7 +57,28 @@ struct GemvArgs {
 };
 
 template <int BITS, int WAVES, int D, int SPL>
-__global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(const GemvArgs a) {
+// (scalar kernel arguments instead of one struct: the first 16 dwords -- the operand pointers
+// and the shape -- are preloaded into SGPRs at wavefront launch, which takes the argument fetch
+// out of the start-up latency of a 5 - 15 us kernel)
+__global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
+    const half_t* x_, const uint32_t* wq_, const half_t* scales_, half_t* y_, int M_, int N_, int K_,
+    int group_shift_, int zero_point_, int lds_stride_, int tiles_, int max_tiles_, int phase_chunks_,
+    const Epilogue ep_) {
+  GemvArgs a;
+  a.x = x_;
+  a.wq = wq_;
+  a.scales = scales_;
+  a.y = y_;
+  a.M = M_;
+  a.N = N_;
+  a.K = K_;
+  a.group_shift = group_shift_;
+  a.zero_point = zero_point_;
+  a.lds_stride = lds_stride_;
+  a.tiles = tiles_;
+  a.max_tiles = max_tiles_;
+  a.phase_chunks = phase_chunks_;
+  a.ep = ep_;
   constexpr int CH = 128 / BITS;  // k per 16-byte lane load
   constexpr int NJ = CH / 8;      // MFMAs per lane load
   constexpr int NT = WAVES * 64;
@@ -327,7 +348,8 @@ int launch_one(const Problem& p, int group_shift, const Plan& plan) {
   if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL>, (int)kLdsPerWgMax, lds_ok))
     return kFailed;
   hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL>), dim3(plan.grid), dim3(WAVES * 64),
-                     plan.lds_bytes, p.stream, a);
+                     plan.lds_bytes, p.stream, a.x, a.wq, a.scales, a.y, a.M, a.N, a.K, a.group_shift,
+                     a.zero_point, a.lds_stride, a.tiles, a.max_tiles, a.phase_chunks, a.ep);
   return kLaunched;
 }
 
