@@ -188,26 +188,6 @@ def main() -> int:
                     relax_amd.wq_matmul(xg[k], wq, s, 4, 32, out=yg[n])
 
         flops = sum(2 * PREFILL_M * n * k for _, n, k in LLAMA7B) * len(use)
-        with torch.cuda.stream(stream):
-            for _ in range(1 + min(args.warmup, 3)):
-                prefill_pass()
-            torch.cuda.synchronize()
-            g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            reps = max(2, args.steps // 2)
-            g0.record(stream)
-            for _ in range(reps):
-                prefill_pass()
-            g1.record(stream)
-            torch.cuda.synchronize()
-        gms = g0.elapsed_time(g1) / reps
-        tflops = flops / (gms * 1e-3) / 1e12
-        result["gemm"] = {"value": round(tflops, 1), "unit": "TFLOP/s", "ms_per_pass": round(gms, 4),
-                          "workload": "q4f16 g32 prefill, M=2048, the four Llama-2-7B shapes x %d layers"
-                                      % len(use)}
-        result["roofline_gemm"] = {"bound": "mfma", "achieved": round(tflops, 1),
-                                   "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                   "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
-                                   "kernel": "wq::wq_gemm_direct_kernel"}
         # Context for the MFMA fraction: the vendor library's plain float16 GEMM (no dequantization)
         # on the same shapes and the same data -- weights dequantized beforehand, outside the timing.
         # With random operands the matrix pipes run power limited, far below the datasheet rate.
@@ -218,19 +198,39 @@ def main() -> int:
                 for (_, _, n, k), wd in zip(mats, dq):
                     torch.matmul(xg[k], wd.t(), out=yg[n])
 
-        with torch.cuda.stream(stream):
-            for _ in range(1 + min(args.warmup, 3)):
-                library_pass()
-            torch.cuda.synchronize()
+        def timed(fn, reps):
+            g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             g0.record(stream)
             for _ in range(reps):
-                library_pass()
+                fn()
             g1.record(stream)
             torch.cuda.synchronize()
-        lms = g0.elapsed_time(g1) / reps
-        result["gemm"]["library_f16_gemm_tflops"] = round(flops / (lms * 1e-3) / 1e12, 1)
-        result["gemm"]["library_f16_gemm_note"] = ("torch.matmul (hipBLASLt) on float16 weights dequantized "
-                                                   "beforehand, same shapes and data")
+            return g0.elapsed_time(g1) / reps
+
+        # the two are timed alternately (two rounds each) so that clock and temperature drift
+        # over the run affects both alike
+        reps = max(2, args.steps // 4)
+        with torch.cuda.stream(stream):
+            for _ in range(1 + min(args.warmup, 3)):
+                prefill_pass()
+                library_pass()
+            torch.cuda.synchronize()
+            ours, theirs = [], []
+            for _ in range(2):
+                ours.append(timed(prefill_pass, reps))
+                theirs.append(timed(library_pass, reps))
+        gms, lms = sum(ours) / len(ours), sum(theirs) / len(theirs)
+        tflops = flops / (gms * 1e-3) / 1e12
+        result["gemm"] = {"value": round(tflops, 1), "unit": "TFLOP/s", "ms_per_pass": round(gms, 4),
+                          "workload": "q4f16 g32 prefill, M=2048, the four Llama-2-7B shapes x %d layers"
+                                      % len(use),
+                          "library_f16_gemm_tflops": round(flops / (lms * 1e-3) / 1e12, 1),
+                          "library_f16_gemm_note": "torch.matmul (hipBLASLt) on float16 weights dequantized "
+                                                   "beforehand, same shapes and data, timed alternately"}
+        result["roofline_gemm"] = {"bound": "mfma", "achieved": round(tflops, 1),
+                                   "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                   "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                                   "kernel": "wq::wq_gemm_direct_kernel"}
         del wds
 
     # ---- fused residual add: O and down projections of every layer, batch 1 and 8 -------------

@@ -174,19 +174,16 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   // lines per instruction for 128 useful bytes and dominate the L1 pipeline.
   constexpr int SW = BITS == 4 ? 4 : 1;  // 32-bit words of scales per row and macro step
   uint32_t sc_cur[2][SW], sc_nxt[2][SW];
-  auto load_scales = [&](uint32_t (&sc)[2][SW], int kt0) {
-    // kt0: first step of the macro step (a multiple of 4)
-    const bool ok = kt0 < kend;
+  auto load_scales_of = [&](uint32_t (&sc)[2][SW], int kt0, auto jc) {
+    // kt0: first step of the macro step (a multiple of 4); jc: column tile
+    constexpr int j = decltype(jc)::value;
+    const uint32_t off = kt0 < kend ? sg[j] + (uint32_t)kt0 * BK / (BITS == 4 ? 32 : 128) * 2u : kStepOobD;
+    if constexpr (BITS == 4) {
+      const u32x4 v = load_b128(rs, off);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const uint32_t off = ok ? sg[j] + (uint32_t)kt0 * BK / (BITS == 4 ? 32 : 128) * 2u : kStepOobD;
-      if constexpr (BITS == 4) {
-        const u32x4 v = load_b128(rs, off);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) sc[j][q] = v[q];
-      } else {
-        sc[j][0] = load_b32(rs, off);
-      }
+      for (int q = 0; q < 4; ++q) sc[j][q] = v[q];
+    } else {
+      sc[j][0] = load_b32(rs, off);
     }
   };
   // scale of (column tile j, step t of the macro step) in the low half of a register
@@ -246,36 +243,37 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
 
   // ---- prologue ---------------------------------------------------------------------------
   // activations of step T: global -> register set T%2 late in step T-4 (one set: in step
-  // T-3), registers -> LDS stage T%4 early in step T-2, multiplied in step T;  packed weights of step T: loaded
-  // into set T%RB three steps ahead (int4), or late in step T-2 (int8, two sets).  (Step numbers below are relative to the group's first.)
+  // T-3), registers -> LDS stage T%4 early in step T-2, multiplied in step T;  packed weights
+  // of step T: loaded into set T%RB three steps ahead (four sets), or late in step T-2 (two
+  // sets).  Step numbers are relative to the K group's first step.
   u32x4 xr[XS][XL];
   RawB<BITS> rb[RB];
-  static_for_d<0, (RB == 2 ? 2 : RB - 1)>([&](auto tc) {
+  // Consumed before the loop: weights and scales of step 0, activations of steps 0 and 1.
+  static_for_d<0, PBL>([&](auto cc) { load_b(rb[0], kbase, cc); });
+  static_for_d<0, 2>([&](auto jc) { load_scales_of(sc_cur, kbase, jc); });
+  static_for_d<0, 2>([&](auto tc) {
     constexpr int T = decltype(tc)::value;
-    static_for_d<0, PBL>([&](auto cc) { load_b(rb[T], kbase + T, cc); });
+    static_for_d<0, XL>([&](auto ic) { load_x(xr[T % XS], kbase + T, ic); });
+    if constexpr (XS == 1) static_for_d<0, XL>([&](auto ic) { store_x(xr[0], (uint32_t)(T * STAGE), ic); });
   });
-  load_scales(sc_cur, kbase);
-  load_scales(sc_nxt, kbase + 4);
   if constexpr (XS == 2) {
-    static_for_d<0, 2>([&](auto tc) {
-      constexpr int T = decltype(tc)::value;
-      static_for_d<0, XL>([&](auto ic) { load_x(xr[T], kbase + T, ic); });
-    });
     static_for_d<0, 2>([&](auto tc) {
       constexpr int T = decltype(tc)::value;
       static_for_d<0, XL>([&](auto ic) { store_x(xr[T], (uint32_t)(T * STAGE), ic); });
     });
-    static_for_d<0, 2>([&](auto tc) {
-      constexpr int T = decltype(tc)::value;
-      static_for_d<0, XL>([&](auto ic) { load_x(xr[T], kbase + 2 + T, ic); });
-    });
-  } else {
-    static_for_d<0, 2>([&](auto tc) {
-      constexpr int T = decltype(tc)::value;
-      static_for_d<0, XL>([&](auto ic) { load_x(xr[0], kbase + T, ic); });
-      static_for_d<0, XL>([&](auto ic) { store_x(xr[0], (uint32_t)(T * STAGE), ic); });
-    });
+  }
+  // Still in flight at loop entry, requested in the order the loop itself requests them before
+  // its back edge: the wait counts the compiler derives for the loop head are then the
+  // steady-state ones instead of a full drain of the memory pipeline every fourth step.
+  if constexpr (RB == 4) {
+    static_for_d<0, PBL>([&](auto cc) { load_b(rb[1], kbase + 1, cc); });
     static_for_d<0, XL>([&](auto ic) { load_x(xr[0], kbase + 2, ic); });
+    static_for_d<0, PBL>([&](auto cc) { load_b(rb[2], kbase + 2, cc); });
+    static_for_d<0, XL>([&](auto ic) { load_x(xr[1], kbase + 3, ic); });
+  } else {
+    static_for_d<0, XL>([&](auto ic) { load_x(xr[0], kbase + 2, ic); });
+    if constexpr (XS == 2) static_for_d<0, XL>([&](auto ic) { load_x(xr[1], kbase + 3, ic); });
+    static_for_d<0, PBL>([&](auto cc) { load_b(rb[1], kbase + 1, cc); });
   }
   __syncthreads();
   static_for_d<0, TM>([&](auto ic) { read_a(0, a_rd[0], ic); });
@@ -347,6 +345,11 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
         // (slot NMFMA - LEAD - 3 - 1 at the latest, i.e. before the last slice)
         if constexpr (kk == 3 && j * TM + i < PBL) load_b(bcur, kt + 2, std::integral_constant<int, j * TM + i>{});
       }
+      // scales of the next macro step: requested in its first step, first used in its last
+      // (a request just before the back edge would be waited for at once: the loop-carried
+      // copy of the loaded words drains the memory pipeline)
+      if constexpr (P == 0 && kk == 2 && j * TM + i < 2)
+        load_scales_of(sc_nxt, kt + 4, std::integral_constant<int, j * TM + i>{});
       __builtin_amdgcn_sched_barrier(0);
     });
     __syncthreads();
@@ -361,7 +364,6 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int q = 0; q < SW; ++q) sc_cur[j][q] = sc_nxt[j][q];
-    load_scales(sc_nxt, kt + 8);
   }
 
   // ---- K groups: the other groups hand their partial sums to the first through LDS ---------
