@@ -77,6 +77,58 @@ def cpu_baseline(quick: bool):
              "sample": sample + ", OpenMP over output rows", "seconds": round(tn, 3)})
 
 
+def probe_mfma(torch, dev) -> int:
+    """A loop of 32x32x16 float16 MFMAs whose operands never leave registers, two wavefronts per
+    SIMD, about 30 ms per launch: the rate depends on the operand values only."""
+    import ctypes
+
+    so = os.path.join(ROOT, "relax_amd", "csrc", "libmi355x_probe.so")
+    if not os.path.exists(so):
+        raise ImportError(f"{so} is missing: build it with `make -C relax_amd/csrc all`")
+    fn = ctypes.CDLL(so).mi355x_probe_mfma_f16
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    blocks, iters = 512, 40000
+    shape = (blocks, 8, 256 * 8)  # [:, :4] A fragments, [:, 4:] B fragments
+    out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+
+    def q4_like():
+        t = torch.randn(shape, device=dev)
+        w = torch.randint(0, 16, (blocks, 4, 256 * 8), device=dev).float() - 7.0
+        sc = (torch.rand((blocks, 4, 256 * 8), device=dev) * 0.015 + 0.005).half().float()
+        t[:, 4:] = w * sc
+        return t
+
+    cases = [
+        ("zeros", lambda: torch.zeros(shape, device=dev)),
+        ("ones", lambda: torch.ones(shape, device=dev)),
+        ("A ~ N(0,1), B = (u{0..15} - 7) * 2^-7", lambda: torch.cat(
+            [torch.randn((blocks, 4, 256 * 8), device=dev),
+             (torch.randint(0, 16, (blocks, 4, 256 * 8), device=dev).float() - 7.0) / 128.0], dim=1)),
+        ("A ~ N(0,1), B = (u{0..15} - 7) * s, s ~ U(0.005, 0.02): the benchmark's weights", q4_like),
+        ("A, B ~ N(0,1)", lambda: torch.randn(shape, device=dev)),
+    ]
+    flops = blocks * 4 * iters * 16 * 32768.0
+    for name, make in cases:
+        ops = make().to(torch.float16).contiguous()
+        rc = fn(ops.data_ptr(), out.data_ptr(), blocks, iters // 10, None)  # warm-up
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc |= fn(ops.data_ptr(), out.data_ptr(), blocks, iters, None)
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            best = ms if best is None else min(best, ms)
+        if rc != 0:
+            raise RuntimeError(f"probe launch failed with HIP error {rc}")
+        print(json.dumps({"probe": "mfma_f32_32x32x16_f16, operands in registers", "operands": name,
+                          "ms": round(best, 2), "tflops": round(flops / best / 1e9, 0),
+                          "frac_of_peak": round(flops / best / 1e9 / MFMA_F16_PEAK_TFLOPS, 3)}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -89,6 +141,10 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times (a kernel of known HBM "
                          "traffic, used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--probe-mfma", action="store_true",
+                    help="instead of the benchmark: time a register-resident float16 MFMA loop on operands "
+                         "of several distributions (what the matrix pipes sustain as a function of the data "
+                         "alone) and print one line per distribution")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the hot path is a single-GPU kernel and this build has no "
@@ -104,6 +160,9 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     torch.manual_seed(0)
+
+    if args.probe_mfma:
+        return probe_mfma(torch, dev)
 
     if args.calibrate_copy:
         src = torch.ones(64 * 1024 * 1024, dtype=torch.int32, device=dev)  # 256 MiB read + 256 MiB written

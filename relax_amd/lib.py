@@ -47,7 +47,7 @@ _lib = None
 
 def build(verbose: bool = False) -> str:
     """Compile the library for gfx950 in-tree (hipcc cross-compiles without a GPU)."""
-    cmd = ["make", "-B", "-j8", "-C", CSRC, "libmi355x_wq.so"]
+    cmd = ["make", "-B", "-j8", "-C", CSRC, "all"]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if verbose or res.returncode != 0:
         print(res.stdout)
