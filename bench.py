@@ -77,6 +77,61 @@ def cpu_baseline(quick: bool):
              "sample": sample + ", OpenMP over output rows", "seconds": round(tn, 3)})
 
 
+LLAMA13B = [("qkv", 15360, 5120), ("o", 5120, 5120), ("gate_up", 27648, 5120), ("down", 5120, 13824)]
+
+
+def config_table(torch, dev, args) -> int:
+    """Every (M, N, K) of the parity configurations timed alone: q4f16 g32 at the 7B shapes for
+    M in {1, 8, 512, 2048}, q8f16 g128 at the 13B shapes for M in {1, 16, 256}.  Each case rotates
+    through enough distinct weight sets (> 512 MB in total) that no launch finds its weights in a
+    cache, inside one HIP graph; the time is the graph's divided by its launches."""
+    import relax_amd
+    from relax_amd import lib
+
+    cases = [(4, 32, m, n, k) for m in (1, 8, 512, 2048) for _, n, k in LLAMA7B]
+    cases += [(8, 128, m, n, k) for m in (1, 16, 256) for _, n, k in LLAMA13B]
+    stream = torch.cuda.Stream()
+    for bits, group, m, n, k in cases:
+        wbytes = n * k * bits // 8 + n * (k // group) * 2
+        sets = max(2, -(-(512 << 20) // wbytes) + 1)
+        ws = [(torch.randint(-2**31, 2**31 - 1, (n, k * bits // 32), dtype=torch.int32, device=dev),
+               (torch.rand((n, k // group), device=dev) * (0.015 if bits == 4 else 0.008)
+                + (0.005 if bits == 4 else 0.002)).to(torch.float16)) for _ in range(sets)]
+        x = torch.randn((m, k), device=dev).to(torch.float16)
+        y = torch.empty((m, n), dtype=torch.float16, device=dev)
+
+        def one_pass():
+            for wq, s in ws:
+                relax_amd.wq_matmul(x, wq, s, bits, group, out=y)
+
+        with torch.cuda.stream(stream):
+            one_pass()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                one_pass()
+            g.replay()
+            torch.cuda.synchronize()
+            reps = max(3, min(args.steps, 2000 // sets))
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(reps):
+                g.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * sets)
+        ab = algorithmic_bytes(bits, group, m, n, k)
+        fl = 2.0 * m * n * k
+        line = {"case": "q%df16 g%d M=%d N=%d K=%d" % (bits, group, m, n, k), "us": round(us, 2),
+                "kernel": {lib.KERNEL_GEMV: "gemv", lib.KERNEL_SKINNY: "skinny", lib.KERNEL_GEMM: "gemm"}[
+                    lib.load().mi355x_wq_select_kernel(lib.make_desc(bits, group, n, k), m)],
+                "GB/s": round(ab / us / 1e3, 0), "frac_hbm": round(ab / us / 1e3 / HBM_PEAK_GBS, 3),
+                "TFLOP/s": round(fl / us / 1e6, 1), "frac_mfma": round(fl / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 3)}
+        print(json.dumps(line), flush=True)
+        del ws, g
+    return 0
+
+
 def probe_mfma(torch, dev) -> int:
     """A loop of 32x32x16 float16 MFMAs whose operands never leave registers, two wavefronts per
     SIMD, about 30 ms per launch: the rate depends on the operand values only."""
@@ -141,6 +196,10 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times (a kernel of known HBM "
                          "traffic, used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--configs", action="store_true",
+                    help="instead of the benchmark: time every shape of the decode, prefill and q8f16 "
+                         "configurations on its own (weights rotated through more than 512 MB, one HIP "
+                         "graph per case) and print one line per case")
     ap.add_argument("--probe-mfma", action="store_true",
                     help="instead of the benchmark: time a register-resident float16 MFMA loop on operands "
                          "of several distributions (what the matrix pipes sustain as a function of the data "
@@ -163,6 +222,8 @@ def main() -> int:
 
     if args.probe_mfma:
         return probe_mfma(torch, dev)
+    if args.configs:
+        return config_table(torch, dev, args)
 
     if args.calibrate_copy:
         src = torch.ones(64 * 1024 * 1024, dtype=torch.int32, device=dev)  # 256 MiB read + 256 MiB written

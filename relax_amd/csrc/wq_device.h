@@ -142,4 +142,33 @@ __device__ __forceinline__ void store_out(const Epilogue& ep, half_t* y, int m, 
   y[idx] = h;
 }
 
+// Whether rows of y (and of the epilogue operands) can be written two adjacent columns at a
+// time with 4-byte accesses: even row length and 4-byte aligned bases (the C ABI only asks for
+// 2-byte alignment of y, bias and residual).
+__device__ __forceinline__ bool pair_store_ok(const Epilogue& ep, const half_t* y, int N) {
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(ep.bias) |
+                         reinterpret_cast<uintptr_t>(ep.residual);
+  return ((N & 1) == 0) && ((bits & 3u) == 0);
+}
+
+// Columns n (even) and n + 1 of row m; `paired` comes from pair_store_ok.  Same per-element
+// arithmetic as store_out.
+__device__ __forceinline__ void store_out2(const Epilogue& ep, half_t* y, int m, int n, int N, float a0, float a1,
+                                           bool paired) {
+  if (paired && n + 1 < N) {
+    half2_t h = half2_t{(half_t)a0, (half_t)a1};
+    const size_t idx = (size_t)m * N + n;
+    if (ep.bias != nullptr) h = h + *reinterpret_cast<const half2_t*>(ep.bias + n);
+    if (ep.activation == 1) {
+      h[0] = h[0] > (half_t)0 ? h[0] : (half_t)0;
+      h[1] = h[1] > (half_t)0 ? h[1] : (half_t)0;
+    }
+    if (ep.residual != nullptr) h = h + *reinterpret_cast<const half2_t*>(ep.residual + idx);
+    *reinterpret_cast<half2_t*>(y + idx) = h;
+  } else {
+    if (n < N) store_out(ep, y, m, n, N, a0);
+    if (n + 1 < N) store_out(ep, y, m, n + 1, N, a1);
+  }
+}
+
 }  // namespace wq

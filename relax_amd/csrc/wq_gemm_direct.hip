@@ -81,8 +81,8 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   // register sets: two wavefronts per SIMD leave 128 VGPRs beside the accumulators and hide
   // latency by themselves, so the K-group variants prefetch only one step deep (deeper rings
   // were measured with the 64-row tile, where registers would allow them: no gain)
-  constexpr int RB = (BITS == 4 && GROUPS == 1) ? 4 : 2;  // packed weights
-  constexpr int XS = GROUPS == 1 ? 2 : 1;                 // activations
+  constexpr int RB = (TM == 2 || (BITS == 4 && GROUPS == 1)) ? 4 : 2;  // packed weights
+  constexpr int XS = (TM == 2 || GROUPS == 1) ? 2 : 1;                 // activations
   static_assert(XL >= 1 && XL <= 2 * TM, "activation chunks per thread must fit the MFMA slots of one k slice");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char wq_gemm_direct_smem[];
@@ -139,7 +139,9 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   uint32_t wg[2], sg[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const int n = min(n0 + wave * 64 + j * 32 + fr, N - 1);  // rows past N: computed, not stored
+    // column tile j of the MFMA holds the tile's columns of parity j (lane fr: column 2 fr + j), so
+    // that a lane ends up with two adjacent outputs of a row and a wavefront stores whole 128-byte lines
+    const int n = min(n0 + wave * 64 + 2 * fr + j, N - 1);  // rows past N: computed, not stored
     wg[j] = (uint32_t)n * row_bytes + (uint32_t)fh * (32u * BITS / 8);
     sg[j] = (uint32_t)n * groups_per_row * 2u;
   }
@@ -405,17 +407,15 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     if (grp != 0) return;
   }
 
-  // ---- epilogue: lane holds column (lane % 32) and rows 8*(v/4) + 4*(lane/32) + v%4 ------
+  // ---- epilogue: lane holds columns 2 (lane % 32), + 1 and rows 8*(v/4) + 4*(lane/32) + v%4 ------
+  const bool paired = pair_store_ok(ep, y, N);
+  const int n = n0 + wave * 64 + 2 * fr;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int n = n0 + wave * 64 + j * 32 + fr;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m0 + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
-        if (m < M && n < N) store_out(ep, y, m, n, N, acc[i][j][v]);
-      }
+    for (int v = 0; v < 16; ++v) {
+      const int m = m0 + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
+      if (m < M) store_out2(ep, y, m, n, N, acc[i][0][v], acc[i][1][v], paired);
     }
 }
 

@@ -421,6 +421,39 @@ def test_fused_residual_in_place(bits, m, n, k):
     assert np.array_equal(h.cpu().numpy().view(np.uint16), separate.view(np.uint16))
 
 
+@pytest.mark.parametrize("variant", [21, 22, 23, 24, 25])
+@pytest.mark.parametrize("n,shift", [(521, 0), (520, 1), (64, 1), (129, 1)])
+def test_gemm_output_pairs_fall_back_when_rows_or_bases_are_not_4_byte_aligned(variant, n, shift):
+    """The direct-weight GEMM writes two adjacent columns per lane with one 4-byte access; with an
+    odd row length, or y / bias / residual that start on an odd float16, it must write (and read
+    the epilogue operands) element by element -- same bits either way."""
+    import relax_amd
+    from relax_amd import lib
+
+    bits, m, k = 4, 130, 1280
+    x, wq, s, g = O.make_case(950 + n + shift, m, n, k, bits)
+    bias, res = _fused_operands(n + shift, m, n)
+    want_plain = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
+
+    def shifted(a):  # a device copy of `a` that starts `shift` float16 into its allocation
+        flat = torch.empty(a.size + shift, dtype=torch.float16, device="cuda")
+        view = flat[shift:].view(a.shape)
+        view.copy_(torch.from_numpy(a))
+        return view
+
+    xd, wd, sd = _dev(x), _dev(wq), _dev(s)
+    y_plain = shifted(np.zeros((m, n), np.float16))
+    relax_amd.wq_matmul(xd, wd, sd, bits, g, kernel=lib.KERNEL_GEMM, variant=variant, out=y_plain)
+    y_fused = shifted(np.zeros((m, n), np.float16))
+    relax_amd.wq_matmul(xd, wd, sd, bits, g, kernel=lib.KERNEL_GEMM, variant=variant, out=y_fused,
+                        bias=shifted(bias), activation="relu", residual=shifted(res))
+    torch.cuda.synchronize()
+    assert y_plain.data_ptr() % 4 == (2 * shift) % 4
+    got_plain, got = y_plain.cpu().numpy(), y_fused.cpu().numpy()
+    assert_close(got_plain, want_plain, (variant, n, shift))
+    assert_fused(got, got_plain, want_plain, bias, "relu", res, (variant, n, shift))
+
+
 def test_fused_special_values_follow_the_cpu_rules():
     """relu(-0) = +0, an overflowing bias add gives inf, inf + (-inf) residual gives NaN."""
     m, n, k = 2, 32, 64
