@@ -410,6 +410,50 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   // ---- epilogue: lane holds columns 2 (lane % 32), + 1 and rows 8*(v/4) + 4*(lane/32) + v%4 ------
   const bool paired = pair_store_ok(ep, y, N);
   const int n = n0 + wave * 64 + 2 * fr;
+  if (paired && m0 + BM <= M && n0 + WAVES * 64 <= N) {
+    // Tile inside the matrix, 4-byte accesses allowed: the tail's shape is decided once, outside the
+    // unrolled stores (per-element tests of the three epilogue fields cost more than the stores).
+    half_t* const y0 = y + (size_t)(m0 + fh * 4) * N + n;
+    auto store_tile = [&](auto has_bias, auto relu, auto has_res) {
+      half2_t b2 = half2_t{(half_t)0, (half_t)0};
+      if constexpr (decltype(has_bias)::value) b2 = *reinterpret_cast<const half2_t*>(ep.bias + n);
+      const half_t* const r0 = decltype(has_res)::value ? ep.residual + (size_t)(m0 + fh * 4) * N + n : nullptr;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          half2_t res[4];
+          if constexpr (decltype(has_res)::value) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              res[e] = *reinterpret_cast<const half2_t*>(r0 + (size_t)(i * 32 + g * 8 + e) * N);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            half2_t h = half2_t{(half_t)acc[i][0][g * 4 + e], (half_t)acc[i][1][g * 4 + e]};
+            if constexpr (decltype(has_bias)::value) h = h + b2;
+            if constexpr (decltype(relu)::value) {
+              h[0] = h[0] > (half_t)0 ? h[0] : (half_t)0;
+              h[1] = h[1] > (half_t)0 ? h[1] : (half_t)0;
+            }
+            if constexpr (decltype(has_res)::value) h = h + res[e];
+            *reinterpret_cast<half2_t*>(y0 + (size_t)(i * 32 + g * 8 + e) * N) = h;
+          }
+        }
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    const bool hb = ep.bias != nullptr, hr = ep.residual != nullptr, ra = ep.activation == 1;
+    if (!hb && !ra && !hr) store_tile(F{}, F{}, F{});
+    else if (hb && !ra && !hr) store_tile(T{}, F{}, F{});
+    else if (hb && ra && !hr) store_tile(T{}, T{}, F{});
+    else if (!hb && !ra && hr) store_tile(F{}, F{}, T{});
+    else if (hb && !ra && hr) store_tile(T{}, F{}, T{});
+    else if (hb && ra && hr) store_tile(T{}, T{}, T{});
+    else if (!hb && ra && !hr) store_tile(F{}, T{}, F{});
+    else store_tile(F{}, T{}, T{});
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
