@@ -267,17 +267,26 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void wq_gemm_pipe_kernel(
   }
 
   // ---- epilogue: lane holds column (lane % 32) and rows 8*(v/4) + 4*(lane/32) + v%4 ---
+  // the tail's shape is tested once, not per element
+  const bool plain = ep.bias == nullptr && ep.residual == nullptr && ep.activation == 0;
+  auto store_tiles = [&](auto plain_c) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = n0 + wn * (BN / WN) + j * 32 + fr;
+      for (int j = 0; j < TN; ++j) {
+        const int n = n0 + wn * (BN / WN) + j * 32 + fr;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm * (BM / WM) + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
-        if (m < M && n < N) store_out(ep, y, m, n, N, acc[i][j][v]);
+        for (int v = 0; v < 16; ++v) {
+          const int m = m0 + wm * (BM / WM) + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
+          if (m < M && n < N) {
+            if constexpr (decltype(plain_c)::value) y[(size_t)m * N + n] = (half_t)acc[i][j][v];
+            else store_out(ep, y, m, n, N, acc[i][j][v]);
+          }
+        }
       }
-    }
+  };
+  if (plain) store_tiles(std::true_type{});
+  else store_tiles(std::false_type{});
 }
 
 namespace {
