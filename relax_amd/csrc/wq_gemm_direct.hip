@@ -250,33 +250,35 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   // sets).  Step numbers are relative to the K group's first step.
   u32x4 xr[XS][XL];
   RawB<BITS> rb[RB];
-  // Consumed before the loop: weights and scales of step 0, activations of steps 0 and 1.
+  // Every request of the prologue goes out before the first wait (one memory round trip, not one
+  // per dependent step).  First what is consumed before the loop: weights and scales of step 0,
+  // activations of steps 0 and 1 (in registers of their own: the loop's sets already receive the
+  // steps after them).
+  u32x4 xp[2][XL];
   static_for_d<0, PBL>([&](auto cc) { load_b(rb[0], kbase, cc); });
   static_for_d<0, 2>([&](auto jc) { load_scales_of(sc_cur, kbase, jc); });
   static_for_d<0, 2>([&](auto tc) {
     constexpr int T = decltype(tc)::value;
-    static_for_d<0, XL>([&](auto ic) { load_x(xr[T % XS], kbase + T, ic); });
-    if constexpr (XS == 1) static_for_d<0, XL>([&](auto ic) { store_x(xr[0], (uint32_t)(T * STAGE), ic); });
+    static_for_d<0, XL>([&](auto ic) { load_x(xp[T], kbase + T, ic); });
   });
-  if constexpr (XS == 2) {
-    static_for_d<0, 2>([&](auto tc) {
-      constexpr int T = decltype(tc)::value;
-      static_for_d<0, XL>([&](auto ic) { store_x(xr[T], (uint32_t)(T * STAGE), ic); });
-    });
-  }
-  // Still in flight at loop entry, requested in the order the loop itself requests them before
-  // its back edge: the wait counts the compiler derives for the loop head are then the
+  // Then what is still in flight at loop entry, requested in the order the loop itself requests
+  // it before its back edge: the wait counts the compiler derives for the loop head are then the
   // steady-state ones instead of a full drain of the memory pipeline every fourth step.
   if constexpr (RB == 4) {
     static_for_d<0, PBL>([&](auto cc) { load_b(rb[1], kbase + 1, cc); });
     static_for_d<0, XL>([&](auto ic) { load_x(xr[0], kbase + 2, ic); });
     static_for_d<0, PBL>([&](auto cc) { load_b(rb[2], kbase + 2, cc); });
-    static_for_d<0, XL>([&](auto ic) { load_x(xr[1], kbase + 3, ic); });
+    if constexpr (XS == 2) static_for_d<0, XL>([&](auto ic) { load_x(xr[1], kbase + 3, ic); });
   } else {
     static_for_d<0, XL>([&](auto ic) { load_x(xr[0], kbase + 2, ic); });
     if constexpr (XS == 2) static_for_d<0, XL>([&](auto ic) { load_x(xr[1], kbase + 3, ic); });
     static_for_d<0, PBL>([&](auto cc) { load_b(rb[1], kbase + 1, cc); });
   }
+  __builtin_amdgcn_sched_barrier(0);
+  static_for_d<0, 2>([&](auto tc) {
+    constexpr int T = decltype(tc)::value;
+    static_for_d<0, XL>([&](auto ic) { store_x(xp[T], (uint32_t)(T * STAGE), ic); });
+  });
   __syncthreads();
   static_for_d<0, TM>([&](auto ic) { read_a(0, a_rd[0], ic); });
 #pragma unroll

@@ -81,6 +81,16 @@ def test_kernel_selection_by_rows():
     assert L.mi355x_wq_select_kernel(d, 17) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(d, 64) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(d, 65) == lib.KERNEL_GEMM
+    # 17..64 rows on wide projections: the GEMM's 64x128 tile costs the same for any row count, the
+    # skinny kernel grows with it
+    wide, mid = lib.make_desc(4, 32, 22016, 4096), lib.make_desc(4, 32, 12288, 4096)
+    assert L.mi355x_wq_select_kernel(wide, 23) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(wide, 24) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(mid, 32) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(mid, 33) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 27648, 5120), 24) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 15360, 5120), 48) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 22016, 4000), 48) == lib.KERNEL_SKINNY  # K % 256 != 0
     assert L.mi355x_wq_select_kernel(d, -1) == -1
 
 
