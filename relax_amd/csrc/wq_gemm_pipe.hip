@@ -19,9 +19,9 @@
 // previous barrier and one barrier per step suffices.
 //
 // LDS layout per stage: activations [BM][64] then weights [BN][64] float16, rows of
-// 128 bytes whose eight 16-byte chunks are XOR-swizzled with (row & 7): the
-// 16-byte operand reads of 8 consecutive lanes (8 consecutive rows, same chunk)
-// then cover all banks exactly once, without padding.
+// 128 bytes whose eight 16-byte chunks are XOR-swizzled with ((row >> 1) & 7): the
+// 16-byte operand reads of 16 consecutive lanes (16 consecutive rows, same chunk)
+// then cover all 64 banks exactly once, without padding.
 //
 // Shape requirements (checked by the launcher; other shapes use the generic GEMM
 // kernel): K a multiple of 64, every operand below 1 GiB.
@@ -101,8 +101,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void wq_gemm_pipe_kernel(
     const int m = m0 + x_row0 + i * (NT / 8);
     xg[i] = m < M ? (uint32_t)m * (uint32_t)K * 2u + (uint32_t)x_c * 16u : kRowOob;
   }
-  // NT/8 is a multiple of 8, so the swizzle term is the same for every i
-  const uint32_t x_lds = (uint32_t)x_row0 * 128u + (uint32_t)((x_c ^ (x_row0 & 7)) << 4);
+  // NT/8 is a multiple of 16, so the swizzle term is the same for every i
+  const uint32_t x_lds = (uint32_t)x_row0 * 128u + (uint32_t)((x_c ^ ((x_row0 >> 1) & 7)) << 4);
 
   uint32_t wg[WL], sg[WL], w_lds[WL][WPC];
   int w_kofs[WL];  // k offset of the packed chunk inside the step
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void wq_gemm_pipe_kernel(
 #pragma unroll
     for (int j = 0; j < WPC; ++j) {
       const int chunk = q * WPC + j;
-      w_lds[i][j] = (uint32_t)BM * 128u + (uint32_t)row * 128u + (uint32_t)((chunk ^ (row & 7)) << 4);
+      w_lds[i][j] = (uint32_t)BM * 128u + (uint32_t)row * 128u + (uint32_t)((chunk ^ ((row >> 1) & 7)) << 4);
     }
   }
 
@@ -126,7 +126,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void wq_gemm_pipe_kernel(
   uint32_t a_rd[4], b_rd[4];
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) {
-    const uint32_t swz = (uint32_t)(((kk * 2 + fh) ^ (fr & 7)) << 4);
+    const uint32_t swz = (uint32_t)(((kk * 2 + fh) ^ ((fr >> 1) & 7)) << 4);
     a_rd[kk] = (uint32_t)(wm * (BM / WM) + fr) * 128u + swz;
     b_rd[kk] = (uint32_t)BM * 128u + (uint32_t)(wn * (BN / WN) + fr) * 128u + swz;
   }
