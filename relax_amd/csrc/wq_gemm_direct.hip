@@ -85,7 +85,7 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   // latency by themselves, so the K-group variants prefetch only one step deep (deeper rings
   // were measured with the 64-row tile, where registers would allow them: no gain)
   constexpr int RB = (TM == 2 || (BITS == 4 && GROUPS == 1)) ? 4 : 2;  // packed weights
-  constexpr int XS = (TM == 2 || GROUPS == 1) ? 2 : 1;                 // activations
+  constexpr int XS = (TM == 2 || GROUPS == 1) ? 2 : 1;  // activations (1, 2 or 4; four sets measured: no gain)
   static_assert(XL >= 1 && XL <= 2 * TM, "activation chunks per thread must fit the MFMA slots of one k slice");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char wq_gemm_direct_smem[];
@@ -247,7 +247,7 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   // ---- prologue ---------------------------------------------------------------------------
-  // activations of step T: global -> register set T%2 late in step T-4 (one set: in step
+  // activations of step T: global -> register set T%XS late in step T-2-XS (one set: in step
   // T-3), registers -> LDS stage T%4 early in step T-2, multiplied in step T;  packed weights
   // of step T: loaded into set T%RB three steps ahead (four sets), or late in step T-2 (two
   // sets).  Step numbers are relative to the K group's first step.
@@ -269,12 +269,17 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   // steady-state ones instead of a full drain of the memory pipeline every fourth step.
   if constexpr (RB == 4) {
     static_for_d<0, PBL>([&](auto cc) { load_b(rb[1], kbase + 1, cc); });
-    static_for_d<0, XL>([&](auto ic) { load_x(xr[0], kbase + 2, ic); });
+    static_for_d<0, XL>([&](auto ic) { load_x(xr[2 % XS], kbase + 2, ic); });
     static_for_d<0, PBL>([&](auto cc) { load_b(rb[2], kbase + 2, cc); });
-    if constexpr (XS == 2) static_for_d<0, XL>([&](auto ic) { load_x(xr[1], kbase + 3, ic); });
+    static_for_d<3, 2 + XS>([&](auto tc) {
+      constexpr int T = decltype(tc)::value;
+      static_for_d<0, XL>([&](auto ic) { load_x(xr[T % XS], kbase + T, ic); });
+    });
   } else {
-    static_for_d<0, XL>([&](auto ic) { load_x(xr[0], kbase + 2, ic); });
-    if constexpr (XS == 2) static_for_d<0, XL>([&](auto ic) { load_x(xr[1], kbase + 3, ic); });
+    static_for_d<2, 2 + XS>([&](auto tc) {
+      constexpr int T = decltype(tc)::value;
+      static_for_d<0, XL>([&](auto ic) { load_x(xr[T % XS], kbase + T, ic); });
+    });
     static_for_d<0, PBL>([&](auto cc) { load_b(rb[1], kbase + 1, cc); });
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -338,9 +343,10 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
         read_a((kk + 1) & 1, a_rd[(kk + 1) & 3] + (kk == 3 ? st_next : st_rd), std::integral_constant<int, i>{});
       // activations: registers -> LDS (step kt+2), then the same registers <- global (step kt+4)
       constexpr int sq = 2 * TM - 1 - (j * TM + i);  // slot index inside the slice, from its end
-      if constexpr (kk == 0 && sq < XL) store_x(xr[P % XS], st_wr, std::integral_constant<int, sq>{});
-      if constexpr (XS == 2) {
-        if constexpr (kk == 2 && sq < XL) load_x(xr[P & 1], kt + 4, std::integral_constant<int, sq>{});
+      // (the activations of step s live in register set s % XS)
+      if constexpr (kk == 0 && sq < XL) store_x(xr[(P + 2) % XS], st_wr, std::integral_constant<int, sq>{});
+      if constexpr (XS >= 2) {
+        if constexpr (kk == 2 && sq < XL) load_x(xr[(P + 2) % XS], kt + 2 + XS, std::integral_constant<int, sq>{});
       } else {
         if constexpr (kk == 1 && sq < XL) load_x(xr[0], kt + 3, std::integral_constant<int, sq>{});
       }
