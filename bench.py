@@ -133,18 +133,19 @@ def config_table(torch, dev, args) -> int:
 
 
 def probe_mfma(torch, dev) -> int:
-    """A loop of 32x32x16 float16 MFMAs whose operands never leave registers, two wavefronts per
-    SIMD, about 30 ms per launch: the rate depends on the operand values only."""
+    """A loop of 32x32x16 float16 MFMAs whose operands never leave registers, one wavefront per
+    SIMD, about 10 - 15 ms per launch: the rate depends on the operand values only."""
     import ctypes
 
     so = os.path.join(ROOT, "relax_amd", "csrc", "libmi355x_probe.so")
     if not os.path.exists(so):
         raise ImportError(f"{so} is missing: build it with `make -C relax_amd/csrc all`")
     fn = ctypes.CDLL(so).mi355x_probe_mfma_f16
-    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
-    blocks, iters = 512, 40000
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    blocks, iters = 256, 40000
     shape = (blocks, 8, 256 * 8)  # [:, :4] A fragments, [:, 4:] B fragments
     out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
 
     def q4_like():
         t = torch.randn(shape, device=dev)
@@ -165,22 +166,25 @@ def probe_mfma(torch, dev) -> int:
     flops = blocks * 4 * iters * 16 * 32768.0
     for name, make in cases:
         ops = make().to(torch.float16).contiguous()
-        rc = fn(ops.data_ptr(), out.data_ptr(), blocks, iters // 10, None)  # warm-up
+        rc = fn(ops.data_ptr(), out.data_ptr(), blocks, iters // 10, clocks.data_ptr(), None)  # warm-up
         torch.cuda.synchronize()
         best = None
         for _ in range(3):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            rc |= fn(ops.data_ptr(), out.data_ptr(), blocks, iters, None)
+            rc |= fn(ops.data_ptr(), out.data_ptr(), blocks, iters, clocks.data_ptr(), None)
             e1.record()
             torch.cuda.synchronize()
             ms = e0.elapsed_time(e1)
-            best = ms if best is None else min(best, ms)
+            if best is None or ms < best:
+                best, (cyc, ref) = ms, clocks.tolist()
         if rc != 0:
             raise RuntimeError(f"probe launch failed with HIP error {rc}")
         print(json.dumps({"probe": "mfma_f32_32x32x16_f16, operands in registers", "operands": name,
                           "ms": round(best, 2), "tflops": round(flops / best / 1e9, 0),
-                          "frac_of_peak": round(flops / best / 1e9 / MFMA_F16_PEAK_TFLOPS, 3)}), flush=True)
+                          "frac_of_peak": round(flops / best / 1e9 / MFMA_F16_PEAK_TFLOPS, 3),
+                          "cycles_per_mfma": round(cyc / (iters * 16.0), 2),
+                          "shader_clock_ghz": round(cyc / (ref * 10.0), 3)}), flush=True)
     return 0
 
 
