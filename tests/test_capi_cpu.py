@@ -37,6 +37,16 @@ def test_library_exports_every_declared_symbol():
     assert sorted(exported) == sorted(names)
 
 
+def test_measurement_probe_library_is_built_and_separate():
+    """bench.py --probe-mfma loads its kernel from a library of its own; the product library has
+    no symbol of it."""
+    probe = os.path.join(os.path.dirname(lib.SO_PATH), "libmi355x_probe.so")
+    assert os.path.exists(probe), "make -C relax_amd/csrc all"
+    out = subprocess.run(["nm", "-D", "--defined-only", probe], capture_output=True, text=True).stdout
+    assert [l.split()[-1] for l in out.splitlines() if " T " in l] == ["mi355x_probe_mfma_f16"]
+    assert not hasattr(lib.load(), "mi355x_probe_mfma_f16")
+
+
 @pytest.mark.parametrize("kw,msg", [
     (dict(bits=5), "bits must be 4 or 8"),
     (dict(group=48), "group must be 32 times a power of two"),
