@@ -108,6 +108,35 @@ MI355X_WQ_API int mi355x_wq_matmul_fused_ex(const mi355x_wq_desc* desc, const vo
 MI355X_WQ_API int mi355x_wq_dequantize(const mi355x_wq_desc* desc, const void* wq, const void* scales, void* wd,
                          void* stream);
 
+/* Tile-major weight layout: a one-off permutation of the bytes of `wq` and `scales` into the order
+ * in which the decode kernel consumes them -- for each tile of 16 rows and each 128 bytes of a row,
+ * two blocks of 1 KB in which lane l of a wavefront owns bytes 16 l .. 16 l + 15 -- so that every
+ * load instruction of the weight stream reads 1 KB contiguously.  The canonical row-major layout stays
+ * the interchange format; this is what a parameter-preparation function run once at load time
+ * produces (the reference's counterpart is a `relax.layout_transform` / packing PrimFunc applied to
+ * the weights before they are bound: python/tvm/relax/op/manipulate.py:113-151,
+ * python/tvm/relax/transform/transform.py:210-233).  Defined for the two benchmark quantizations:
+ * int4 / group 32 with K % 256 == 0 and int8 / group 128 with K % 128 == 0.  Both tiled buffers
+ * have the size of the canonical ones with N rounded up to a multiple of 16 (rows past N are zero).
+ * Tiling followed by untiling returns the input bit for bit, and the matmul computes the same
+ * values in the same order from either layout (bit-identical outputs). */
+MI355X_WQ_API int mi355x_wq_tiled_sizes(const mi355x_wq_desc* desc, int64_t* wq_bytes, int64_t* scales_bytes);
+
+/* canonical (wq, scales) -> tile-major (wq_tiled, scales_tiled); all four 16-byte aligned, device. */
+MI355X_WQ_API int mi355x_wq_tile_weights(const mi355x_wq_desc* desc, const void* wq, const void* scales,
+                                        void* wq_tiled, void* scales_tiled, void* stream);
+
+/* tile-major -> canonical (the inverse; used to hand the weights back in the interchange format). */
+MI355X_WQ_API int mi355x_wq_untile_weights(const mi355x_wq_desc* desc, const void* wq_tiled, const void* scales_tiled,
+                                          void* wq, void* scales, void* stream);
+
+/* mi355x_wq_matmul_fused on tile-major weights (`ep` may be NULL).  M <= 16 runs the decode
+ * kernel on the contiguous stream; larger M runs the direct-weight GEMM with tile-major
+ * addressing and needs K % 256 == 0. */
+MI355X_WQ_API int mi355x_wq_matmul_tiled(const mi355x_wq_desc* desc, const void* x, const void* wq_tiled,
+                                        const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y,
+                                        int64_t m, void* stream);
+
 /* Validates a descriptor and a row count without touching the GPU: 0 if
  * mi355x_wq_matmul would accept them. */
 MI355X_WQ_API int mi355x_wq_check(const mi355x_wq_desc* desc, int64_t m);

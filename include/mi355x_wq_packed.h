@@ -103,6 +103,22 @@ MI355X_WQ_API int mi355x_q8f16_dequantize(mi355x_tvm_value* args, int* type_code
                             mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
                             void* resource_handle);
 
+/* Tile-major weight layout (mi355x_wq_tile_weights / mi355x_wq_matmul_tiled in mi355x_wq.h) as
+ * destination-passing externs, the way a parameter-preparation function and the model's main
+ * function would call them (R.call_tir with one or two outputs: src/relax/transform/call_tir_rewrite.cc:94-110):
+ *   tile_weights(wq[N, K*bits/32] u32, scales[N, K/group] f16, wq_tiled[Np, K*bits/32] u32, scales_tiled[Np, K/group] f16)
+ *   matmul_tiled(x[M, K] f16, wq_tiled[Np, ...], scales_tiled[Np, ...], y[M, N] f16)
+ * with Np = N rounded up to a multiple of 16: the tile-major buffers are declared as tensors of the
+ * canonical shape with whole tiles of rows (N itself comes from y). */
+MI355X_WQ_API int mi355x_q4f16_tile_weights(mi355x_tvm_value* args, int* type_codes, int num_args,
+                              mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
+MI355X_WQ_API int mi355x_q8f16_tile_weights(mi355x_tvm_value* args, int* type_codes, int num_args,
+                              mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
+MI355X_WQ_API int mi355x_q4f16_matmul_tiled(mi355x_tvm_value* args, int* type_codes, int num_args,
+                              mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
+MI355X_WQ_API int mi355x_q8f16_matmul_tiled(mi355x_tvm_value* args, int* type_codes, int num_args,
+                              mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
+
 /*
  * Per-symbol call description for generated entries.  FuseOpsByPattern orders the
  * parameters of a composite function by first use

@@ -163,9 +163,70 @@ int mi355x_wq_select_kernel(const mi355x_wq_desc* desc, int64_t m) {
   return wq::select_kernel(desc, m);
 }
 
+namespace {
+
+int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
+                      const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int kernel, bool tiled);
+
+}  // namespace
+
 int mi355x_wq_matmul_fused_ex(const mi355x_wq_desc* desc, const void* x, const void* wq_,
                               const void* scales, const mi355x_wq_epilogue* ep, void* y, int64_t m,
                               void* stream, int kernel) {
+  return matmul_any_layout(desc, x, wq_, scales, ep, y, m, stream, kernel, false);
+}
+
+int mi355x_wq_matmul_tiled(const mi355x_wq_desc* desc, const void* x, const void* wq_tiled,
+                           const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y, int64_t m,
+                           void* stream) {
+  return matmul_any_layout(desc, x, wq_tiled, scales_tiled, ep, y, m, stream, MI355X_WQ_KERNEL_AUTO, true);
+}
+
+int mi355x_wq_tiled_sizes(const mi355x_wq_desc* desc, int64_t* wq_bytes, int64_t* scales_bytes) {
+  using namespace wq;
+  if (!check_desc(desc, 0)) return -1;
+  if (!tiled_layout_defined(desc->bits, desc->group, desc->k)) {
+    set_error("tile-major layout: needs int4 / group 32 with K %% 256 == 0 or int8 / group 128 with K %% 128 == 0, "
+              "got bits=%d group=%d K=%lld", desc->bits, desc->group, (long long)desc->k);
+    return -1;
+  }
+  const int64_t rows = (desc->n + 15) / 16 * 16;
+  if (wq_bytes != nullptr) *wq_bytes = rows * (desc->k * desc->bits / 8);
+  if (scales_bytes != nullptr) *scales_bytes = rows * (desc->k / desc->group) * 2;
+  return 0;
+}
+
+namespace {
+
+int tile_or_untile(const mi355x_wq_desc* desc, const void* wq_src, const void* scales_src, void* wq_dst,
+                   void* scales_dst, void* stream, bool forward) {
+  using namespace wq;
+  if (!check_desc(desc, 0)) return -1;
+  if (desc->n == 0 || desc->k == 0) return 0;
+  if (!check_ptr(wq_src, forward ? "wq" : "wq_tiled", 16) || !check_ptr(scales_src, forward ? "scales" : "scales_tiled", 16) ||
+      !check_ptr(wq_dst, forward ? "wq_tiled" : "wq", 16) || !check_ptr(scales_dst, forward ? "scales_tiled" : "scales", 16))
+    return -1;
+  Problem p{nullptr, wq_src, scales_src, nullptr, 0, desc->n, desc->k, desc->bits, desc->group,
+            desc->zero_point, static_cast<hipStream_t>(stream)};
+  return launch_tile_weights(p, wq_dst, scales_dst, forward);
+}
+
+}  // namespace
+
+int mi355x_wq_tile_weights(const mi355x_wq_desc* desc, const void* wq_, const void* scales, void* wq_tiled,
+                           void* scales_tiled, void* stream) {
+  return tile_or_untile(desc, wq_, scales, wq_tiled, scales_tiled, stream, true);
+}
+
+int mi355x_wq_untile_weights(const mi355x_wq_desc* desc, const void* wq_tiled, const void* scales_tiled, void* wq_,
+                             void* scales, void* stream) {
+  return tile_or_untile(desc, wq_tiled, scales_tiled, wq_, scales, stream, false);
+}
+
+namespace {
+
+int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
+                      const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int kernel, bool tiled) {
   using namespace wq;
   if (!check_desc(desc, m)) return -1;
   if (ep != nullptr) {
@@ -198,6 +259,16 @@ int mi355x_wq_matmul_fused_ex(const mi355x_wq_desc* desc, const void* x, const v
     p.residual = ep->residual;
     p.activation = ep->activation;
   }
+  if (tiled) {
+    if (!tiled_layout_defined(desc->bits, desc->group, desc->k)) {
+      set_error("tile-major layout: needs int4 / group 32 with K %% 256 == 0 or int8 / group 128 with "
+                "K %% 128 == 0, got bits=%d group=%d K=%lld", desc->bits, desc->group, (long long)desc->k);
+      return -1;
+    }
+    p.tiled = true;
+    // the decode kernel up to 16 rows (while its LDS plan fits), the direct-weight GEMM beyond
+    return gemv_applicable(p) ? launch_gemv(p, 0) : launch_gemm(p, 0);
+  }
   int chosen = family == MI355X_WQ_KERNEL_AUTO ? select_kernel(desc, m) : family;
   switch (chosen) {
     case MI355X_WQ_KERNEL_GEMV: return launch_gemv(p, variant);
@@ -206,6 +277,8 @@ int mi355x_wq_matmul_fused_ex(const mi355x_wq_desc* desc, const void* x, const v
     default: set_error("unknown kernel family %d", family); return -1;
   }
 }
+
+}  // namespace
 
 int mi355x_wq_matmul_fused(const mi355x_wq_desc* desc, const void* x, const void* wq_,
                            const void* scales, const mi355x_wq_epilogue* ep, void* y, int64_t m,

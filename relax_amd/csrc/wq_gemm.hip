@@ -218,7 +218,25 @@ int launch_gemm(const Problem& p, int variant) {
     set_error("gemm kernel: group %d must be %d times a power of two", p.group, ch);
     return -1;
   }
-  if (variant == 0 && gemm_pipe_applicable(p)) {
+  if (p.tiled) {
+    // only the direct-weight kernel addresses the tile-major layout
+    const int64_t tiles128 = ((p.m + 127) / 128) * ((p.n + 255) / 256);
+    const int64_t tiles64x128 = ((p.m + 63) / 64) * ((p.n + 127) / 128);
+    const int first = tiles128 <= cu_count() / 2 ? 4 : 2;
+    bool ok = false;
+    if (variant == 0)
+      ok = (tiles64x128 <= cu_count() && launch_gemm_direct(p, group_shift, 5)) ||
+           launch_gemm_direct(p, group_shift, first) || launch_gemm_direct(p, group_shift, first - 1);
+    else if (variant >= 21)
+      ok = launch_gemm_direct(p, group_shift, variant - 20);
+    if (!ok) {
+      set_error("gemm kernel: tile-major weights need the direct-weight kernel (K %% 256 == 0, operands below "
+                "1 GiB; variant 0 or 21..25), got M=%lld N=%lld K=%lld variant=%d", (long long)p.m,
+                (long long)p.n, (long long)p.k, variant);
+      return -1;
+    }
+    variant = -1;
+  } else if (variant == 0 && gemm_pipe_applicable(p)) {
     // Measured on MI355X, M = 128 .. 4096 on the Llama shapes: the direct-weight kernel with two
     // K groups wins wherever it applies -- with 64-row tiles while 128-row tiles would leave
     // half of the CUs without one; next the same kernel with one group (K below 512), then the

@@ -66,7 +66,7 @@ struct RawB {
   u32x4 w[2][NV];                               // [column tile][load]
 };
 
-template <int BITS, int GROUPS, int TM, int WAVES>
+template <int BITS, int GROUPS, int TM, int WAVES, bool TILED>
 __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
     half_t* y, int M, int N, int K, int group_shift, int zero_point, int tiles_m, int tiles_n,
@@ -124,8 +124,11 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
 
   const uint32_t row_bytes = (uint32_t)K * BITS / 8;
   const uint32_t groups_per_row = ((uint32_t)K / CH) >> group_shift;
-  const rsrc_t rw = make_rsrc(wq, (uint32_t)N * row_bytes);
-  const rsrc_t rs = make_rsrc(scales, (uint32_t)N * groups_per_row * 2u);
+  // (tile-major buffers hold whole 16-row tiles, zero filled past N)
+  const uint32_t n_stored = TILED ? ((uint32_t)N + 15u) / 16u * 16u : (uint32_t)N;
+  const uint32_t nsuper = row_bytes / 128u;  // 128-byte super steps per weight row (tile-major addressing)
+  const rsrc_t rw = make_rsrc(wq, n_stored * row_bytes);
+  const rsrc_t rs = make_rsrc(scales, n_stored * groups_per_row * 2u);
   const rsrc_t rx = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
 
   // ---- activations: global offsets and LDS store address of this thread ---------------
@@ -144,9 +147,17 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   for (int j = 0; j < 2; ++j) {
     // column tile j of the MFMA holds the tile's columns of parity j (lane fr: column 2 fr + j), so
     // that a lane ends up with two adjacent outputs of a row and a wavefront stores whole 128-byte lines
-    const int n = min(n0 + wave * 64 + 2 * fr + j, N - 1);  // rows past N: computed, not stored
-    wg[j] = (uint32_t)n * row_bytes + (uint32_t)fh * (32u * BITS / 8);
-    sg[j] = (uint32_t)n * groups_per_row * 2u;
+    const int n = min(n0 + wave * 64 + 2 * fr + j, (int)n_stored - 1);  // rows past N: computed, not stored
+    if constexpr (TILED) {
+      // chunk c of row n sits at ((tile*S + c/8)*2 + c%2)*1024 + ((c%8)/2*16 + n%16)*16; the lane's chunks
+      // of step kt are 2 kt + fh (int4) or 4 kt + 2 fh + v (int8), which leaves these lane constants
+      const uint32_t tile = (uint32_t)n >> 4, col = (uint32_t)n & 15u;
+      wg[j] = tile * nsuper * 2048u + (uint32_t)fh * (BITS == 4 ? 1024u : 256u) + col * 16u;
+      sg[j] = BITS == 4 ? (tile * nsuper * 64u + col) * 4u : (tile * nsuper * 16u + col) * 2u;
+    } else {
+      wg[j] = (uint32_t)n * row_bytes + (uint32_t)fh * (32u * BITS / 8);
+      sg[j] = (uint32_t)n * groups_per_row * 2u;
+    }
   }
 
   // ---- A fragment read addresses: row fr, chunk fh*4 + kk ------------------------------
@@ -169,8 +180,14 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   // piece c of the packed-weight loads of step kt
   auto load_b = [&](RawB<BITS>& b, int kt, auto cc) {
     constexpr int c = decltype(cc)::value, j = c / NV, v = c % NV;
-    const uint32_t k0 = (uint32_t)kt * BK;
-    b.w[j][v] = load_b128(rw, wg[j] + (kt < kend ? k0 * BITS / 8 : kStepOobD) + v * 16u);
+    if constexpr (TILED) {
+      const uint32_t ukt = (uint32_t)kt;
+      const uint32_t step = BITS == 4 ? (ukt >> 2) * 2048u + (ukt & 3u) * 256u : (ukt >> 1) * 2048u + (ukt & 1u) * 512u;
+      b.w[j][v] = load_b128(rw, wg[j] + (kt < kend ? step : kStepOobD) + v * 1024u);
+    } else {
+      const uint32_t k0 = (uint32_t)kt * BK;
+      b.w[j][v] = load_b128(rw, wg[j] + (kt < kend ? k0 * BITS / 8 : kStepOobD) + v * 16u);
+    }
   };
   constexpr int PBL = 2 * NV;  // packed-weight load pieces per step
 
@@ -182,6 +199,19 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   auto load_scales_of = [&](uint32_t (&sc)[2][SW], int kt0, auto jc) {
     // kt0: first step of the macro step (a multiple of 4); jc: column tile
     constexpr int j = decltype(jc)::value;
+    if constexpr (TILED) {
+      if constexpr (BITS == 4) {
+        // the eight scales of (row, super step) are four 4-byte pairs, one per kq, 64 bytes apart
+        const uint32_t base = kt0 < kend ? sg[j] + ((uint32_t)kt0 >> 2) * 256u : kStepOobD;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sc[j][q] = load_b32(rs, base + (uint32_t)q * 64u);
+      } else {
+        // one float16 per (row, super step); a macro step of 256 k spans two of them
+        const uint32_t base = kt0 < kend ? sg[j] + ((uint32_t)kt0 >> 1) * 32u : kStepOobD;
+        sc[j][0] = load_b16(rs, base) | (load_b16(rs, base + 32u) << 16);
+      }
+      return;
+    }
     const uint32_t off = kt0 < kend ? sg[j] + (uint32_t)kt0 * BK / (BITS == 4 ? 32 : 128) * 2u : kStepOobD;
     if constexpr (BITS == 4) {
       const u32x4 v = load_b128(rs, off);
@@ -476,7 +506,7 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
 
 namespace {
 
-template <int BITS, int GROUPS, int TM, int WAVES>
+template <int BITS, int GROUPS, int TM, int WAVES, bool TILED>
 bool launch_direct(const Problem& p, int group_shift) {
   constexpr int BM = TM * 32, BN = WAVES * 64;
   const int tiles_m = (int)((p.m + BM - 1) / BM);
@@ -487,9 +517,9 @@ bool launch_direct(const Problem& p, int group_shift) {
   constexpr size_t lds_bytes = stages > exchange ? stages : exchange;
   static_assert(lds_bytes <= 160 * 1024, "LDS per workgroup");
   static bool lds_ok[kMaxDevices] = {false};
-  if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES>, (int)lds_bytes, lds_ok))
+  if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED>, (int)lds_bytes, lds_ok))
     return false;
-  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES>), grid, block, lds_bytes, p.stream,
+  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
                      tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
@@ -498,8 +528,11 @@ bool launch_direct(const Problem& p, int group_shift) {
 
 template <int GROUPS, int TM, int WAVES>
 bool launch_bits(const Problem& p, int group_shift) {
-  return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES>(p, group_shift)
-                     : launch_direct<8, GROUPS, TM, WAVES>(p, group_shift);
+  if (p.tiled)
+    return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES, true>(p, group_shift)
+                       : launch_direct<8, GROUPS, TM, WAVES, true>(p, group_shift);
+  return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES, false>(p, group_shift)
+                     : launch_direct<8, GROUPS, TM, WAVES, false>(p, group_shift);
 }
 
 }  // namespace

@@ -56,7 +56,7 @@ struct GemvArgs {
   Epilogue ep;
 };
 
-template <int BITS, int WAVES, int D, int SPL>
+template <int BITS, int WAVES, int D, int SPL, bool TILED>
 // (scalar kernel arguments instead of one struct: the first 16 dwords -- the operand pointers
 // and the shape -- are preloaded into SGPRs at wavefront launch, which takes the argument fetch
 // out of the start-up latency of a 5 - 15 us kernel)
@@ -83,6 +83,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
   constexpr int NJ = CH / 8;      // MFMAs per lane load
   constexpr int NT = WAVES * 64;
   static_assert(SPL == 1 || SPL == D, "one scale per super step, or one per chunk");
+  static_assert(!TILED || D == 2, "the tile-major layout is written for super steps of eight chunks");
   static_assert(SPL == 1 || (SPL % 2 == 0 && SPL <= 8), "scale vector is 4, 8 or 16 bytes");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -98,8 +99,10 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
   const uint32_t row_bytes = (uint32_t)K * BITS / 8;
   const int nchunks = K / CH;
   const uint32_t groups_per_row = (uint32_t)nchunks >> a.group_shift;
-  const rsrc_t rw = make_rsrc(a.wq, (uint32_t)N * row_bytes);
-  const rsrc_t rs = make_rsrc(a.scales, (uint32_t)N * groups_per_row * 2u);
+  // (the tile-major buffers hold whole tiles: rows up to the next multiple of 16, zero filled)
+  const uint32_t n_stored = TILED ? (uint32_t)a.tiles * 16u : (uint32_t)N;
+  const rsrc_t rw = make_rsrc(a.wq, n_stored * row_bytes);
+  const rsrc_t rs = make_rsrc(a.scales, n_stored * groups_per_row * 2u);
   const rsrc_t rx = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
 
   const int G = gridDim.x;
@@ -110,6 +113,21 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
 
   // weights of (tile index i, super step ss of the current phase) -> registers
   auto load_super = [&](GemvBuf<D, SPL>& b, int i, int ss, int chunk_base, int ss_end) {
+    if constexpr (TILED) {
+      // Tile-major stream: the D 1 KB blocks of (tile, super step) are consecutive and lane l owns
+      // bytes 16 l .. 16 l + 15 of each -- every load instruction of the wavefront reads 1 KB
+      // contiguously.  Scales: int4 / group 32 one 4-byte pair per lane, int8 / group 128 one
+      // float16 per (row, super step).
+      const uint32_t nsuper_all = (uint32_t)nchunks / (4 * D);
+      const uint32_t item = (uint32_t)(blockIdx.x + i * G) * nsuper_all + (uint32_t)(chunk_base / (4 * D) + ss);
+      const bool ok = (i < my_tiles) && (ss < ss_end) && (chunk_base + ss * 4 * D < nchunks);
+      const uint32_t woff = ok ? item * (D * 1024u) + (uint32_t)lane * 16u : kOobOffset;
+#pragma unroll
+      for (int d = 0; d < D; ++d) b.w[d] = load_b128(rw, woff + d * 1024u);
+      if constexpr (SPL == 1) b.sc[0] = load_b16(rs, ok ? (item * 16u + (uint32_t)col) * 2u : kOobOffset);
+      else b.sc[0] = load_b32(rs, ok ? (item * 64u + (uint32_t)lane) * 4u : kOobOffset);
+      return;
+    }
     const int n = min((int)(blockIdx.x + i * G) * 16 + col, N - 1);  // rows past N: computed, not stored
     const int chunk0 = chunk_base + ss * 4 * D + kq * D;
     // D > 1 is only launched when K is a multiple of 4*D chunks, so a lane's D
@@ -327,7 +345,7 @@ bool make_plan(const Problem& p, int wgs_per_cu, Plan* out) {
 // the kernel was launched, or a runtime call failed (error already set).
 enum { kNotApplicable = 0, kLaunched = 1, kFailed = -1 };
 
-template <int BITS, int WAVES, int D, int SPL>
+template <int BITS, int WAVES, int D, int SPL, bool TILED = false>
 int launch_one(const Problem& p, int group_shift, const Plan& plan) {
   GemvArgs a;
   a.x = (const half_t*)p.x;
@@ -345,9 +363,9 @@ int launch_one(const Problem& p, int group_shift, const Plan& plan) {
   a.phase_chunks = plan.phase_chunks;
   a.ep = Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation};
   static bool lds_ok[kMaxDevices] = {false};
-  if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL>, (int)kLdsPerWgMax, lds_ok))
+  if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED>, (int)kLdsPerWgMax, lds_ok))
     return kFailed;
-  hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL>), dim3(plan.grid), dim3(WAVES * 64),
+  hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED>), dim3(plan.grid), dim3(WAVES * 64),
                      plan.lds_bytes, p.stream, a.x, a.wq, a.scales, a.y, a.M, a.N, a.K, a.group_shift,
                      a.zero_point, a.lds_stride, a.tiles, a.max_tiles, a.phase_chunks, a.ep);
   return kLaunched;
@@ -361,6 +379,15 @@ int try_launch(const Problem& p, int group_shift, int wgs_per_cu) {
   if (D > 1 && p.k % (4 * D * ch) != 0) return kNotApplicable;
   Plan plan;
   if (!make_plan<BITS, WAVES, D>(p, wgs_per_cu, &plan)) return kNotApplicable;
+  if (p.tiled) {
+    // only the layout's own shape: super steps of eight chunks, scales per chunk (int4 / group 32)
+    // or per super step (int8 / group 128)
+    if constexpr (D == 2) {
+      if (BITS == 4 && group_shift == 0) return launch_one<BITS, WAVES, 2, 2, true>(p, group_shift, plan);
+      if (BITS == 8 && group_shift == 3) return launch_one<BITS, WAVES, 2, 1, true>(p, group_shift, plan);
+    }
+    return kNotApplicable;
+  }
   if (group_shift == 0) return launch_one<BITS, WAVES, D, D>(p, group_shift, plan);
   if ((1 << group_shift) >= D) return launch_one<BITS, WAVES, D, 1>(p, group_shift, plan);
   return kNotApplicable;
@@ -437,8 +464,11 @@ bool gemv_applicable(const Problem& p) {
   while ((1 << gs) < ratio) ++gs;
   if (ratio < 1 || (1 << gs) != ratio) return false;
   const int* order = default_order(p);
-  for (int q = 0; q < 4; ++q)
+  for (int q = 0; q < 4; ++q) {
+    const int shape = order[q] % 10;
+    if (p.tiled && shape != 2 && shape != 5 && shape != 8) continue;  // tile-major: two-chunk super steps only
     if (p.bits == 4 ? variant_has_plan<4>(p, gs, order[q]) : variant_has_plan<8>(p, gs, order[q])) return true;
+  }
   return false;
 }
 

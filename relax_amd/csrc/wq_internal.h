@@ -17,6 +17,8 @@ struct Problem {
   const void* bias = nullptr;
   const void* residual = nullptr;
   int activation = 0;  // 0 none, 1 relu
+  // wq / scales are in the tile-major layout written by launch_tile_weights (see wq_tiled.hip)
+  bool tiled = false;
 };
 
 // Tuning variant: 0 = library default for the shape, >0 = explicit choice
@@ -29,6 +31,11 @@ bool gemm_pipe_applicable(const Problem& p);  // K % 64 == 0, operands below 1 G
 bool launch_gemm_pipe(const Problem& p, int group_shift, int variant);
 bool launch_gemm_direct(const Problem& p, int group_shift, int variant);
 int launch_dequant(const Problem& p, void* wd);
+// canonical -> tile-major (forward) or back; p.wq / p.scales are the source, p.y is unused
+int launch_tile_weights(const Problem& p, void* wq_out, void* scales_out, bool forward);
+// K and (bits, group) for which the tile-major layout is defined: int4 / group 32 with K % 256 == 0,
+// int8 / group 128 with K % 128 == 0
+bool tiled_layout_defined(int bits, int group, int64_t k);
 
 // Upper bound of rows the skinny family accepts.
 constexpr int64_t kSkinnyMaxM = 64;

@@ -284,6 +284,83 @@ MI355X_FIXED_ENTRY(mi355x_q4f16_dequantize, 1, 4, 7, 0, 0, 0)
 MI355X_FIXED_ENTRY(mi355x_q8f16_dequantize, 1, 8, 0, 0, 0, 0)
 #undef MI355X_FIXED_ENTRY
 
+// ---- tile-major layout: the one-off transform and the matmul on its output ----------------
+// tile_weights(wq[N,K*bits/32], scales[N,K/group], wq_tiled[Np,K*bits/32], scales_tiled[Np,K/group])
+// matmul_tiled(x[M,K], wq_tiled[Np,...], scales_tiled[Np,...], y[M,N]) with Np = N rounded up to 16:
+// the tile-major buffers are passed as tensors of the canonical shape with whole tiles of rows.
+static int packed_tiled(bool is_matmul, int bits, int zero_point, mi355x_tvm_value* args, int* type_codes,
+                        int num_args) {
+  if (num_args != 4 || args == nullptr || type_codes == nullptr) {
+    wq::set_error("%s expects 4 tensor arguments, got %d", is_matmul ? "matmul_tiled" : "tile_weights", num_args);
+    return fail();
+  }
+  const int iw = is_matmul ? 1 : 0, is = is_matmul ? 2 : 1;  // the weight / scale tensor that fixes K and group
+  const mi355x_dl_tensor *t0 = nullptr, *tw = nullptr, *ts = nullptr, *t3 = nullptr, *t2 = nullptr;
+  void *p0 = nullptr, *pw = nullptr, *ps = nullptr, *p3 = nullptr, *p2 = nullptr;
+  if (!take_tensor(args, type_codes, iw, is_matmul ? "wq_tiled" : "wq", kU32, -1, &tw, &pw)) return fail();
+  const int dev = tw->device.device_id;
+  if (!take_tensor(args, type_codes, is, is_matmul ? "scales_tiled" : "scales", kF16, dev, &ts, &ps)) return fail();
+  mi355x_wq_desc d;
+  memset(&d, 0, sizeof(d));
+  d.bits = bits;
+  d.zero_point = zero_point;
+  d.k = tw->shape[1] * (32 / bits);
+  if (ts->shape[0] != tw->shape[0] || ts->shape[1] <= 0 || d.k % ts->shape[1] != 0) {
+    wq::set_error("scales shape (%lld, %lld) does not match weights of %lld rows and K=%lld", (long long)ts->shape[0],
+                  (long long)ts->shape[1], (long long)tw->shape[0], (long long)d.k);
+    return fail();
+  }
+  d.group = (int32_t)(d.k / ts->shape[1]);
+  int64_t m = 0;
+  if (is_matmul) {
+    if (!take_tensor(args, type_codes, 0, "x", kF16, dev, &t0, &p0)) return fail();
+    if (!take_tensor(args, type_codes, 3, "y", kF16, dev, &t3, &p3)) return fail();
+    m = t0->shape[0];
+    d.n = t3->shape[1];
+    if (t0->shape[1] != d.k || t3->shape[0] != m || tw->shape[0] != (d.n + 15) / 16 * 16) {
+      wq::set_error("matmul_tiled: x (%lld, %lld), tiled weights of %lld rows and K=%lld, y (%lld, %lld) do not fit "
+                    "(tiled rows must be N rounded up to 16)", (long long)t0->shape[0], (long long)t0->shape[1],
+                    (long long)tw->shape[0], (long long)d.k, (long long)t3->shape[0], (long long)t3->shape[1]);
+      return fail();
+    }
+  } else {
+    d.n = tw->shape[0];
+    if (!take_tensor(args, type_codes, 2, "wq_tiled", kU32, dev, &t2, &p2)) return fail();
+    if (!take_tensor(args, type_codes, 3, "scales_tiled", kF16, dev, &t3, &p3)) return fail();
+    const int64_t np = (d.n + 15) / 16 * 16;
+    if (t2->shape[0] != np || t2->shape[1] != tw->shape[1] || t3->shape[0] != np || t3->shape[1] != ts->shape[1]) {
+      wq::set_error("tile_weights: outputs must have the input shapes with %lld rows (N rounded up to 16)",
+                    (long long)np);
+      return fail();
+    }
+  }
+  if (mi355x_wq_check(&d, m) != 0) return fail();
+  if (d.n == 0 || (is_matmul && m == 0)) return 0;
+  int cur = -1;
+  if (hipGetDevice(&cur) != hipSuccess) {
+    (void)hipGetLastError();
+    wq::set_error("no usable HIP device in this process");
+    return fail();
+  }
+  if (cur != dev) {
+    wq::set_error("tensors live on ROCm device %d but the current HIP device is %d", dev, cur);
+    return fail();
+  }
+  const int rc = is_matmul ? mi355x_wq_matmul_tiled(&d, p0, pw, ps, nullptr, p3, m, g_stream)
+                           : mi355x_wq_tile_weights(&d, pw, ps, p2, p3, g_stream);
+  return rc == 0 ? 0 : fail();
+}
+
+#define MI355X_TILED_ENTRY(NAME, IS_MATMUL, BITS, ZP)                                               \
+  int NAME(mi355x_tvm_value* args, int* type_codes, int num_args, mi355x_tvm_value*, int*, void*) { \
+    return packed_tiled(IS_MATMUL, BITS, ZP, args, type_codes, num_args);                           \
+  }
+MI355X_TILED_ENTRY(mi355x_q4f16_tile_weights, false, 4, 7)
+MI355X_TILED_ENTRY(mi355x_q8f16_tile_weights, false, 8, 0)
+MI355X_TILED_ENTRY(mi355x_q4f16_matmul_tiled, true, 4, 7)
+MI355X_TILED_ENTRY(mi355x_q8f16_matmul_tiled, true, 8, 0)
+#undef MI355X_TILED_ENTRY
+
 // ---- registration in TVM's global table through its C API -----------------------
 typedef int (*backend_fn_t)(mi355x_tvm_value*, int*, int, mi355x_tvm_value*, int*, void*);
 
@@ -318,7 +395,11 @@ int mi355x_wq_register_tvm_globals(int allow_override) {
                            {"mi355x.q4f16_matmul_residual", mi355x_q4f16_matmul_residual},
                            {"mi355x.q8f16_matmul_residual", mi355x_q8f16_matmul_residual},
                            {"mi355x.q4f16_dequantize", mi355x_q4f16_dequantize},
-                           {"mi355x.q8f16_dequantize", mi355x_q8f16_dequantize}};
+                           {"mi355x.q8f16_dequantize", mi355x_q8f16_dequantize},
+                           {"mi355x.q4f16_tile_weights", mi355x_q4f16_tile_weights},
+                           {"mi355x.q8f16_tile_weights", mi355x_q8f16_tile_weights},
+                           {"mi355x.q4f16_matmul_tiled", mi355x_q4f16_matmul_tiled},
+                           {"mi355x.q8f16_matmul_tiled", mi355x_q8f16_matmul_tiled}};
   int count = 0;
   for (const Entry& e : entries) {
     void* handle = nullptr;

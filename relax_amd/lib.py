@@ -16,11 +16,13 @@ ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "relax.nn.rel
 EXPORTED_SYMBOLS = (
     "mi355x_wq_matmul", "mi355x_wq_matmul_ex", "mi355x_wq_matmul_fused", "mi355x_wq_matmul_fused_ex",
     "mi355x_wq_dequantize", "mi355x_wq_check",
+    "mi355x_wq_tiled_sizes", "mi355x_wq_tile_weights", "mi355x_wq_untile_weights", "mi355x_wq_matmul_tiled",
     "mi355x_wq_select_kernel", "mi355x_wq_last_error", "mi355x_wq_version",
     "mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_matmul_bias", "mi355x_q8f16_matmul_bias",
     "mi355x_q4f16_matmul_bias_relu", "mi355x_q8f16_matmul_bias_relu", "mi355x_q4f16_matmul_residual",
     "mi355x_q8f16_matmul_residual", "mi355x_q4f16_dequantize",
-    "mi355x_q8f16_dequantize", "mi355x_wq_packed_call", "mi355x_wq_packed_set_stream",
+    "mi355x_q8f16_dequantize", "mi355x_q4f16_tile_weights", "mi355x_q8f16_tile_weights",
+    "mi355x_q4f16_matmul_tiled", "mi355x_q8f16_matmul_tiled", "mi355x_wq_packed_call", "mi355x_wq_packed_set_stream",
     "mi355x_wq_packed_get_stream", "mi355x_wq_register_tvm_globals",
 )
 PACKED_ENTRIES = tuple(s for s in EXPORTED_SYMBOLS if s.startswith(("mi355x_q4f16_", "mi355x_q8f16_")))
@@ -67,12 +69,16 @@ def load() -> C.CDLL:
     L = C.CDLL(SO_PATH)
     vp, i64, ci = C.c_void_p, C.c_int64, C.c_int
     dp = C.POINTER(WqDesc)
+    ep = C.POINTER(WqEpilogue)
     L.mi355x_wq_matmul.argtypes = [dp, vp, vp, vp, vp, i64, vp]
     L.mi355x_wq_matmul_ex.argtypes = [dp, vp, vp, vp, vp, i64, vp, ci]
-    ep = C.POINTER(WqEpilogue)
     L.mi355x_wq_matmul_fused.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp]
     L.mi355x_wq_matmul_fused_ex.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp, ci]
     L.mi355x_wq_dequantize.argtypes = [dp, vp, vp, vp, vp]
+    L.mi355x_wq_tiled_sizes.argtypes = [dp, C.POINTER(i64), C.POINTER(i64)]
+    L.mi355x_wq_tile_weights.argtypes = [dp, vp, vp, vp, vp, vp]
+    L.mi355x_wq_untile_weights.argtypes = [dp, vp, vp, vp, vp, vp]
+    L.mi355x_wq_matmul_tiled.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp]
     L.mi355x_wq_check.argtypes = [dp, i64]
     L.mi355x_wq_select_kernel.argtypes = [dp, i64]
     L.mi355x_wq_last_error.restype = C.c_char_p

@@ -21,11 +21,18 @@ def _as_u32_storage(wq: torch.Tensor) -> torch.Tensor:
 def wq_matmul(x: torch.Tensor, wq: torch.Tensor, scales: torch.Tensor, bits: int, group: int,
               zero_point: int | None = None, out: torch.Tensor | None = None, kernel: int = 0,
               variant: int = 0, stream=None, bias: torch.Tensor | None = None,
-              activation: str | None = None, residual: torch.Tensor | None = None) -> torch.Tensor:
+              activation: str | None = None, residual: torch.Tensor | None = None,
+              tiled_n: int | None = None) -> torch.Tensor:
     """y[M,N] = f16(x[M,K] @ dequant(wq, scales)^T) on the current HIP device (asynchronous).
 
     Optional fused epilogue, each step one float16 operation: ``+ bias[N]``, then ``activation``
-    ("relu"), then ``+ residual[M,N]`` (``residual`` may be ``out`` itself)."""
+    ("relu"), then ``+ residual[M,N]`` (``residual`` may be ``out`` itself).
+
+    ``tiled_n=N``: ``wq`` and ``scales`` are the tile-major buffers `wq_tile_weights` returns
+    for an N-row matrix (their row count is N rounded up to 16)."""
+    if tiled_n is not None:
+        return _wq_matmul_tiled(x, wq, scales, bits, group, tiled_n, zero_point, out, stream, bias,
+                                activation, residual)
     L = _lib.load()
     wq = _as_u32_storage(wq)
     if not (x.is_cuda and wq.is_cuda and scales.is_cuda):
@@ -66,6 +73,77 @@ def wq_matmul(x: torch.Tensor, wq: torch.Tensor, scales: torch.Tensor, bits: int
     rc = L.mi355x_wq_matmul_fused_ex(desc, x.data_ptr(), wq.data_ptr(), scales.data_ptr(), ep,
                                      out.data_ptr(), m, _stream_ptr(stream), kernel | (variant << 8))
     _lib.check(rc)
+    return out
+
+
+def _tiled_sizes(L, desc):
+    import ctypes as C
+
+    wb, sb = C.c_int64(0), C.c_int64(0)
+    _lib.check(L.mi355x_wq_tiled_sizes(desc, C.byref(wb), C.byref(sb)))
+    return wb.value, sb.value
+
+
+def wq_tile_weights(wq: torch.Tensor, scales: torch.Tensor, bits: int, group: int,
+                    stream=None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Canonical (wq[N, K*bits/32], scales[N, K/group]) -> the tile-major buffers of
+    `mi355x_wq_tile_weights`, as tensors of the canonical shapes with N rounded up to 16 rows (their
+    bytes are in tile-major order, not row-major).  A one-off, done when weights are loaded."""
+    L = _lib.load()
+    wq = _as_u32_storage(wq)
+    if not (wq.is_cuda and scales.is_cuda and wq.is_contiguous() and scales.is_contiguous()):
+        raise ValueError("wq and scales must be compact device tensors")
+    n, k = wq.shape[0], wq.shape[1] * (32 // bits)
+    if scales.dtype != torch.float16 or tuple(scales.shape) != (n, k // group):
+        raise ValueError(f"scales must be float16 of shape {(n, k // group)}")
+    desc = _lib.make_desc(bits, group, n, k)
+    wb, sb = _tiled_sizes(L, desc)
+    rows = (n + 15) // 16 * 16  # whole tiles; same row length as the canonical tensors
+    wq_t = torch.empty((rows, wq.shape[1]), dtype=torch.int32, device=wq.device)
+    s_t = torch.empty((rows, scales.shape[1]), dtype=torch.float16, device=wq.device)
+    assert wq_t.numel() * 4 == wb and s_t.numel() * 2 == sb
+    _lib.check(L.mi355x_wq_tile_weights(desc, wq.data_ptr(), scales.data_ptr(), wq_t.data_ptr(), s_t.data_ptr(),
+                                        _stream_ptr(stream)))
+    return wq_t, s_t
+
+
+def wq_untile_weights(wq_tiled: torch.Tensor, scales_tiled: torch.Tensor, bits: int, group: int, n: int, k: int,
+                      stream=None) -> tuple[torch.Tensor, torch.Tensor]:
+    """The inverse of `wq_tile_weights`: back to the canonical interchange layout."""
+    L = _lib.load()
+    desc = _lib.make_desc(bits, group, n, k)
+    wb, sb = _tiled_sizes(L, desc)
+    if wq_tiled.numel() * wq_tiled.element_size() != wb or scales_tiled.numel() * scales_tiled.element_size() != sb:
+        raise ValueError(f"tile-major buffers must hold {wb} and {sb} bytes")
+    wq = torch.empty((n, k * bits // 32), dtype=torch.int32, device=wq_tiled.device)
+    s = torch.empty((n, k // group), dtype=torch.float16, device=wq_tiled.device)
+    _lib.check(L.mi355x_wq_untile_weights(desc, wq_tiled.data_ptr(), scales_tiled.data_ptr(), wq.data_ptr(),
+                                          s.data_ptr(), _stream_ptr(stream)))
+    return wq, s
+
+
+def _wq_matmul_tiled(x, wq_t, s_t, bits, group, n, zero_point, out, stream, bias, activation, residual):
+    L = _lib.load()
+    if not (x.is_cuda and wq_t.is_cuda and s_t.is_cuda):
+        raise ValueError("x, wq and scales must be device tensors")
+    if x.dtype != torch.float16 or s_t.dtype != torch.float16 or not x.is_contiguous():
+        raise TypeError("x and scales must be float16, x compact")
+    m, k = x.shape
+    desc = _lib.make_desc(bits, group, n, k, zero_point)
+    wb, sb = _tiled_sizes(L, desc)
+    if wq_t.numel() * wq_t.element_size() != wb or s_t.numel() * s_t.element_size() != sb:
+        raise ValueError(f"tile-major buffers must hold {wb} and {sb} bytes for N={n}, K={k}")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    elif tuple(out.shape) != (m, n) or out.dtype != torch.float16 or not out.is_contiguous():
+        raise ValueError("out must be a compact float16 [M, N] tensor")
+    if activation not in _lib.ACTIVATIONS:
+        raise ValueError(f"unsupported activation {activation!r}")
+    ep = _lib.WqEpilogue(bias.data_ptr() if bias is not None else None,
+                         residual.data_ptr() if residual is not None else None,
+                         _lib.ACTIVATIONS[activation], 0)
+    _lib.check(L.mi355x_wq_matmul_tiled(desc, x.data_ptr(), wq_t.data_ptr(), s_t.data_ptr(), ep, out.data_ptr(), m,
+                                        _stream_ptr(stream)))
     return out
 
 
