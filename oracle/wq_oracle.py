@@ -211,6 +211,50 @@ def wq_matmul_fused(x, wq, s, bits: int, group: int, bias=None, activation: str 
     return epilogue(wq_matmul(x, wq, s, bits, group), bias, activation, residual)
 
 
+# ---------------------------------------------------------------- tile-major weight layout
+# No counterpart in the reference (its weights stay row-major): the definition below is this
+# build's own, restated with explicit loops so that the device transform has something
+# independent to be compared with.  Chunk = 16 bytes of a weight row, super step = 8 chunks,
+# tile = 16 rows; S = super steps per row.
+#   weights: chunk (row t*16 + col, index s*8 + kq*2 + d) -> 16 bytes at ((t*S + s)*2 + d)*1024 + (kq*16 + col)*16
+#   scales : int4 / group 32 -> float16 at (((t*S + s)*64 + kq*16 + col)*2 + e)*2 for group s*8 + kq*2 + e
+#            int8 / group 128 -> float16 at ((t*S + s)*16 + col)*2 for group s
+def tile_weights(wq: np.ndarray, s: np.ndarray, bits: int):
+    """Canonical (wq [N, K*bits/32] uint32, scales [N, K/group] float16) -> tile-major arrays of the same
+    shapes with N rounded up to 16 rows (bytes in tile-major order; rows past N are zero)."""
+    n, words = wq.shape
+    nsuper = words * 4 // 128
+    assert words * 4 % 128 == 0 and s.shape == (n, nsuper * (8 if bits == 4 else 1))
+    tiles = (n + 15) // 16
+    wt = np.zeros(tiles * nsuper * 2 * 64 * 4, np.uint32)
+    st = np.zeros(tiles * nsuper * (128 if bits == 4 else 16), np.float16)
+    for row in range(n):
+        t, col = divmod(row, 16)
+        for chunk in range(nsuper * 8):
+            sstep, r = divmod(chunk, 8)
+            kq, d = divmod(r, 2)
+            dst = (((t * nsuper + sstep) * 2 + d) * 64 + kq * 16 + col) * 4
+            wt[dst:dst + 4] = wq[row, chunk * 4:chunk * 4 + 4]
+            if bits == 4:
+                st[((t * nsuper + sstep) * 64 + kq * 16 + col) * 2 + d] = s[row, chunk]
+        if bits == 8:
+            for sstep in range(nsuper):
+                st[(t * nsuper + sstep) * 16 + col] = s[row, sstep]
+    return wt.reshape(tiles * 16, words), st.reshape(tiles * 16, s.shape[1])
+
+
+def untile_weights(wt: np.ndarray, st: np.ndarray, bits: int, n: int):
+    """Inverse of tile_weights (vectorized independently of it: reshape / transpose)."""
+    rows, words = wt.shape
+    tiles, nsuper = rows // 16, words * 4 // 128
+    w = wt.reshape(tiles, nsuper, 2, 4, 16, 4).transpose(0, 4, 1, 3, 2, 5).reshape(rows, words)  # [t,s,d,kq,col,4] -> [t,col,s,kq,d,4]
+    if bits == 4:
+        sc = st.reshape(tiles, nsuper, 4, 16, 2).transpose(0, 3, 1, 2, 4).reshape(rows, nsuper * 8)  # [t,s,kq,col,e] -> [t,col,s,kq,e]
+    else:
+        sc = st.reshape(tiles, nsuper, 16).transpose(0, 2, 1).reshape(rows, nsuper)
+    return np.ascontiguousarray(w[:n]), np.ascontiguousarray(sc[:n])
+
+
 def make_case(seed: int, m: int, n: int, k: int, bits: int, group: int | None = None):
     """x ~ N(0,1) f16; q4: w ~ U{0..15}, S ~ U(0.005,0.02); q8: w ~ U{-127..127}, S ~ U(0.002,0.01)."""
     rng = np.random.default_rng(seed)

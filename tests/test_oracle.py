@@ -350,3 +350,37 @@ def test_fused_path_is_epilogue_of_plain_path(bits, m, n, k):
             t = np.maximum(t, np.float16(0))
         want = (t.astype(np.float64) + res.astype(np.float64)).astype(np.float16)
         assert np.array_equal(a.view(np.uint16), want.view(np.uint16))
+
+
+# ---------------------------------------------------------------- tile-major weight layout
+@pytest.mark.parametrize("bits,n,k", [(4, 16, 256), (4, 37, 512), (8, 16, 128), (8, 50, 384)])
+def test_tile_major_layout_definition_and_round_trip(bits, n, k):
+    """The loop restatement places known chunks where the definition says, pads whole tiles with
+    zeros, and the independently written inverse (reshape / transpose) returns the input."""
+    rng = np.random.default_rng(bits * 1000 + n)
+    group = 32 if bits == 4 else 128
+    wq = rng.integers(0, 2**32, size=(n, k * bits // 32), dtype=np.uint64).astype(np.uint32)
+    s = rng.standard_normal((n, k // group)).astype(np.float16)
+    wt, st = O.tile_weights(wq, s, bits)
+    rows = (n + 15) // 16 * 16
+    assert wt.shape == (rows, wq.shape[1]) and st.shape == (rows, s.shape[1])
+    flat, nsuper = wt.reshape(-1), k * bits // 8 // 128
+    # hand-computed positions (in 32-bit words): row 0 chunk 0 first; row 1 chunk 0 one lane (4 words) later;
+    # row 0 chunk 1 (d = 1) one 1 KB block later; row 0 chunk 2 (kq = 1) sixteen lanes later
+    assert np.array_equal(flat[0:4], wq[0, 0:4]) and np.array_equal(flat[4:8], wq[1, 0:4])
+    assert np.array_equal(flat[256:260], wq[0, 4:8]) and np.array_equal(flat[64:68], wq[0, 8:12])
+    if nsuper > 1:  # row 0, chunk 8 = super step 1: two 1 KB blocks further
+        assert np.array_equal(flat[512:516], wq[0, 32:36])
+    if n > 16:      # row 16 = tile 1: after all super steps of tile 0
+        assert np.array_equal(flat[nsuper * 512:nsuper * 512 + 4], wq[16, 0:4])
+    sf = st.reshape(-1)
+    if bits == 4:
+        assert sf[0] == s[0, 0] and sf[1] == s[0, 1] and sf[2] == s[1, 0] and sf[32] == s[0, 2]
+    else:
+        assert sf[0] == s[0, 0] and sf[1] == s[1, 0] and (nsuper == 1 or sf[16] == s[0, 1])
+    # every byte is placed exactly once; the padding rows are zero
+    assert np.array_equal(np.sort(flat[flat != 0]), np.sort(wq.reshape(-1)[wq.reshape(-1) != 0]))
+    w2, s2 = O.untile_weights(wt, st, bits, n)
+    assert np.array_equal(w2, wq) and np.array_equal(s2.view(np.uint16), s.view(np.uint16))
+    wpad, spad = O.untile_weights(wt, st, bits, rows)
+    assert not wpad[n:].any() and not spad[n:].any()
