@@ -84,7 +84,8 @@ def config_table(torch, dev, args) -> int:
     """Every (M, N, K) of the parity configurations timed alone: q4f16 g32 at the 7B shapes for
     M in {1, 8, 512, 2048}, q8f16 g128 at the 13B shapes for M in {1, 16, 256}.  Each case rotates
     through enough distinct weight sets (> 512 MB in total) that no launch finds its weights in a
-    cache, inside one HIP graph; the time is the graph's divided by its launches."""
+    cache, inside one HIP graph; the time is the graph's divided by its launches.  Every case is
+    timed on canonical and on tile-major weights."""
     import relax_amd
     from relax_amd import lib
 
@@ -100,35 +101,46 @@ def config_table(torch, dev, args) -> int:
         x = torch.randn((m, k), device=dev).to(torch.float16)
         y = torch.empty((m, n), dtype=torch.float16, device=dev)
 
-        def one_pass():
-            for wq, s in ws:
-                relax_amd.wq_matmul(x, wq, s, bits, group, out=y)
+        wt = [relax_amd.wq_tile_weights(wq, s, bits, group) for wq, s in ws]
 
-        with torch.cuda.stream(stream):
-            one_pass()
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=stream):
-                one_pass()
-            g.replay()
-            torch.cuda.synchronize()
-            reps = max(3, min(args.steps, 2000 // sets))
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(reps):
+        def one_pass(tiled):
+            if tiled:
+                for wq, s in wt:
+                    relax_amd.wq_matmul(x, wq, s, bits, group, out=y, tiled_n=n)
+            else:
+                for wq, s in ws:
+                    relax_amd.wq_matmul(x, wq, s, bits, group, out=y)
+
+        times = {}
+        for tiled in (False, True):
+            with torch.cuda.stream(stream):
+                one_pass(tiled)
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    one_pass(tiled)
                 g.replay()
-            e1.record(stream)
-            torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) * 1e3 / (reps * sets)
+                torch.cuda.synchronize()
+                reps = max(3, min(args.steps, 2000 // sets))
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(reps):
+                    g.replay()
+                e1.record(stream)
+                torch.cuda.synchronize()
+            times[tiled] = e0.elapsed_time(e1) * 1e3 / (reps * sets)
+            del g
+        us = times[False]
         ab = algorithmic_bytes(bits, group, m, n, k)
         fl = 2.0 * m * n * k
         line = {"case": "q%df16 g%d M=%d N=%d K=%d" % (bits, group, m, n, k), "us": round(us, 2),
                 "kernel": {lib.KERNEL_GEMV: "gemv", lib.KERNEL_SKINNY: "skinny", lib.KERNEL_GEMM: "gemm"}[
                     lib.load().mi355x_wq_select_kernel(lib.make_desc(bits, group, n, k), m)],
                 "GB/s": round(ab / us / 1e3, 0), "frac_hbm": round(ab / us / 1e3 / HBM_PEAK_GBS, 3),
-                "TFLOP/s": round(fl / us / 1e6, 1), "frac_mfma": round(fl / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 3)}
+                "TFLOP/s": round(fl / us / 1e6, 1), "frac_mfma": round(fl / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 3),
+                "us_tile_major": round(times[True], 2), "tile_major_speedup": round(us / times[True], 3)}
         print(json.dumps(line), flush=True)
-        del ws, g
+        del ws, wt
     return 0
 
 
@@ -197,6 +209,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--no-epilogue", action="store_true", help="skip the fused-residual leg")
+    ap.add_argument("--no-tiled", action="store_true", help="skip the tile-major-weights decode leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times (a kernel of known HBM "
                          "traffic, used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
@@ -299,6 +312,40 @@ def main() -> int:
                      "avg_launch_us": round(avg_launch_us, 3)},
     }
     result["roofline"]["traffic"] = GEMV_HBM_TRAFFIC_PER_LAUNCH
+
+    # ---- the same decode step on tile-major weights (the one-off layout transform applied at load) ----
+    if not args.no_tiled:
+        tiled_layers = [[relax_amd.wq_tile_weights(wq, s, 4, 32) + (n, k) for wq, s, n, k in mats] for mats in layers]
+
+        def decode_pass_tiled():
+            for m in DECODE_BATCHES:
+                for mats in tiled_layers:
+                    for wt, st, n, k in mats:
+                        relax_amd.wq_matmul(xs[(m, k)], wt, st, 4, 32, out=ys[(m, n)], tiled_n=n)
+
+        with torch.cuda.stream(stream):
+            decode_pass_tiled()
+            torch.cuda.synchronize()
+            tgraph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(tgraph, stream=stream):
+                decode_pass_tiled()
+            for _ in range(args.warmup):
+                tgraph.replay()
+            torch.cuda.synchronize()
+            t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0.record(stream)
+            for _ in range(args.steps):
+                tgraph.replay()
+            t1.record(stream)
+            torch.cuda.synchronize()
+        tms = t0.elapsed_time(t1) / args.steps
+        tgbs = bytes_per_step / (tms * 1e-3) / 1e9
+        result["tile_major"] = {
+            "value": round(tgbs, 1), "unit": "GB/s", "frac": round(tgbs / HBM_PEAK_GBS, 4),
+            "ms_per_step": round(tms, 4), "avg_launch_us": round(tms * 1e3 / launches_per_step, 3),
+            "workload": "the same decode step with the weights in the tile-major layout "
+                        "(mi355x_wq_tile_weights applied once at load, outside the timing)"}
+        del tiled_layers, tgraph
 
     # ---- prefill GEMM leg: M = 2048, the four shapes, layer-rotated weights -----------------
     if not args.no_gemm:
