@@ -266,8 +266,13 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
       return -1;
     }
     p.tiled = true;
-    // the decode kernel up to 16 rows (while its LDS plan fits), the direct-weight GEMM beyond
-    return gemv_applicable(p) ? launch_gemv(p, 0) : launch_gemm(p, 0);
+    // the same choice as for canonical weights; the kernels that read the layout are the decode
+    // kernel, the skinny kernel and the direct-weight GEMM (which needs K % 256 == 0)
+    switch (select_kernel(desc, m)) {
+      case MI355X_WQ_KERNEL_GEMV: return launch_gemv(p, 0);
+      case MI355X_WQ_KERNEL_SKINNY: return launch_skinny(p, 0);
+      default: return launch_gemm(p, 0);
+    }
   }
   int chosen = family == MI355X_WQ_KERNEL_AUTO ? select_kernel(desc, m) : family;
   switch (chosen) {

@@ -29,7 +29,7 @@ struct SkinnyBatch {
   u32x4 xa[U][MT][NJ];
 };
 
-template <int BITS, int R, int MT, int WAVES, int U>
+template <int BITS, int R, int MT, int WAVES, int U, bool TILED>
 __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
     half_t* y, int M, int N, int K, int group_shift, int zero_point, const Epilogue ep) {
@@ -48,8 +48,11 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
   const int ks_end = min(ks_begin + per_wave, nsteps);
   const uint32_t groups_per_row = (uint32_t)nchunks >> group_shift;
 
-  const rsrc_t rw = make_rsrc(wq, (uint32_t)N * row_bytes);
-  const rsrc_t rs = make_rsrc(scales, (uint32_t)N * groups_per_row * 2u);
+  // (tile-major buffers hold whole 16-row tiles, zero filled past N)
+  const uint32_t n_stored = TILED ? ((uint32_t)N + 15u) / 16u * 16u : (uint32_t)N;
+  const uint32_t nsuper = row_bytes / 128u;  // 128-byte super steps per weight row (tile-major addressing)
+  const rsrc_t rw = make_rsrc(wq, n_stored * row_bytes);
+  const rsrc_t rs = make_rsrc(scales, n_stored * groups_per_row * 2u);
   const rsrc_t rx = make_rsrc(x, (uint32_t)M * (uint32_t)K * 2u);
 
   // per-lane row bases.  Weight rows past N are clamped to the last row (their
@@ -58,9 +61,18 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
   bool xrow_ok[MT];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int n = min((int)(blockIdx.x * R + r) * 16 + col, N - 1);
-    wbase[r] = (uint32_t)n * row_bytes;
-    sbase[r] = (uint32_t)n * groups_per_row * 2u;
+    const int n = min((int)(blockIdx.x * R + r) * 16 + col, (int)n_stored - 1);
+    if constexpr (TILED) {
+      // chunk c of row n: ((tile*S + c/8)*2 + c%2)*1024 + ((c%8)/2*16 + n%16)*16; its scale (int4) is
+      // half c%2 of the 4-byte pair at ((tile*S + c/8)*64 + (c%8)/2*16 + n%16)*4, (int8) the float16 at
+      // ((tile*S + c/8)*16 + n%16)*2
+      const uint32_t tile = (uint32_t)n >> 4, c16 = (uint32_t)n & 15u;
+      wbase[r] = tile * nsuper * 2048u + c16 * 16u;
+      sbase[r] = BITS == 4 ? (tile * nsuper * 64u + c16) * 4u : (tile * nsuper * 16u + c16) * 2u;
+    } else {
+      wbase[r] = (uint32_t)n * row_bytes;
+      sbase[r] = (uint32_t)n * groups_per_row * 2u;
+    }
   }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -83,8 +95,12 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
       const int ks = ks0 + u;
       const int chunk = ks * 4 + kq;
       const bool ok = (ks < ks_end) && (chunk < nchunks);
-      const uint32_t winc = ok ? (uint32_t)chunk * 16u : kOobOffset;
-      const uint32_t sinc = ok ? ((uint32_t)chunk >> group_shift) * 2u : kOobOffset;
+      const uint32_t uc = (uint32_t)chunk, c8 = uc & 7u;
+      const uint32_t winc = !ok ? kOobOffset
+                            : TILED ? (uc >> 3) * 2048u + (c8 & 1u) * 1024u + (c8 >> 1) * 256u : uc * 16u;
+      const uint32_t sinc = !ok ? kOobOffset
+                            : !TILED ? (uc >> group_shift) * 2u
+                            : BITS == 4 ? (uc >> 3) * 256u + (c8 >> 1) * 64u + (c8 & 1u) * 2u : (uc >> 3) * 32u;
       const uint32_t xinc = (uint32_t)chunk * (CH * 2u);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
@@ -182,11 +198,11 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
 
 namespace {
 
-template <int BITS, int R, int MT, int WAVES, int U>
+template <int BITS, int R, int MT, int WAVES, int U, bool TILED = false>
 void launch_one(const Problem& p, int group_shift) {
   const int tiles = (int)((p.n + 15) / 16);
   dim3 grid((tiles + R - 1) / R), block(WAVES * 64);
-  hipLaunchKernelGGL((wq_skinny_kernel<BITS, R, MT, WAVES, U>), grid, block, 0, p.stream,
+  hipLaunchKernelGGL((wq_skinny_kernel<BITS, R, MT, WAVES, U, TILED>), grid, block, 0, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point,
                      Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
@@ -194,6 +210,16 @@ void launch_one(const Problem& p, int group_shift) {
 
 template <int BITS, int MT>
 bool dispatch_variant(const Problem& p, int group_shift, int variant) {
+  if (p.tiled) {  // the variants the default choice uses, reading the tile-major layout
+    switch (variant) {
+      case 1: launch_one<BITS, 1, MT, 4, 2, true>(p, group_shift); return true;
+      case 2: launch_one<BITS, 2, MT, 4, 2, true>(p, group_shift); return true;
+      case 5: launch_one<BITS, 2, MT, 8, 1, true>(p, group_shift); return true;
+      case 7: launch_one<BITS, 4, MT, 4, 1, true>(p, group_shift); return true;
+      case 9: launch_one<BITS, 4, MT, 2, 1, true>(p, group_shift); return true;
+      default: return false;
+    }
+  }
   switch (variant) {
     case 1: launch_one<BITS, 1, MT, 4, 2>(p, group_shift); return true;
     case 2: launch_one<BITS, 2, MT, 4, 2>(p, group_shift); return true;

@@ -46,21 +46,22 @@ def test_tile_weights_matches_the_loop_restatement_and_round_trips(bits, n, k):
 GEMV_CASES = [(4, 1, 48, 256), (4, 3, 100, 512), (4, 16, 72, 1024), (4, 8, 4096, 4096), (4, 1, 22016, 4096),
               (4, 16, 4096, 11008), (4, 5, 1000, 8192), (8, 2, 40, 128), (8, 16, 72, 384), (8, 1, 5120, 5120),
               (8, 16, 5120, 13824), (8, 7, 333, 1280)]
-GEMM_CASES = [(4, 17, 136, 768), (4, 64, 200, 1280), (4, 70, 136, 768), (4, 300, 521, 1024), (4, 2048, 4096, 4096),
-              (8, 33, 300, 2304), (8, 129, 72, 256), (8, 513, 260, 1024), (8, 256, 5120, 5120)]
+SKINNY_CASES = [(4, 17, 136, 768), (4, 64, 200, 1280), (4, 40, 4096, 4096), (4, 16, 4096, 4096), (4, 24, 12288, 4096),
+                (8, 33, 300, 2304), (8, 48, 5120, 5120), (4, 20, 6200, 512), (4, 30, 16400, 256),
+                (4, 20, 5120, 512), (4, 1, 152064, 256), (4, 40, 16400, 256)]  # every tile-major skinny variant
+GEMM_CASES = [(4, 70, 136, 768), (4, 300, 521, 1024), (4, 2048, 4096, 4096), (4, 48, 12288, 4096), (4, 24, 22016, 4096),
+              (8, 129, 72, 256), (8, 513, 260, 1024), (8, 256, 5120, 5120)]
 
 
-@pytest.mark.parametrize("bits,m,n,k", GEMV_CASES + GEMM_CASES)
+@pytest.mark.parametrize("bits,m,n,k", GEMV_CASES + SKINNY_CASES + GEMM_CASES)
 def test_matmul_on_tile_major_weights_is_bit_identical_to_canonical(bits, m, n, k):
     import relax_amd
-    from relax_amd import lib
 
     x, wq, s, g = O.make_case(40 + m + n, m, n, k, bits)
     wt, st = _tiled(wq, s, bits, g)
     xd = _dev(x)
-    # the same kernel family the tile-major entry uses for this M
-    family = lib.KERNEL_GEMV if m <= 16 else lib.KERNEL_GEMM
-    y_canon = relax_amd.wq_matmul(xd, _dev(wq), _dev(s), bits, g, kernel=family)
+    # both layouts go through the same kernel selection, hence the same kernel
+    y_canon = relax_amd.wq_matmul(xd, _dev(wq), _dev(s), bits, g)
     y_tiled = relax_amd.wq_matmul(xd, wt, st, bits, g, tiled_n=n)
     torch.cuda.synchronize()
     assert np.array_equal(y_tiled.cpu().numpy().view(np.uint16), y_canon.cpu().numpy().view(np.uint16))
