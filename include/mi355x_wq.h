@@ -137,6 +137,11 @@ MI355X_WQ_API int mi355x_wq_matmul_tiled(const mi355x_wq_desc* desc, const void*
                                         const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y,
                                         int64_t m, void* stream);
 
+/* Same, with the kernel family forced (tests and benchmarks). */
+MI355X_WQ_API int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const void* x, const void* wq_tiled,
+                                           const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y,
+                                           int64_t m, void* stream, int kernel);
+
 /* Validates a descriptor and a row count without touching the GPU: 0 if
  * mi355x_wq_matmul would accept them. */
 MI355X_WQ_API int mi355x_wq_check(const mi355x_wq_desc* desc, int64_t m);

@@ -182,6 +182,12 @@ int mi355x_wq_matmul_tiled(const mi355x_wq_desc* desc, const void* x, const void
   return matmul_any_layout(desc, x, wq_tiled, scales_tiled, ep, y, m, stream, MI355X_WQ_KERNEL_AUTO, true);
 }
 
+int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const void* x, const void* wq_tiled,
+                              const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y, int64_t m,
+                              void* stream, int kernel) {
+  return matmul_any_layout(desc, x, wq_tiled, scales_tiled, ep, y, m, stream, kernel, true);
+}
+
 int mi355x_wq_tiled_sizes(const mi355x_wq_desc* desc, int64_t* wq_bytes, int64_t* scales_bytes) {
   using namespace wq;
   if (!check_desc(desc, 0)) return -1;
@@ -268,10 +274,11 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
     p.tiled = true;
     // the same choice as for canonical weights; the kernels that read the layout are the decode
     // kernel, the skinny kernel and the direct-weight GEMM (which needs K % 256 == 0)
-    switch (select_kernel(desc, m)) {
-      case MI355X_WQ_KERNEL_GEMV: return launch_gemv(p, 0);
-      case MI355X_WQ_KERNEL_SKINNY: return launch_skinny(p, 0);
-      default: return launch_gemm(p, 0);
+    switch (family == MI355X_WQ_KERNEL_AUTO ? select_kernel(desc, m) : family) {
+      case MI355X_WQ_KERNEL_GEMV: return launch_gemv(p, variant);
+      case MI355X_WQ_KERNEL_SKINNY: return launch_skinny(p, variant);
+      case MI355X_WQ_KERNEL_GEMM: return launch_gemm(p, variant);
+      default: set_error("unknown kernel family %d", family); return -1;
     }
   }
   int chosen = family == MI355X_WQ_KERNEL_AUTO ? select_kernel(desc, m) : family;

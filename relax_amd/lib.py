@@ -16,7 +16,7 @@ ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "relax.nn.rel
 EXPORTED_SYMBOLS = (
     "mi355x_wq_matmul", "mi355x_wq_matmul_ex", "mi355x_wq_matmul_fused", "mi355x_wq_matmul_fused_ex",
     "mi355x_wq_dequantize", "mi355x_wq_check",
-    "mi355x_wq_tiled_sizes", "mi355x_wq_tile_weights", "mi355x_wq_untile_weights", "mi355x_wq_matmul_tiled",
+    "mi355x_wq_tiled_sizes", "mi355x_wq_tile_weights", "mi355x_wq_untile_weights", "mi355x_wq_matmul_tiled", "mi355x_wq_matmul_tiled_ex",
     "mi355x_wq_select_kernel", "mi355x_wq_last_error", "mi355x_wq_version",
     "mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_matmul_bias", "mi355x_q8f16_matmul_bias",
     "mi355x_q4f16_matmul_bias_relu", "mi355x_q8f16_matmul_bias_relu", "mi355x_q4f16_matmul_residual",
@@ -79,6 +79,7 @@ def load() -> C.CDLL:
     L.mi355x_wq_tile_weights.argtypes = [dp, vp, vp, vp, vp, vp]
     L.mi355x_wq_untile_weights.argtypes = [dp, vp, vp, vp, vp, vp]
     L.mi355x_wq_matmul_tiled.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp]
+    L.mi355x_wq_matmul_tiled_ex.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp, ci]
     L.mi355x_wq_check.argtypes = [dp, i64]
     L.mi355x_wq_select_kernel.argtypes = [dp, i64]
     L.mi355x_wq_last_error.restype = C.c_char_p

@@ -32,7 +32,7 @@ def wq_matmul(x: torch.Tensor, wq: torch.Tensor, scales: torch.Tensor, bits: int
     for an N-row matrix (their row count is N rounded up to 16)."""
     if tiled_n is not None:
         return _wq_matmul_tiled(x, wq, scales, bits, group, tiled_n, zero_point, out, stream, bias,
-                                activation, residual)
+                                activation, residual, kernel | (variant << 8))
     L = _lib.load()
     wq = _as_u32_storage(wq)
     if not (x.is_cuda and wq.is_cuda and scales.is_cuda):
@@ -122,7 +122,8 @@ def wq_untile_weights(wq_tiled: torch.Tensor, scales_tiled: torch.Tensor, bits: 
     return wq, s
 
 
-def _wq_matmul_tiled(x, wq_t, s_t, bits, group, n, zero_point, out, stream, bias, activation, residual):
+def _wq_matmul_tiled(x, wq_t, s_t, bits, group, n, zero_point, out, stream, bias, activation, residual,
+                     kernel=0):
     L = _lib.load()
     if not (x.is_cuda and wq_t.is_cuda and s_t.is_cuda):
         raise ValueError("x, wq and scales must be device tensors")
@@ -142,8 +143,8 @@ def _wq_matmul_tiled(x, wq_t, s_t, bits, group, n, zero_point, out, stream, bias
     ep = _lib.WqEpilogue(bias.data_ptr() if bias is not None else None,
                          residual.data_ptr() if residual is not None else None,
                          _lib.ACTIVATIONS[activation], 0)
-    _lib.check(L.mi355x_wq_matmul_tiled(desc, x.data_ptr(), wq_t.data_ptr(), s_t.data_ptr(), ep, out.data_ptr(), m,
-                                        _stream_ptr(stream)))
+    _lib.check(L.mi355x_wq_matmul_tiled_ex(desc, x.data_ptr(), wq_t.data_ptr(), s_t.data_ptr(), ep, out.data_ptr(),
+                                           m, _stream_ptr(stream), kernel))
     return out
 
 

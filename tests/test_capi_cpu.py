@@ -27,7 +27,7 @@ def declared_symbols():
 def test_library_exports_every_declared_symbol():
     L = lib.load()
     names = declared_symbols()
-    assert len(names) == 31 and set(names) == set(lib.EXPORTED_SYMBOLS)
+    assert len(names) == 32 and set(names) == set(lib.EXPORTED_SYMBOLS)
     for n in names:
         assert hasattr(L, n), n
     assert L.mi355x_wq_version() >= 100
