@@ -212,6 +212,10 @@ int tile_or_untile(const mi355x_wq_desc* desc, const void* wq_src, const void* s
   if (!check_ptr(wq_src, forward ? "wq" : "wq_tiled", 16) || !check_ptr(scales_src, forward ? "scales" : "scales_tiled", 16) ||
       !check_ptr(wq_dst, forward ? "wq_tiled" : "wq", 16) || !check_ptr(scales_dst, forward ? "scales_tiled" : "scales", 16))
     return -1;
+  if (wq_dst == wq_src || scales_dst == scales_src) {
+    set_error("the layout transform is not an in-place operation: source and destination must differ");
+    return -1;
+  }
   Problem p{nullptr, wq_src, scales_src, nullptr, 0, desc->n, desc->k, desc->bits, desc->group,
             desc->zero_point, static_cast<hipStream_t>(stream)};
   return launch_tile_weights(p, wq_dst, scales_dst, forward);

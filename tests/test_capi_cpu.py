@@ -37,6 +37,25 @@ def test_library_exports_every_declared_symbol():
     assert sorted(exported) == sorted(names)
 
 
+def test_tile_major_layout_entry_checks_without_a_gpu():
+    L = lib.load()
+    wb, sb = C.c_int64(0), C.c_int64(0)
+    assert L.mi355x_wq_tiled_sizes(lib.make_desc(4, 32, 100, 512), C.byref(wb), C.byref(sb)) == 0
+    assert (wb.value, sb.value) == (112 * 256, 112 * 16 * 2)       # 100 rows -> 112: whole 16-row tiles
+    assert L.mi355x_wq_tiled_sizes(lib.make_desc(8, 128, 16, 384), C.byref(wb), C.byref(sb)) == 0
+    assert (wb.value, sb.value) == (16 * 384, 16 * 3 * 2)
+    assert L.mi355x_wq_tiled_sizes(lib.make_desc(4, 32, 100, 320), C.byref(wb), C.byref(sb)) == -1
+    assert "K % 256 == 0" in lib.last_error()
+    assert L.mi355x_wq_tiled_sizes(lib.make_desc(4, 64, 100, 512), None, None) == -1 and "group 32" in lib.last_error()
+    d, ok = lib.make_desc(4, 32, 64, 256), 0x10000
+    assert L.mi355x_wq_tile_weights(d, ok, ok + 0x1000, ok, ok + 0x2000, None) == -1 and "in-place" in lib.last_error()
+    assert L.mi355x_wq_tile_weights(d, ok, ok + 8, ok + 0x1000, ok + 0x2000, None) == -1 \
+        and "scales" in lib.last_error() and "16-byte aligned" in lib.last_error()
+    assert L.mi355x_wq_untile_weights(d, None, ok, ok, ok, None) == -1 and "wq_tiled is NULL" in lib.last_error()
+    assert L.mi355x_wq_matmul_tiled(lib.make_desc(4, 32, 64, 320), ok, ok, ok, None, ok, 4, None) == -1 \
+        and "tile-major layout" in lib.last_error()
+
+
 def test_measurement_probe_library_is_built_and_separate():
     """bench.py --probe-mfma loads its kernel from a library of its own; the product library has
     no symbol of it."""
