@@ -353,6 +353,9 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
       constexpr int s = decltype(sc)::value;
       constexpr int kk = s / (2 * TM), j = (s / TM) % 2, i = s % TM;
       constexpr int q = kk * 2 + j;  // index of the B fragment in use
+      // Two wavefronts share a SIMD (K groups): the one further back in its step gets the issue slots,
+      // so that both reach the step's barrier together instead of one idling there.
+      if constexpr (GROUPS > 1 && s % (2 * TM) == 0) __builtin_amdgcn_s_setprio(3 - kk);
       const half8_t bm = __builtin_bit_cast(half8_t, fbq[q & 3]);
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk & 1][i], bm, acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
