@@ -130,9 +130,9 @@ MI355X_WQ_API int mi355x_wq_tile_weights(const mi355x_wq_desc* desc, const void*
 MI355X_WQ_API int mi355x_wq_untile_weights(const mi355x_wq_desc* desc, const void* wq_tiled, const void* scales_tiled,
                                           void* wq, void* scales, void* stream);
 
-/* mi355x_wq_matmul_fused on tile-major weights (`ep` may be NULL).  Same kernel selection as for
- * canonical weights: the decode kernel reads the contiguous stream, the skinny kernel and the
- * direct-weight GEMM address the layout; M > 64 (and the wide 24..64-row cases) need K % 256 == 0. */
+/* mi355x_wq_matmul_fused on tile-major weights (`ep` may be NULL).  The same three kernel families
+ * (the decode kernel reads the contiguous stream, the skinny kernel and the direct-weight GEMM
+ * address the layout) with crossovers measured on this layout; M > 64 needs K % 256 == 0. */
 MI355X_WQ_API int mi355x_wq_matmul_tiled(const mi355x_wq_desc* desc, const void* x, const void* wq_tiled,
                                         const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y,
                                         int64_t m, void* stream);

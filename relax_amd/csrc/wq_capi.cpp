@@ -122,7 +122,7 @@ bool check_ptr(const void* p, const char* name, size_t align) {
   return true;
 }
 
-int select_kernel(const mi355x_wq_desc* d, int64_t m) {
+int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
   Problem p{nullptr, nullptr, nullptr, nullptr, m, d->n, d->k, d->bits, d->group, d->zero_point, nullptr};
   if (gemv_applicable(p)) {
     // The GEMV kernel stages the activations in LDS.  Measured on MI355X: once they
@@ -140,6 +140,15 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m) {
   const int64_t tiles128 = (d->n + 127) / 128;
   const bool direct_small_tile = d->k % 256 == 0 && d->k >= 1024 && tiles128 <= cu_count() &&
                                  ((d->bits == 4 && d->group == 32) || (d->bits == 8 && d->group == 128));
+  if (tiled) {
+    // On tile-major weights the skinny kernel's loads are contiguous and it holds out longer
+    // (N = 12288, 32 rows: 14 us against the GEMM's 22 us): the GEMM takes over from 32 rows (int4) or
+    // 40 rows (int8) with 160 or more column tiles, and for int4 from 57 rows with 64 or more.
+    if (direct_small_tile && ((tiles128 >= 160 && m >= (d->bits == 4 ? 32 : 40)) ||
+                              (d->bits == 4 && m > 56 && tiles128 >= 64)))
+      return MI355X_WQ_KERNEL_GEMM;
+    return MI355X_WQ_KERNEL_SKINNY;
+  }
   if (direct_small_tile && ((m >= 24 && tiles128 >= 160) || (d->bits == 4 && m > 32 && tiles128 >= 64)))
     return MI355X_WQ_KERNEL_GEMM;
   return MI355X_WQ_KERNEL_SKINNY;
@@ -278,7 +287,7 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
     p.tiled = true;
     // the same choice as for canonical weights; the kernels that read the layout are the decode
     // kernel, the skinny kernel and the direct-weight GEMM (which needs K % 256 == 0)
-    switch (family == MI355X_WQ_KERNEL_AUTO ? select_kernel(desc, m) : family) {
+    switch (family == MI355X_WQ_KERNEL_AUTO ? select_kernel(desc, m, true) : family) {
       case MI355X_WQ_KERNEL_GEMV: return launch_gemv(p, variant);
       case MI355X_WQ_KERNEL_SKINNY: return launch_skinny(p, variant);
       case MI355X_WQ_KERNEL_GEMM: return launch_gemm(p, variant);
