@@ -129,14 +129,19 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
     // are large (more than 64 KB, one workgroup per CU) and there is at most one row tile per CU
     // to amortise the staging, the register-activation kernel is faster.
     const int64_t x_bytes = m * d->k * 2, tiles = (d->n + 15) / 16;
-    if (!(x_bytes > 64 * 1024 && tiles <= 256)) return MI355X_WQ_KERNEL_GEMV;
+    // (for rows of 16384 and more the staging kernel wins again: 4096 x 16384 at 4 rows 13.7 against
+    // 17.4 us; and with at most 2048 columns of K or a few dozen row tiles the matrix is so small --
+    // 4 MB -- that the staging kernel's start-up costs more than it saves: 4096 x 2048, 5.6 against 4.9 us)
+    const bool big_x = x_bytes > 64 * 1024 && tiles <= 256 && d->k < 16384;
+    const bool tiny = tiles <= 256 && (d->k <= 2048 || (tiles <= 128 && m <= 2));
+    if (!big_x && !tiny) return MI355X_WQ_KERNEL_GEMV;
   }
   if (m > kSkinnyMaxM) return MI355X_WQ_KERNEL_GEMM;
   // 17..64 rows.  The skinny kernel re-reads the activations from L2 once per 16-row weight tile, so
   // its time grows with M and N; the direct-weight GEMM with its 64x128 tile and four K groups costs
   // the same from 1 to 64 rows.  Measured crossovers on MI355X (q4f16 and q8f16, K = 4096 ... 13824):
   // with 160 or more 128-column tiles the GEMM wins from 24 rows on (N = 22016: 29 us against
-  // 36 - 52 us), with 64 or more tiles of int4 weights from 33 rows on.
+  // 36 - 52 us), with 96 or more tiles of int4 weights from 33 rows on, with 64 or more from 49.
   const int64_t tiles128 = (d->n + 127) / 128;
   const bool direct_small_tile = d->k % 256 == 0 && d->k >= 1024 && tiles128 <= cu_count() &&
                                  ((d->bits == 4 && d->group == 32) || (d->bits == 8 && d->group == 128));
@@ -149,7 +154,8 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
       return MI355X_WQ_KERNEL_GEMM;
     return MI355X_WQ_KERNEL_SKINNY;
   }
-  if (direct_small_tile && ((m >= 24 && tiles128 >= 160) || (d->bits == 4 && m > 32 && tiles128 >= 64)))
+  if (direct_small_tile && ((m >= 24 && tiles128 >= 160) || (d->bits == 4 && m > 32 && tiles128 >= 96) ||
+                            (d->bits == 4 && m > 48 && tiles128 >= 64)))
     return MI355X_WQ_KERNEL_GEMM;
   return MI355X_WQ_KERNEL_SKINNY;
 }

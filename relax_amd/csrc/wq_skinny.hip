@@ -252,13 +252,14 @@ int launch_skinny(const Problem& p, int variant) {
   const int mt = (int)((p.m + 15) / 16);
   if (variant == 0) {
     // Measured on MI355X (q4f16, Llama-2-7B shapes, M = 4 .. 64): the number of workgroups is what
-    // matters.  At most one row tile per CU: one tile per 4-wave workgroup; a few more: two
+    // matters: as few tiles per workgroup as still give every CU at most one workgroup.
+    // At most one row tile per CU: one tile per 4-wave workgroup; up to two per CU: two
     // tiles per workgroup, eight wavefronts for int4 and four for int8 (a second, mostly empty
     // round of workgroups costs more: 5120 x 13824 at 64 rows 114 -> 67 us); more: four
     // tiles per workgroup; many: two tiles per 8-wave workgroup for one row block, else four.
     const int64_t tiles = (p.n + 15) / 16;
     if (tiles <= 256) variant = 1;
-    else if (tiles <= 384) variant = p.bits == 4 ? 5 : 2;  // (one tile per workgroup is 1.5 - 1.8x slower here)
+    else if (tiles <= 512) variant = p.bits == 4 ? 5 : 2;  // (one tile per workgroup is 1.5 - 1.8x slower here)
     else if (tiles <= 1024) variant = 7;
     else variant = mt == 1 ? 5 : (mt == 2 ? 7 : 9);
   }
