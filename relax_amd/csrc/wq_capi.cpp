@@ -130,10 +130,10 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
     // to amortise the staging, the register-activation kernel is faster.
     const int64_t x_bytes = m * d->k * 2, tiles = (d->n + 15) / 16;
     // (for rows of 16384 and more the staging kernel wins again: 4096 x 16384 at 4 rows 13.7 against
-    // 17.4 us; and with at most 2048 columns of K or a few dozen row tiles the matrix is so small --
-    // 4 MB -- that the staging kernel's start-up costs more than it saves: 4096 x 2048, 5.6 against 4.9 us)
+    // 17.4 us; and with at most 2048 columns of K and 256 row tiles the matrix is so small -- 4 MB --
+    // that the staging kernel's start-up costs more than it saves: 4096 x 2048, 5.6 against 4.9 us)
     const bool big_x = x_bytes > 64 * 1024 && tiles <= 256 && d->k < 16384;
-    const bool tiny = tiles <= 256 && (d->k <= 2048 || (tiles <= 128 && m <= 2));
+    const bool tiny = tiles <= 256 && d->k <= 2048;
     if (!big_x && !tiny) return MI355X_WQ_KERNEL_GEMV;
   }
   if (m > kSkinnyMaxM) return MI355X_WQ_KERNEL_GEMM;
