@@ -147,10 +147,10 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
                                  ((d->bits == 4 && d->group == 32) || (d->bits == 8 && d->group == 128));
   if (tiled) {
     // On tile-major weights the skinny kernel's loads are contiguous and it holds out longer
-    // (N = 12288, 32 rows: 14 us against the GEMM's 22 us): the GEMM takes over from 32 rows (int4) or
-    // 40 rows (int8) with 160 or more column tiles, and for int4 from 57 rows with 64 or more.
-    if (direct_small_tile && ((tiles128 >= 160 && m >= (d->bits == 4 ? 32 : 40)) ||
-                              (d->bits == 4 && m > 56 && tiles128 >= 64)))
+    // (N = 12288, 32 rows: 14 us against the GEMM's 22 us): for int4 the GEMM takes over from 40 rows
+    // with 160 or more column tiles and from 57 rows with 64 or more; int8 stays with the skinny
+    // kernel up to 64 rows (27648 x 5120 at 48 rows: 44 against 50 us).
+    if (direct_small_tile && d->bits == 4 && ((tiles128 >= 160 && m >= 40) || (m > 56 && tiles128 >= 64)))
       return MI355X_WQ_KERNEL_GEMM;
     return MI355X_WQ_KERNEL_SKINNY;
   }

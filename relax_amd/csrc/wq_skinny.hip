@@ -217,6 +217,7 @@ bool dispatch_variant(const Problem& p, int group_shift, int variant) {
       case 5: launch_one<BITS, 2, MT, 8, 1, true>(p, group_shift); return true;
       case 7: launch_one<BITS, 4, MT, 4, 1, true>(p, group_shift); return true;
       case 9: launch_one<BITS, 4, MT, 2, 1, true>(p, group_shift); return true;
+      case 11: launch_one<BITS, 8, MT, 4, 1, true>(p, group_shift); return true;
       default: return false;
     }
   }
@@ -231,6 +232,7 @@ bool dispatch_variant(const Problem& p, int group_shift, int variant) {
     case 8: launch_one<BITS, 4, MT, 8, 1>(p, group_shift); return true;
     case 9: launch_one<BITS, 4, MT, 2, 1>(p, group_shift); return true;
     case 10: launch_one<BITS, 2, MT, 2, 2>(p, group_shift); return true;
+    case 11: launch_one<BITS, 8, MT, 4, 1>(p, group_shift); return true;
     default: return false;
   }
 }
@@ -261,7 +263,7 @@ int launch_skinny(const Problem& p, int variant) {
     if (tiles <= 256) variant = 1;
     else if (tiles <= 512) variant = p.bits == 4 ? 5 : 2;  // (one tile per workgroup is 1.5 - 1.8x slower here)
     else if (tiles <= 1024) variant = 7;
-    else variant = mt == 1 ? 5 : (mt == 2 ? 7 : 9);
+    else variant = mt == 1 ? 5 : 11;  // several rounds of workgroups: eight tiles share one pass over the activations
   }
   bool ok;
   if (p.bits == 4) {

@@ -149,7 +149,7 @@ def test_gemv_refuses_more_than_16_rows():
 
 
 # ------------------------------------------------------------------ skinny kernel (activations in registers)
-SKINNY_VARIANTS = [1, 2, 3, 4, 5, 6]
+SKINNY_VARIANTS = [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11]
 
 
 @pytest.mark.parametrize("variant", SKINNY_VARIANTS)

@@ -48,7 +48,7 @@ GEMV_CASES = [(4, 1, 48, 256), (4, 3, 100, 512), (4, 16, 72, 1024), (4, 8, 4096,
               (8, 16, 5120, 13824), (8, 7, 333, 1280)]
 SKINNY_CASES = [(4, 17, 136, 768), (4, 64, 200, 1280), (4, 40, 4096, 4096), (4, 16, 4096, 4096), (4, 24, 12288, 4096),
                 (8, 33, 300, 2304), (8, 48, 5120, 5120), (4, 20, 6200, 512), (4, 30, 16400, 256),
-                (4, 20, 5120, 512), (4, 1, 152064, 256), (4, 40, 16400, 256)]  # every tile-major skinny variant
+                (4, 20, 5120, 512), (4, 1, 152064, 256), (4, 40, 16400, 256), (8, 30, 16400, 256)]  # every tile-major skinny variant
 GEMM_CASES = [(4, 70, 136, 768), (4, 300, 521, 1024), (4, 2048, 4096, 4096), (4, 48, 12288, 4096), (4, 24, 22016, 4096),
               (8, 129, 72, 256), (8, 513, 260, 1024), (8, 256, 5120, 5120)]
 
