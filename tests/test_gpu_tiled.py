@@ -128,3 +128,31 @@ def test_tile_major_layout_is_refused_where_it_is_not_defined():
     relax_amd.wq_matmul(_dev(x[:8]), wt, st, 8, g, tiled_n=64)
     with pytest.raises(lib.WqError, match="direct-weight kernel"):
         relax_amd.wq_matmul(_dev(x), wt, st, 8, g, tiled_n=64)
+
+
+@pytest.mark.parametrize("chunk", range(4))
+def test_seeded_random_shapes_on_tile_major_weights(chunk):
+    """Ragged N from 1, every M class, every K the layout is defined for: the tiled entry's own kernel
+    choice against the oracle, plain and with the full fused tail, and the transform's round trip."""
+    import relax_amd
+
+    rng = np.random.default_rng(2000 + chunk)
+    for _ in range(12):
+        bits = int(rng.choice([4, 8]))
+        g = 32 if bits == 4 else 128
+        k = 256 * int(rng.integers(1, 9))
+        m = int(rng.choice([1, 2, 3, 5, 8, 13, 16, 17, 31, 40, 64, 65, 100, 129, 257, 300]))
+        n = int(rng.integers(1, 700))
+        x, wq, s, _ = O.make_case(chunk * 100 + m + n, m, n, k, bits, g)
+        wt, st = _tiled(wq, s, bits, g)
+        w2, s2 = relax_amd.wq_untile_weights(wt, st, bits, g, n, k)
+        got = relax_amd.wq_matmul(_dev(x), wt, st, bits, g, tiled_n=n)
+        bias, res = _fused_operands(m + n + k, m, n)
+        fused = relax_amd.wq_matmul(_dev(x), wt, st, bits, g, tiled_n=n, bias=_dev(bias), activation="relu",
+                                    residual=_dev(res))
+        torch.cuda.synchronize()
+        assert np.array_equal(w2.cpu().numpy().view(np.uint32), wq), (bits, m, n, k)
+        assert np.array_equal(s2.cpu().numpy().view(np.uint16), s.view(np.uint16)), (bits, m, n, k)
+        want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
+        assert_close(got.cpu().numpy(), want, (bits, m, n, k))
+        assert_fused(fused.cpu().numpy(), got.cpu().numpy(), want, bias, "relu", res, ("fused", bits, m, n, k))
