@@ -4,7 +4,7 @@ The reference holds no vectors for a quantized matmul (it has no such operator),
 fixtures are outputs of the pinned CPU oracle on seeded inputs; they freeze the layout
 (least-significant field first) and the rounding sequence.  Run from the repo root:
 
-    python tests/golden/make_golden.py
+    python tests/golden/make_golden.py            (--fused-only / --tiled-only: just those fixtures)
 """
 import os
 import sys
@@ -30,6 +30,12 @@ FUSED_CASES = [  # name, seed, M, N, K, bits, group, bias?, activation, residual
 ]
 
 
+TILED_CASES = [  # name, seed, N, K, bits: the tile-major layout frozen as data (it is a storage format)
+    ("tiled_q4f16_n37_k512", 31, 37, 512, 4),
+    ("tiled_q8f16_n50_k384", 32, 50, 384, 8),
+]
+
+
 def fused_operands(seed, m, n, with_bias, with_residual):
     """bias ~ N(0, 0.5), residual ~ N(0, 1), float16, from their own seeded stream."""
     rng = np.random.default_rng(1000 + seed)
@@ -40,6 +46,14 @@ def fused_operands(seed, m, n, with_bias, with_residual):
 
 if __name__ == "__main__":
     here = os.path.dirname(os.path.abspath(__file__))
+    for name, seed, n, k, bits in TILED_CASES:
+        _, wq, s, g = O.make_case(seed, 1, n, k, bits)
+        wt, st = O.tile_weights(wq, s, bits)
+        np.savez_compressed(os.path.join(here, name + ".npz"), wq=wq, scales=s, wq_tiled=wt, scales_tiled=st,
+                            bits=np.int32(bits), group=np.int32(g))
+        print(name, wt.shape, st.shape)
+    if "--tiled-only" in sys.argv:
+        sys.exit(0)
     for name, seed, m, n, k, bits, group, wb, act, wr in FUSED_CASES:
         x, wq, s, g = O.make_case(seed, m, n, k, bits, group)
         bias, res = fused_operands(seed, m, n, wb, wr)

@@ -9,8 +9,9 @@ from oracle import c_oracle, wq_oracle as O
 FILES = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
 
 
-PLAIN = [f for f in FILES if not os.path.basename(f).startswith("fused_")]
+PLAIN = [f for f in FILES if not os.path.basename(f).startswith(("fused_", "tiled_"))]
 FUSED = [f for f in FILES if os.path.basename(f).startswith("fused_")]
+TILED = [f for f in FILES if os.path.basename(f).startswith("tiled_")]
 
 
 def test_fixtures_exist():
@@ -73,3 +74,16 @@ def test_fixture_known_fields():
     s0 = np.float64(z["scales"][0, 0])
     want = (np.array(fields, dtype=np.float64) - 7) * s0
     assert np.array_equal(z["wd"][0, :8], want.astype(np.float16))
+
+
+def test_tile_major_fixtures_match_the_oracle_both_ways():
+    """The storage format is frozen as data: the loop restatement reproduces the fixture, the
+    independently written inverse takes the fixture back to the canonical tensors."""
+    assert len(TILED) >= 2
+    for f in TILED:
+        z = np.load(f)
+        bits = int(z["bits"])
+        wt, st = O.tile_weights(z["wq"], z["scales"], bits)
+        assert np.array_equal(wt, z["wq_tiled"]) and np.array_equal(st.view(np.uint16), z["scales_tiled"].view(np.uint16)), f
+        w, s = O.untile_weights(z["wq_tiled"], z["scales_tiled"], bits, z["wq"].shape[0])
+        assert np.array_equal(w, z["wq"]) and np.array_equal(s.view(np.uint16), z["scales"].view(np.uint16)), f

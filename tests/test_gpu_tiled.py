@@ -43,6 +43,27 @@ def test_tile_weights_matches_the_loop_restatement_and_round_trips(bits, n, k):
     assert np.array_equal(s2.cpu().numpy().view(np.uint16), s.view(np.uint16))
 
 
+def test_tile_weights_reproduces_the_committed_fixtures():
+    import glob
+    import os
+
+    import relax_amd
+
+    files = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "tiled_*.npz")))
+    assert len(files) >= 2
+    for f in files:
+        z = np.load(f)
+        bits, g = int(z["bits"]), int(z["group"])
+        wt, st = _tiled(z["wq"], z["scales"], bits, g)
+        w2, s2 = relax_amd.wq_untile_weights(_dev(z["wq_tiled"]), _dev(z["scales_tiled"]), bits, g, *(
+            z["wq"].shape[0], z["wq"].shape[1] * (32 // bits)))
+        torch.cuda.synchronize()
+        assert np.array_equal(wt.cpu().numpy().view(np.uint32), z["wq_tiled"]), f
+        assert np.array_equal(st.cpu().numpy().view(np.uint16), z["scales_tiled"].view(np.uint16)), f
+        assert np.array_equal(w2.cpu().numpy().view(np.uint32), z["wq"]), f
+        assert np.array_equal(s2.cpu().numpy().view(np.uint16), z["scales"].view(np.uint16)), f
+
+
 GEMV_CASES = [(4, 1, 48, 256), (4, 3, 100, 512), (4, 16, 72, 1024), (4, 8, 4096, 4096), (4, 1, 22016, 4096),
               (4, 16, 4096, 11008), (4, 5, 1000, 8192), (8, 2, 40, 128), (8, 16, 72, 384), (8, 1, 5120, 5120),
               (8, 16, 5120, 13824), (8, 7, 333, 1280)]
