@@ -269,10 +269,12 @@ int launch_skinny(const Problem& p, int variant) {
   if (p.bits == 4) {
     ok = mt <= 1   ? dispatch_variant<4, 1>(p, group_shift, variant)
          : mt == 2 ? dispatch_variant<4, 2>(p, group_shift, variant)
+         : mt == 3 ? dispatch_variant<4, 3>(p, group_shift, variant)
                    : dispatch_variant<4, 4>(p, group_shift, variant);
   } else {
     ok = mt <= 1   ? dispatch_variant<8, 1>(p, group_shift, variant)
          : mt == 2 ? dispatch_variant<8, 2>(p, group_shift, variant)
+         : mt == 3 ? dispatch_variant<8, 3>(p, group_shift, variant)
                    : dispatch_variant<8, 4>(p, group_shift, variant);
   }
   if (!ok) {
