@@ -1,12 +1,15 @@
 // MFMA GEMM for prefill (M > 64) whose weight operand never touches LDS:
 // y[M,N] = x[M,K] @ dequant(Wq,S)^T.
 //
-// Bound: dense float16 MFMA; the design goal is to keep LDS traffic (128 B/clk/CU on
-// gfx950) well below the matrix pipe's appetite.  A workgroup owns a BM x 256 output tile
-// (BM = 128, or 64 when M is too small to give every CU a 128-row tile); all wavefronts share the same BM activation rows (staged in LDS) and
-// each owns 64 distinct weight rows, i.e. a BM x 64 sub-tile of 32x32x16 MFMAs.  The
+// Bound: dense float16 MFMA; the design goal is to keep LDS traffic well below the matrix
+// pipe's appetite.  A workgroup owns a BM x 256 output tile (BM = 128, or 64 when M is too
+// small to give every CU a 128-row tile); all wavefronts share the same BM activation rows
+// (staged in LDS) and each owns 64 distinct weight rows, i.e. a BM x 64 sub-tile of 32x32x16
+// MFMAs.  The two 32-column MFMA tiles of a wavefront hold the even and the odd columns of
+// its 64 (lane col: columns 2 col and 2 col + 1), so a lane finishes with two adjacent outputs
+// of a row and stores them with one 4-byte access.  The
 // MFMA B operand of lane (col = lane % 32, kh = lane / 32) for 16-wide k slice kk is
-// the 8 weights k = k0 + (kh*4 + kk)*8 .. +8 of row `col` -- exactly one packed int4
+// the 8 weights k = k0 + (kh*4 + kk)*8 .. +8 of its row -- exactly one packed int4
 // word, or two int8 words -- so a lane loads the 16 bytes (int4) it needs for a whole
 // 64-wide K step straight from global memory with one buffer load, together with the
 // one group scale that covers them, and dequantizes word by word in registers, to
@@ -24,8 +27,8 @@
 //
 // Pipeline per K step t (four activation stages in LDS; program order is issue order, a
 // handful of independent instructions after every MFMA, fenced with sched_barrier):
-//   global -> registers : activations of step t+4 (t+3 with K groups), packed weights of
-//                         step t+3 (t+2 with two register sets), scales per four steps
+//   global -> registers : activations of step t+4 (t+3 with one register set), packed weights
+//                         of step t+3 (t+2 with two register sets), scales per four steps
 //   registers -> LDS    : activations of step t+2
 //   LDS -> registers    : A fragments of the next k slice (of step t+1 at the end)
 //   dequantize          : one stage each of four pair conversions per MFMA slot
@@ -36,6 +39,13 @@
 // first through LDS.  A stall of one wavefront (barrier, memory wait) is covered by the
 // other one on its SIMD, and a tile takes half as many sequential K steps, which is what
 // counts when M is too small to give every CU a tile.
+//
+// With two wavefronts on a SIMD the one further back in its step gets the higher priority
+// (s_setprio per k slice), so that both reach the step's barrier together.
+//
+// TILED: the packed weights and scales are in the tile-major layout (wq_tiled.hip); only the
+// address arithmetic of the weight and scale loads changes -- 16 lanes then read 256
+// contiguous bytes instead of 16 rows' worth of 16-byte pieces.
 //
 // Shape requirements (checked by the launcher): K a multiple of 256 (at least 512 for K
 // groups), group 32 (int4) or 128 (int8), operands < 1 GiB; other shapes use the other GEMM
