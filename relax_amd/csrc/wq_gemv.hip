@@ -29,6 +29,10 @@
 // The int4 activations are written to LDS already in the pair order
 // (k0,k4)(k1,k5)(k2,k6)(k3,k7) the nibble unpack produces, so the loop has no
 // permutes.
+//
+// TILED: weights and scales are in the tile-major layout (wq_tiled.hip), whose blocks are
+// exactly what a wavefront reads per instruction (D = 2): every load of the weight stream
+// is 1 KB contiguous.  Same lanes, same chunks, same order: bit-identical results.
 #include <algorithm>
 
 #include "wq_device.h"

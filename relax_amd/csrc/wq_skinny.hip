@@ -12,6 +12,9 @@
 // `col` of the tile and the kq-th 16-byte chunk of every 64-byte row segment, so
 // one load instruction covers 16 rows x 64 contiguous bytes.
 //
+// TILED: weights and scales are addressed in the tile-major layout (wq_tiled.hip); a load
+// instruction then reads two runs of 512 contiguous bytes.
+//
 // Tails never branch: activation rows >= M, chunks >= K and k-steps past the
 // wavefront's share are loaded from an out-of-range buffer offset, which returns
 // zeros (zero scale => zero weight, zero activation); weight rows >= N are
