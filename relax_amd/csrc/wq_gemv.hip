@@ -310,7 +310,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
 namespace {
 
 constexpr size_t kLdsPerCu = 160 * 1024;
-constexpr size_t kLdsPerWgMax = 150 * 1024;
+constexpr size_t kLdsPerWgMax = 159 * 1024;  // of the 160 KB a workgroup can address
 
 struct Plan {
   int grid, max_tiles, phase_chunks, lds_stride;
