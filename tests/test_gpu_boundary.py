@@ -284,3 +284,52 @@ def test_layer_chain_captured_in_a_hip_graph_replays_like_eager():
             assert torch.isfinite(got).all()
             assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     vm_harness.set_stream(torch.cuda.current_stream())
+
+
+def test_concurrent_callers_on_their_own_streams():
+    """Several VM threads call the packed entries at once, each on its own stream and its own problem
+    (src/runtime/relax_vm/vm.cc:780-790: a VM runs on its caller's thread).  The stream and the error
+    text are per thread; results must equal the single-threaded ones bit for bit."""
+    import threading
+
+    import relax_amd
+    from relax_amd import lib, vm_harness
+
+    cases = [(4, 1, 4096, 4096), (4, 8, 200, 1024), (8, 40, 136, 512), (4, 200, 520, 1024), (8, 300, 260, 1024)]
+    jobs = []
+    for i, (bits, m, n, k) in enumerate(cases):
+        x, wq, s, g = O.make_case(300 + i, m, n, k, bits)
+        xd, wd, sd = _dev(x), _dev(wq), _dev(s)
+        want = relax_amd.wq_matmul(xd, wd, sd, bits, g)
+        jobs.append((bits, m, n, xd, wd, sd, want))
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(idx):
+        try:
+            bits, m, n, xd, wd, sd, want = jobs[idx]
+            stream = torch.cuda.Stream()
+            vm_harness.set_stream(stream)
+            assert lib.load().mi355x_wq_packed_get_stream() == stream.cuda_stream
+            for it in range(40):
+                y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+                args = [vm_harness.TensorArg(xd), vm_harness.TensorArg(wd, as_uint32=True), vm_harness.TensorArg(sd),
+                        vm_harness.TensorArg(y)]
+                vm_harness.call_packed("mi355x_q%df16_matmul" % bits, args)
+                if it % 8 == idx % 8:   # a failing call in between: the message belongs to this thread
+                    with pytest.raises(vm_harness.PackedError, match="expects 4 arguments, got 3"):
+                        vm_harness.call_packed("mi355x_q%df16_matmul" % bits, args[:3])
+                stream.synchronize()
+                if not torch.equal(y.view(torch.int16), want.view(torch.int16)):
+                    errors.append((idx, it, "result differs"))
+        except BaseException as e:  # noqa: BLE001 - reported by the main thread
+            errors.append((idx, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(jobs))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    assert not any(t.is_alive() for t in threads), "a caller thread did not finish"
+    assert not errors, errors[:3]
+    vm_harness.set_stream()
