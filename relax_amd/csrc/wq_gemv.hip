@@ -34,6 +34,7 @@
 // exactly what a wavefront reads per instruction (D = 2): every load of the weight stream
 // is 1 KB contiguous.  Same lanes, same chunks, same order: bit-identical results.
 #include <algorithm>
+#include <type_traits>
 
 #include "wq_device.h"
 #include "wq_internal.h"
@@ -60,7 +61,7 @@ struct GemvArgs {
   Epilogue ep;
 };
 
-template <int BITS, int WAVES, int D, int SPL, bool TILED>
+template <int BITS, int WAVES, int D, int SPL, bool TILED, bool ROWS>
 // (scalar kernel arguments instead of one struct: the first 16 dwords -- the operand pointers
 // and the shape -- are preloaded into SGPRs at wavefront launch, which takes the argument fetch
 // out of the start-up latency of a 5 - 15 us kernel)
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     const int cnt = max(ss_end - ss_begin, 0);  // super steps per tile for this wavefront
 
     // ---- stage this phase's activations (zero padded to a whole k-step) ---------------
-    // The first two vectors per thread are requested before the first weights and
+    // The first batch of vectors per thread is requested before the first weights and
     // stored after them: global loads retire in order, so the LDS fill does not wait
     // for the much slower first weight loads.
     GemvBuf<D, SPL> b0, b1;
@@ -221,39 +222,83 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
       const int kbase = chunk_base * CH;
       const int kpad = ((ph_chunks + 3) / 4) * 4 * CH;
       const int vec_per_row = kpad / 8;
-      const int total = M * vec_per_row;
-      auto x_load = [&](int idx) -> u32x4 {
-        const int m = idx / vec_per_row, kv = idx - m * vec_per_row;
-        const bool ok = idx < total && kbase + kv * 8 < K;
-        return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
-      };
-      auto x_store = [&](int idx, u32x4 v) {
-        if (idx >= total) return;
-        const int m = idx / vec_per_row, kv = idx - m * vec_per_row;
+      auto permute_x = [&](u32x4 v) -> u32x4 {
         if constexpr (BITS == 4) {
           u32x4 p;
           p[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
           p[1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
           p[2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
           p[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
-          v = p;
+          return p;
+        } else {
+          return v;
         }
-        *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = v;
       };
       if (ph > 0) __syncthreads();  // every wavefront is done reading the previous phase
-      const u32x4 x0 = x_load(tid), x1 = x_load(tid + NT);
-      __builtin_amdgcn_sched_barrier(0);
-      load_super(b0, 0, ss_begin, chunk_base, ss_end);
-      __builtin_amdgcn_sched_barrier(0);
-      x_store(tid, x0);
-      x_store(tid + NT, x1);
-      // the rest four vectors at a time: all four requests are in flight before the first store
-      for (int idx = tid + 2 * NT; idx < total; idx += 4 * NT) {
-        const u32x4 v0 = x_load(idx), v1 = x_load(idx + NT), v2 = x_load(idx + 2 * NT), v3 = x_load(idx + 3 * NT);
-        x_store(idx, v0);
-        x_store(idx + NT, v1);
-        x_store(idx + 2 * NT, v2);
-        x_store(idx + 3 * NT, v3);
+      if constexpr (!ROWS) {
+        // one or two rows, or rows longer than the workgroup has threads: a flat index over (row, column),
+        // two vectors per thread ahead of the weights
+        // (every extra request, even one that is masked off, takes its turn in the memory pipeline
+        // ahead of the first weights: the batch-1 start-up is kept as short as it can be)
+        const int total = M * vec_per_row;
+        auto x_load = [&](int idx) -> u32x4 {
+          const int m = idx / vec_per_row, kv = idx - m * vec_per_row;
+          const bool ok = idx < total && kbase + kv * 8 < K;
+          return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
+        };
+        auto x_store = [&](int idx, u32x4 v) {
+          if (idx >= total) return;
+          const int m = idx / vec_per_row, kv = idx - m * vec_per_row;
+          *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = permute_x(v);
+        };
+        const u32x4 x0 = x_load(tid), x1 = x_load(tid + NT);
+        __builtin_amdgcn_sched_barrier(0);
+        load_super(b0, 0, ss_begin, chunk_base, ss_end);
+        __builtin_amdgcn_sched_barrier(0);
+        x_store(tid, x0);
+        x_store(tid + NT, x1);
+        for (int idx = tid + 2 * NT; idx < total; idx += 4 * NT) {
+          const u32x4 v0 = x_load(idx), v1 = x_load(idx + NT), v2 = x_load(idx + 2 * NT), v3 = x_load(idx + 3 * NT);
+          x_store(idx, v0);
+          x_store(idx + NT, v1);
+          x_store(idx + 2 * NT, v2);
+          x_store(idx + 3 * NT, v3);
+        }
+      } else {
+        // more rows, and a phase of at most one vector per thread and row (launch_one checks): a thread
+        // stages its column of RM rows per batch.  No address needs a division (with the flat index the
+        // divisions alone cost half a microsecond at eight rows), the RM requests of the first batch are
+        // in flight together and all go out before the first weights.  (Measured alternatives, all
+        // slower: part of the batch behind the weights -- it returns after them, i.e. after a cold trip
+        // to HBM; sixteen in flight; requests under per-vector branches, which the wait-count
+        // insertion serialises.)
+        auto x_load = [&](int m, int kv) -> u32x4 {
+          const bool ok = m < M && kv < vec_per_row && kbase + kv * 8 < K;
+          return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
+        };
+        auto x_store = [&](int m, int kv, u32x4 v) {
+          if (m >= M || kv >= vec_per_row) return;
+          *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = permute_x(v);
+        };
+        auto stage = [&](auto rmc) {
+          constexpr int RM = decltype(rmc)::value;
+          u32x4 xv[RM];
+#pragma unroll
+          for (int r = 0; r < RM; ++r) xv[r] = x_load(r, tid);
+          __builtin_amdgcn_sched_barrier(0);
+          load_super(b0, 0, ss_begin, chunk_base, ss_end);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int r = 0; r < RM; ++r) x_store(r, tid, xv[r]);
+          for (int m0 = RM; m0 < M; m0 += RM) {
+#pragma unroll
+            for (int r = 0; r < RM; ++r) xv[r] = x_load(m0 + r, tid);
+#pragma unroll
+            for (int r = 0; r < RM; ++r) x_store(m0 + r, tid, xv[r]);
+          }
+        };
+        if (M <= 4) stage(std::integral_constant<int, 4>{});
+        else stage(std::integral_constant<int, 8>{});
       }
     }
     __syncthreads();
@@ -366,13 +411,21 @@ int launch_one(const Problem& p, int group_shift, const Plan& plan) {
   a.max_tiles = plan.max_tiles;
   a.phase_chunks = plan.phase_chunks;
   a.ep = Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation};
-  static bool lds_ok[kMaxDevices] = {false};
-  if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED>, (int)kLdsPerWgMax, lds_ok))
-    return kFailed;
-  hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED>), dim3(plan.grid), dim3(WAVES * 64),
-                     plan.lds_bytes, p.stream, a.x, a.wq, a.scales, a.y, a.M, a.N, a.K, a.group_shift,
-                     a.zero_point, a.lds_stride, a.tiles, a.max_tiles, a.phase_chunks, a.ep);
-  return kLaunched;
+  // two builds of the kernel, by the way the activations are staged: flat index / a column per thread
+  auto go = [&](auto rows) -> int {
+    constexpr bool ROWS = decltype(rows)::value;
+    static bool lds_ok[kMaxDevices] = {false};
+    if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS>, (int)kLdsPerWgMax, lds_ok))
+      return kFailed;
+    hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS>), dim3(plan.grid), dim3(WAVES * 64),
+                       plan.lds_bytes, p.stream, a.x, a.wq, a.scales, a.y, a.M, a.N, a.K, a.group_shift,
+                       a.zero_point, a.lds_stride, a.tiles, a.max_tiles, a.phase_chunks, a.ep);
+    return kLaunched;
+  };
+  constexpr int ch = 128 / BITS;
+  const int phase_vectors = (plan.phase_chunks + 3) / 4 * 4 * ch / 8;  // 16-byte vectors per staged row
+  if (p.m <= 2 || phase_vectors > WAVES * 64) return go(std::false_type{});
+  return go(std::true_type{});
 }
 
 // D chunks per lane need K to be a multiple of 4*D chunks, and the lane's D
