@@ -144,9 +144,10 @@ def config_table(torch, dev, args) -> int:
     return 0
 
 
-def audit_dispatch(torch, dev) -> int:
+def audit_dispatch(torch, dev, tiled: bool = False) -> int:
     """Default kernel selection against every explicit (family, variant) for M <= 64: the tool the
-    selection rules were checked with.  One HIP graph over 2-6 distinct weight sets per timing."""
+    selection rules were checked with.  One HIP graph over 2-6 distinct weight sets per timing.
+    `tiled`: the same on weights in the tile-major layout (their own selection rules)."""
     import relax_amd
     from relax_amd import lib
 
@@ -171,8 +172,8 @@ def audit_dispatch(torch, dev) -> int:
 
     shapes = [(2048, 4096), (4096, 2048), (4096, 4096), (5120, 5120), (6144, 4096), (8192, 4096), (8192, 8192),
               (11008, 4096), (16384, 4096), (32000, 4096), (4096, 16384)]
-    cands = [(lib.KERNEL_GEMV, v) for v in (14, 15, 24, 25)] + [(lib.KERNEL_SKINNY, v) for v in (1, 2, 5, 7, 9)] \
-        + [(lib.KERNEL_GEMM, 25)]
+    cands = [(lib.KERNEL_GEMV, v) for v in ((15, 25) if tiled else (14, 15, 24, 25))] \
+        + [(lib.KERNEL_SKINNY, v) for v in ((1, 2, 5, 7, 9, 11) if tiled else (1, 2, 5, 7, 9))] + [(lib.KERNEL_GEMM, 25)]
     names = {lib.KERNEL_GEMV: "gemv", lib.KERNEL_SKINNY: "skinny", lib.KERNEL_GEMM: "gemm"}
     behind = 0
     for bits, group in ((4, 32), (8, 128)):
@@ -180,6 +181,8 @@ def audit_dispatch(torch, dev) -> int:
             nsets = max(2, min(6, (400 << 20) // (n * k * bits // 8)))
             sets = [(torch.randint(-2**31, 2**31 - 1, (n, k * bits // 32), dtype=torch.int32, device=dev),
                      (torch.rand((n, k // group), device=dev) * 0.015 + 0.005).to(torch.float16)) for _ in range(nsets)]
+            if tiled:
+                sets = [relax_amd.wq_tile_weights(wq, sc, bits, group) for wq, sc in sets]
             for m in (1, 4, 8, 16, 24, 32, 48, 64):
                 x = torch.randn((m, k), device=dev).to(torch.float16)
                 y = torch.empty((m, n), dtype=torch.float16, device=dev)
@@ -187,7 +190,8 @@ def audit_dispatch(torch, dev) -> int:
                 def run(fam, var):
                     def f():
                         for wq, sc in sets:
-                            relax_amd.wq_matmul(x, wq, sc, bits, group, out=y, kernel=fam, variant=var)
+                            relax_amd.wq_matmul(x, wq, sc, bits, group, out=y, kernel=fam, variant=var,
+                                                tiled_n=n if tiled else None)
                     return graph_us(f, nsets)
 
                 run(0, 0)  # first use of a kernel on this device: code load, LDS attribute
@@ -203,13 +207,14 @@ def audit_dispatch(torch, dev) -> int:
                     if t < best:
                         best, best_name = t, "%s %d" % (names[fam], var)
                 base = min(base, run(0, 0))  # again after the candidates: clocks and caches have settled
-                line = {"case": "q%df16 M=%d N=%d K=%d" % (bits, m, n, k), "default_us": round(base, 2),
+                line = {"case": "q%df16 M=%d N=%d K=%d%s" % (bits, m, n, k, " tile-major" if tiled else ""), "default_us": round(base, 2),
                         "best_us": round(best, 2), "best": best_name, "behind": round(base / best - 1.0, 3)}
                 if base > 1.08 * best:
                     behind += 1
                     print(json.dumps(line), flush=True)
             del sets
-    print(json.dumps({"cases": 2 * len(shapes) * 8, "more_than_8_percent_behind": behind}), flush=True)
+    print(json.dumps({"layout": "tile-major" if tiled else "canonical", "cases": 2 * len(shapes) * 8,
+                      "more_than_8_percent_behind": behind}), flush=True)
     return 0
 
 
@@ -290,6 +295,8 @@ def main() -> int:
                     help="instead of the benchmark: for 11 shapes x 8 row counts (1..64) per quantization, time the "
                          "library's default kernel choice against every explicit variant of every family and print "
                          "the cases where the default is more than 8 %% behind the best")
+    ap.add_argument("--audit-tile-major", action="store_true",
+                    help="the same audit on weights in the tile-major layout")
     ap.add_argument("--probe-mfma", action="store_true",
                     help="instead of the benchmark: time a register-resident float16 MFMA loop on operands "
                          "of several distributions (what the matrix pipes sustain as a function of the data "
@@ -314,8 +321,8 @@ def main() -> int:
         return probe_mfma(torch, dev)
     if args.configs:
         return config_table(torch, dev, args)
-    if args.audit_dispatch:
-        return audit_dispatch(torch, dev)
+    if args.audit_dispatch or args.audit_tile_major:
+        return audit_dispatch(torch, dev, tiled=args.audit_tile_major)
 
     if args.calibrate_copy:
         src = torch.ones(64 * 1024 * 1024, dtype=torch.int32, device=dev)  # 256 MiB read + 256 MiB written

@@ -118,8 +118,10 @@ MI355X_WQ_API int mi355x_wq_dequantize(const mi355x_wq_desc* desc, const void* w
  * python/tvm/relax/transform/transform.py:210-233).  Defined for the two benchmark quantizations:
  * int4 / group 32 with K % 256 == 0 and int8 / group 128 with K % 128 == 0.  Both tiled buffers
  * have the size of the canonical ones with N rounded up to a multiple of 16 (rows past N are zero).
- * Tiling followed by untiling returns the input bit for bit, and the matmul computes the same
- * values in the same order from either layout (bit-identical outputs). */
+ * Tiling followed by untiling returns the input bit for bit, and every kernel family computes the
+ * same values in the same order from either layout (bit-identical outputs for the same family; the
+ * automatic choice of family has crossovers of its own per layout, and two families differ in the
+ * order of the float32 additions). */
 MI355X_WQ_API int mi355x_wq_tiled_sizes(const mi355x_wq_desc* desc, int64_t* wq_bytes, int64_t* scales_bytes);
 
 /* canonical (wq, scales) -> tile-major (wq_tiled, scales_tiled); all four 16-byte aligned, device. */

@@ -134,7 +134,25 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
     // that the staging kernel's start-up costs more than it saves: 4096 x 2048, 5.6 against 4.9 us)
     const bool big_x = x_bytes > 64 * 1024 && tiles <= 256 && d->k < 16384;
     const bool tiny = tiles <= 256 && d->k <= 2048;
-    if (!big_x && !tiny) return MI355X_WQ_KERNEL_GEMV;
+    // Tile-major weights, at most two row tiles per CU: the staging is spread over so few tiles that the
+    // register-activation kernel, whose loads are as contiguous on this layout, wins -- int8 at every
+    // batch (5120 x 5120: 8.0 - 10.6 us against 9.4 - 12.6 us; 5120 x 13824 at 8 rows: 19.2 against
+    // 24.1 us); int4 with rows of up to 2 KB at up to 8 rows (4096 x 4096: 4.3 against 4.6 us at batch 1)
+    // or once there is more than one tile per CU; int4 with longer rows from 8 rows on, from 4 with more
+    // than one tile per CU.  From 640 tiles on the staging kernel is ahead again (10240 x 4096: 7.9
+    // against 8.8 us).
+    bool few_tiles = false;
+    if (tiled && tiles <= 2 * cu_count() && d->k < 16384) {
+      const bool long_rows = d->k * d->bits / 8 > 4096, over_one = tiles > cu_count();
+      few_tiles = d->bits == 8 || (!long_rows && (m <= 8 || over_one)) || (long_rows && (m >= 8 || (m >= 4 && over_one)));
+    }
+    // (and with up to four tiles per CU at 12 rows or more, where the staging kernel's time has grown with
+    // the rows and the other's has not: 16384 x 4096 at 16 rows, 11.4 against 13.4 us)
+    if (tiled && m >= 12 && tiles > 2 * cu_count() && tiles <= 4 * cu_count() && d->k < 16384) few_tiles = true;
+    // (rows of 16384 and more, one tile per CU: the staging kernel at batch 1 - 4, 17.7 against 19.8 us, the
+    // other from 8 rows on, 14.7 against 16.7 us)
+    if (tiled && d->k >= 16384 && tiles <= cu_count() && m >= 8) few_tiles = true;
+    if (!big_x && !tiny && !few_tiles) return MI355X_WQ_KERNEL_GEMV;
   }
   if (m > kSkinnyMaxM) return MI355X_WQ_KERNEL_GEMM;
   // 17..64 rows.  The skinny kernel re-reads the activations from L2 once per 16-row weight tile, so

@@ -264,7 +264,9 @@ int launch_skinny(const Problem& p, int variant) {
     // tiles per workgroup; many: two tiles per 8-wave workgroup for one row block, else four.
     const int64_t tiles = (p.n + 15) / 16;
     if (tiles <= 256) variant = 1;
-    else if (tiles <= 512) variant = p.bits == 4 ? 5 : 2;  // (one tile per workgroup is 1.5 - 1.8x slower here)
+    // (one tile per workgroup is 1.5 - 1.8x slower here; int8 at up to 4 rows on tile-major weights:
+    // eight wavefronts, 3 - 5 % ahead)
+    else if (tiles <= 512) variant = (p.bits == 4 || (p.tiled && p.m <= 4)) ? 5 : 2;
     else if (tiles <= 1024) variant = 7;
     else variant = mt == 1 ? 5 : 11;  // several rounds of workgroups: eight tiles share one pass over the activations
   }
