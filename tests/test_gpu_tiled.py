@@ -177,3 +177,32 @@ def test_seeded_random_shapes_on_tile_major_weights(chunk):
         want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
         assert_close(got.cpu().numpy(), want, (bits, m, n, k))
         assert_fused(fused.cpu().numpy(), got.cpu().numpy(), want, bias, "relu", res, ("fused", bits, m, n, k))
+
+
+def test_tile_major_weights_of_one_and_a_half_gib():
+    """The largest weight operand: 98309 x 16384 int8 (1.5 GiB, ragged last tile).  Tiling round-trips bit
+    for bit, the register-activation kernel gives the canonical layout's bits (whose parity
+    with the oracle test_weights_between_one_and_two_gib checks), and more than 64 rows are refused:
+    only the direct-weight GEMM reads this layout, and it addresses operands below 1 GiB."""
+    import relax_amd
+    from relax_amd import lib
+
+    bits, group, n, k = 8, 128, 98309, 16384
+    gen = torch.Generator(device="cuda").manual_seed(29)
+    wq = torch.randint(-2**31, 2**31 - 1, (n, k * bits // 32), dtype=torch.int32, device="cuda", generator=gen)
+    s = (torch.rand((n, k // group), device="cuda", generator=gen) * 0.008 + 0.002).to(torch.float16)
+    wq_t, s_t = relax_amd.wq_tile_weights(wq, s, bits, group)
+    wq_back, s_back = relax_amd.wq_untile_weights(wq_t, s_t, bits, group, n, k)
+    assert torch.equal(wq_back, wq) and torch.equal(s_back.view(torch.int16), s.view(torch.int16))
+    del wq_back, s_back
+    # (6145 row tiles are more than the decode kernel's LDS slots hold: every batch runs the
+    # register-activation kernel, as on the canonical layout)
+    for m, kernel in ((1, lib.KERNEL_SKINNY), (8, lib.KERNEL_SKINNY), (32, lib.KERNEL_SKINNY), (4, lib.KERNEL_AUTO)):
+        x = (torch.randn((m, k), device="cuda", generator=gen) * 0.25).to(torch.float16)
+        y_c = relax_amd.wq_matmul(x, wq, s, bits, group, kernel=kernel)
+        y_t = relax_amd.wq_matmul(x, wq_t, s_t, bits, group, kernel=kernel, tiled_n=n)
+        torch.cuda.synchronize()
+        assert torch.equal(y_c.view(torch.int16), y_t.view(torch.int16)), (m, kernel)
+    x = torch.zeros((128, k), dtype=torch.float16, device="cuda")
+    with pytest.raises(lib.WqError, match="direct-weight kernel"):
+        relax_amd.wq_matmul(x, wq_t, s_t, bits, group, tiled_n=n)
