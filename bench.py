@@ -283,6 +283,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--no-epilogue", action="store_true", help="skip the fused-residual leg")
+    ap.add_argument("--no-ksplit", action="store_true", help="skip the caller-workspace (K split) leg")
     ap.add_argument("--no-tiled", action="store_true", help="skip the tile-major-weights decode leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times (a kernel of known HBM "
@@ -525,6 +526,42 @@ def main() -> int:
                         "residual add h += y (one HIP graph)" % args.layers,
             "us_per_projection_separate_add": round(times[False] * 1e3 / pairs, 3),
             "us_per_projection_fused": round(times[True] * 1e3 / pairs, 3),
+            "speedup": round(times[False] / times[True], 3)}
+
+    if not args.no_ksplit:
+        # the down projection (4096 x 11008) of every layer at 8 rows: the one case of this step where a
+        # caller workspace lets the decode kernel split K across workgroups (mi355x_wq_matmul_ws)
+        m, k = 8, 11008
+        downs = [mats[3] for mats in layers]
+        need = relax_amd.wq_workspace_bytes(4, 32, downs[0][2], k, m)
+        wsp = relax_amd.wq_workspace(need)
+        yk = torch.empty((m, downs[0][2]), dtype=torch.float16, device=dev)
+
+        def down_pass(ws):
+            for wq, s, n, kk in downs:
+                relax_amd.wq_matmul(xs[(m, k)], wq, s, 4, 32, out=yk, workspace=ws)
+
+        times = {}
+        with torch.cuda.stream(stream):
+            for ws in (None, wsp):
+                down_pass(ws)
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=stream):
+                    down_pass(ws)
+                gr.replay()
+                torch.cuda.synchronize()
+                r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                r0.record(stream)
+                for _ in range(args.steps):
+                    gr.replay()
+                r1.record(stream)
+                torch.cuda.synchronize()
+                times[ws is not None] = r0.elapsed_time(r1) / args.steps * 1e3 / len(downs)
+        result["k_split"] = {
+            "workload": "down projection 4096x11008 of %d layers at batch 8, without and with a caller "
+                        "workspace (K split over 2 workgroups per tile, %d bytes)" % (args.layers, need),
+            "us_plain": round(times[False], 3), "us_with_workspace": round(times[True], 3),
             "speedup": round(times[False] / times[True], 3)}
 
     if not args.no_cpu:

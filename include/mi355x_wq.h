@@ -144,6 +144,25 @@ MI355X_WQ_API int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const vo
                                            const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y,
                                            int64_t m, void* stream, int kernel);
 
+/* Decode with a caller workspace: for M <= 16 and projections whose 16-row tiles leave CUs idle for
+ * whole rounds (5120 rows: 320 tiles on 256 CUs) or whose activations are large against one tile per CU,
+ * the decode kernel splits K over two to four workgroups per tile; each writes a float32 partial tile
+ * to the workspace, and the last to arrive adds them in the order of their K windows (the result does
+ * not depend on the order of arrival), applies the epilogue and stores.  5120 x 13824 int8 at batch 1:
+ * 22 -> 16 us.  The reference's counterpart is CUTLASS split-K, whose workspace the generated host code
+ * allocates per call (python/tvm/contrib/cutlass/build.py:335, conv2d_operation.py:417-418); here the
+ * caller owns it, so that nothing is allocated under a stream capture or in a serving loop.
+ *
+ * mi355x_wq_workspace_bytes: the size mi355x_wq_matmul_ws needs to split K for (desc, m, layout); 0 if it
+ * would not split (then the call equals mi355x_wq_matmul_fused / _tiled), -1 on an invalid descriptor.
+ * Workspace rules: device memory, 16-byte aligned, all zero before its first use (the kernel leaves it
+ * ready for the next call); calls that share a workspace must not overlap in time (one stream, or
+ * ordered by events); a workspace that is NULL or smaller than required disables the split for that call. */
+MI355X_WQ_API int64_t mi355x_wq_workspace_bytes(const mi355x_wq_desc* desc, int64_t m, int tiled);
+MI355X_WQ_API int mi355x_wq_matmul_ws(const mi355x_wq_desc* desc, const void* x, const void* wq, const void* scales,
+                                     const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int tiled,
+                                     void* workspace, int64_t workspace_bytes);
+
 /* Validates a descriptor and a row count without touching the GPU: 0 if
  * mi355x_wq_matmul would accept them. */
 MI355X_WQ_API int mi355x_wq_check(const mi355x_wq_desc* desc, int64_t m);

@@ -119,6 +119,16 @@ MI355X_WQ_API int mi355x_q4f16_matmul_tiled(mi355x_tvm_value* args, int* type_co
 MI355X_WQ_API int mi355x_q8f16_matmul_tiled(mi355x_tvm_value* args, int* type_codes, int num_args,
                               mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
 
+/* Decode with a workspace (mi355x_wq_matmul_ws in mi355x_wq.h) as a destination-passing extern:
+ *   matmul_ws(x[M, K] f16, wq[N, K*bits/32] u32, scales[N, K/group] f16, workspace[bytes] u8, y[M, N] f16)
+ * The workspace is a 1-d uint8 tensor the module allocates once (R.builtin.alloc_tensor, zero filled),
+ * sized with mi355x_wq_workspace_bytes for its largest projection, and passes to every call on the
+ * stream; an empty or too small one makes the call equal to matmul. */
+MI355X_WQ_API int mi355x_q4f16_matmul_ws(mi355x_tvm_value* args, int* type_codes, int num_args,
+                              mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
+MI355X_WQ_API int mi355x_q8f16_matmul_ws(mi355x_tvm_value* args, int* type_codes, int num_args,
+                              mi355x_tvm_value* out_ret_value, int* out_ret_tcode, void* resource_handle);
+
 /*
  * Per-symbol call description for generated entries.  FuseOpsByPattern orders the
  * parameters of a composite function by first use

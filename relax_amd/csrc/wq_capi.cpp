@@ -199,7 +199,8 @@ int mi355x_wq_select_kernel(const mi355x_wq_desc* desc, int64_t m) {
 namespace {
 
 int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
-                      const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int kernel, bool tiled);
+                      const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int kernel, bool tiled,
+                      void* workspace = nullptr, int64_t workspace_bytes = 0);
 
 }  // namespace
 
@@ -213,6 +214,23 @@ int mi355x_wq_matmul_tiled(const mi355x_wq_desc* desc, const void* x, const void
                            const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y, int64_t m,
                            void* stream) {
   return matmul_any_layout(desc, x, wq_tiled, scales_tiled, ep, y, m, stream, MI355X_WQ_KERNEL_AUTO, true);
+}
+
+int64_t mi355x_wq_workspace_bytes(const mi355x_wq_desc* desc, int64_t m, int tiled) {
+  using namespace wq;
+  if (!check_desc(desc, m)) return -1;
+  if (tiled != 0 && !tiled_layout_defined(desc->bits, desc->group, desc->k)) return 0;
+  if (m == 0 || desc->n == 0 || desc->k == 0) return 0;
+  Problem p{nullptr, nullptr, nullptr, nullptr, m, desc->n, desc->k, desc->bits, desc->group, desc->zero_point, nullptr};
+  p.tiled = tiled != 0;
+  return gemv_split_workspace_bytes(p);
+}
+
+int mi355x_wq_matmul_ws(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
+                        const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int tiled, void* workspace,
+                        int64_t workspace_bytes) {
+  return matmul_any_layout(desc, x, wq_, scales, ep, y, m, stream, MI355X_WQ_KERNEL_AUTO, tiled != 0, workspace,
+                           workspace_bytes);
 }
 
 int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const void* x, const void* wq_tiled,
@@ -269,7 +287,8 @@ int mi355x_wq_untile_weights(const mi355x_wq_desc* desc, const void* wq_tiled, c
 namespace {
 
 int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
-                      const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int kernel, bool tiled) {
+                      const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int kernel, bool tiled,
+                      void* workspace, int64_t workspace_bytes) {
   using namespace wq;
   if (!check_desc(desc, m)) return -1;
   if (ep != nullptr) {
@@ -309,6 +328,14 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
       return -1;
     }
     p.tiled = true;
+  }
+  if (workspace != nullptr && family == MI355X_WQ_KERNEL_AUTO) {
+    // a caller workspace allows the decode kernel's K split where it pays; everything else is as without
+    if (!check_ptr(workspace, "workspace", 16)) return -1;
+    const int rc = launch_gemv_split(p, workspace, workspace_bytes);
+    if (rc != 0) return rc < 0 ? -1 : 0;
+  }
+  if (tiled) {
     // the same choice as for canonical weights; the kernels that read the layout are the decode
     // kernel, the skinny kernel and the direct-weight GEMM (which needs K % 256 == 0)
     switch (family == MI355X_WQ_KERNEL_AUTO ? select_kernel(desc, m, true) : family) {

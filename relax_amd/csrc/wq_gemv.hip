@@ -61,14 +61,14 @@ struct GemvArgs {
   Epilogue ep;
 };
 
-template <int BITS, int WAVES, int D, int SPL, bool TILED, bool ROWS>
+template <int BITS, int WAVES, int D, int SPL, bool TILED, bool ROWS, bool KSPLIT>
 // (scalar kernel arguments instead of one struct: the first 16 dwords -- the operand pointers
 // and the shape -- are preloaded into SGPRs at wavefront launch, which takes the argument fetch
 // out of the start-up latency of a 5 - 15 us kernel)
 __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     const half_t* x_, const uint32_t* wq_, const half_t* scales_, half_t* y_, int M_, int N_, int K_,
     int group_shift_, int zero_point_, int lds_stride_, int tiles_, int max_tiles_, int phase_chunks_,
-    const Epilogue ep_) {
+    const Epilogue ep_, int ksplit_, float* partials_, unsigned int* counters_) {
   GemvArgs a;
   a.x = x_;
   a.wq = wq_;
@@ -110,8 +110,14 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
   const rsrc_t rs = make_rsrc(a.scales, n_stored * groups_per_row * 2u);
   const rsrc_t rx = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
 
+  // Tiles of this workgroup: tile0, tile0 + tstride, ...  With the K split, R consecutive workgroups
+  // share a tile list and each walks its own window of K (phase_chunks chunks from kr * phase_chunks).
   const int G = gridDim.x;
-  const int my_tiles = (a.tiles - (int)blockIdx.x + G - 1) / G;  // tiles blockIdx.x, +G, +2G, ...
+  const int R = KSPLIT ? ksplit_ : 1;
+  const int kr = KSPLIT ? (int)blockIdx.x % R : 0;
+  const int tile0 = KSPLIT ? (int)blockIdx.x / R : (int)blockIdx.x;
+  const int tstride = KSPLIT ? G / R : G;
+  const int my_tiles = (a.tiles - tile0 + tstride - 1) / tstride;
 
   const Q4Consts qc = make_q4_consts(a.zero_point);
   const half_t* xrow = xs + (size_t)(col < M ? col : 0) * a.lds_stride;
@@ -124,7 +130,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
       // contiguously.  Scales: int4 / group 32 one 4-byte pair per lane, int8 / group 128 one
       // float16 per (row, super step).
       const uint32_t nsuper_all = (uint32_t)nchunks / (4 * D);
-      const uint32_t item = (uint32_t)(blockIdx.x + i * G) * nsuper_all + (uint32_t)(chunk_base / (4 * D) + ss);
+      const uint32_t item = (uint32_t)(tile0 + i * tstride) * nsuper_all + (uint32_t)(chunk_base / (4 * D) + ss);
       const bool ok = (i < my_tiles) && (ss < ss_end) && (chunk_base + ss * 4 * D < nchunks);
       const uint32_t woff = ok ? item * (D * 1024u) + (uint32_t)lane * 16u : kOobOffset;
 #pragma unroll
@@ -133,7 +139,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
       else b.sc[0] = load_b32(rs, ok ? (item * 64u + (uint32_t)lane) * 4u : kOobOffset);
       return;
     }
-    const int n = min((int)(blockIdx.x + i * G) * 16 + col, N - 1);  // rows past N: computed, not stored
+    const int n = min((tile0 + i * tstride) * 16 + col, N - 1);  // rows past N: computed, not stored
     const int chunk0 = chunk_base + ss * 4 * D + kq * D;
     // D > 1 is only launched when K is a multiple of 4*D chunks, so a lane's D
     // chunks are valid together; D == 1 checks its single chunk.
@@ -203,9 +209,9 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     acc = float4_t{0.f, 0.f, 0.f, 0.f};
   };
 
-  const int nphases = (nchunks + a.phase_chunks - 1) / a.phase_chunks;
+  const int nphases = KSPLIT ? 1 : (nchunks + a.phase_chunks - 1) / a.phase_chunks;
   for (int ph = 0; ph < nphases; ++ph) {
-    const int chunk_base = ph * a.phase_chunks;
+    const int chunk_base = (KSPLIT ? kr : ph) * a.phase_chunks;
     const int ph_chunks = min(a.phase_chunks, nchunks - chunk_base);
     const int nsuper = (ph_chunks + 4 * D - 1) / (4 * D);
     const int per_wave = (nsuper + WAVES - 1) / WAVES;
@@ -339,16 +345,57 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
 
   // ---- sum the wavefronts' partial tiles, convert, store -----------------------------
   __syncthreads();
-  for (int idx = tid; idx < my_tiles * 256; idx += NT) {
-    const int i = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
-    const int m = 4 * (l >> 4) + r;
-    const int n = (int)(blockIdx.x + i * G) * 16 + (l & 15);
-    if (m < M && n < N) {
+  if constexpr (!KSPLIT) {
+    for (int idx = tid; idx < my_tiles * 256; idx += NT) {
+      const int i = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
+      const int m = 4 * (l >> 4) + r;
+      const int n = (tile0 + i * tstride) * 16 + (l & 15);
+      if (m < M && n < N) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) sum += slots[((size_t)(i * WAVES + w) * 4 + r) * 64 + l];
+        store_out(a.ep, a.y, m, n, N, sum);
+      }
+    }
+  } else {
+    // K split over R workgroups: every workgroup writes its float32 partial tile (1 KB) to the
+    // workspace and counts itself in; the one that finds R - 1 others counted adds the R partials in
+    // the order of their K windows -- whoever arrives last, the sum is the same -- applies the
+    // epilogue, stores, and returns the counter to zero for the next launch.  Nobody waits for anybody.
+    //
+    // Visibility across the chip's eight L2s without cache-wide fences (a device-scope fence writes
+    // back and invalidates a whole L2; one per wavefront cost 65 us per launch): the partial tiles and
+    // the counters are only ever touched by device-scope atomic stores, loads and adds, which are
+    // performed at the memory side of the L2s; a workgroup's stores have completed (vmcnt(0)) before
+    // the barrier after which its count goes out.
+    for (int idx = tid; idx < my_tiles * 256; idx += NT) {
+      const int i = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
       float sum = 0.f;
 #pragma unroll
       for (int w = 0; w < WAVES; ++w) sum += slots[((size_t)(i * WAVES + w) * 4 + r) * 64 + l];
-      store_out(a.ep, a.y, m, n, N, sum);
+      __hip_atomic_store(&partials_[((size_t)(tile0 + i * tstride) * R + kr) * 256 + (idx & 255)], sum,
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    int* const last = reinterpret_cast<int*>(slots);  // (the slots have been read)
+    if (tid < my_tiles)
+      last[tid] = __hip_atomic_fetch_add(&counters_[tile0 + tid * tstride], 1u, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(R - 1);
+    __syncthreads();
+    for (int idx = tid; idx < my_tiles * 256; idx += NT) {
+      const int i = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
+      if (!last[i]) continue;
+      const int m = 4 * (l >> 4) + r;
+      const int n = (tile0 + i * tstride) * 16 + (l & 15);
+      float* const part = partials_ + (size_t)(tile0 + i * tstride) * R * 256 + (idx & 255);
+      float sum = 0.f;
+      for (int q = 0; q < R; ++q) sum += __hip_atomic_load(part + q * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (m < M && n < N) store_out(a.ep, a.y, m, n, N, sum);
+    }
+    __syncthreads();
+    if (tid < my_tiles && last[tid])
+      __hip_atomic_store(&counters_[tile0 + tid * tstride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -394,8 +441,8 @@ bool make_plan(const Problem& p, int wgs_per_cu, Plan* out) {
 // the kernel was launched, or a runtime call failed (error already set).
 enum { kNotApplicable = 0, kLaunched = 1, kFailed = -1 };
 
-template <int BITS, int WAVES, int D, int SPL, bool TILED = false>
-int launch_one(const Problem& p, int group_shift, const Plan& plan) {
+template <int BITS, int WAVES, int D, int SPL, bool TILED = false, bool KSPLIT = false>
+int launch_one(const Problem& p, int group_shift, const Plan& plan, int ksplit = 1, void* workspace = nullptr) {
   GemvArgs a;
   a.x = (const half_t*)p.x;
   a.wq = (const uint32_t*)p.wq;
@@ -411,15 +458,20 @@ int launch_one(const Problem& p, int group_shift, const Plan& plan) {
   a.max_tiles = plan.max_tiles;
   a.phase_chunks = plan.phase_chunks;
   a.ep = Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation};
+  // workspace of the K split: [tiles][ksplit][256] float partial tiles, then [tiles] counters
+  float* const partials = static_cast<float*>(workspace);
+  unsigned int* const counters = reinterpret_cast<unsigned int*>(partials + (size_t)a.tiles * ksplit * 256);
   // two builds of the kernel, by the way the activations are staged: flat index / a column per thread
   auto go = [&](auto rows) -> int {
     constexpr bool ROWS = decltype(rows)::value;
     static bool lds_ok[kMaxDevices] = {false};
-    if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS>, (int)kLdsPerWgMax, lds_ok))
+    if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT>, (int)kLdsPerWgMax,
+                            lds_ok))
       return kFailed;
-    hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS>), dim3(plan.grid), dim3(WAVES * 64),
+    hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT>), dim3(plan.grid), dim3(WAVES * 64),
                        plan.lds_bytes, p.stream, a.x, a.wq, a.scales, a.y, a.M, a.N, a.K, a.group_shift,
-                       a.zero_point, a.lds_stride, a.tiles, a.max_tiles, a.phase_chunks, a.ep);
+                       a.zero_point, a.lds_stride, a.tiles, a.max_tiles, a.phase_chunks, a.ep, ksplit, partials,
+                       counters);
     return kLaunched;
   };
   constexpr int ch = 128 / BITS;
@@ -567,6 +619,136 @@ int launch_gemv(const Problem& p, int variant) {
     return -1;
   }
   return 0;
+}
+
+namespace {
+
+// Cross-workgroup K split of the 8-wavefront, two-chunk kernel (one workgroup per CU).
+constexpr int kSplitWaves = 8, kSplitD = 2, kSplitMaxR = 4;
+
+struct SplitPlan {
+  int r = 1;
+  Plan plan;
+  int64_t workspace_bytes = 0;
+};
+
+// LDS plan for `r` K windows, or false.  *path = the longest chain of super steps a wavefront walks.
+template <int BITS>
+bool split_plan_for(const Problem& p, int r, Plan* out, int64_t* path) {
+  constexpr int ch = 128 / BITS;
+  const int tiles = (int)((p.n + 15) / 16);
+  const int nsuper = (int)(p.k / ch) / (4 * kSplitD);
+  const int groups = std::min(tiles, std::max(1, cu_count() / r));  // tile lists, each shared by r workgroups
+  const int max_tiles = (tiles + groups - 1) / groups;
+  const int window = (nsuper + r - 1) / r;  // super steps per K window
+  if (window < 1 || (int64_t)(r - 1) * window >= nsuper) return false;
+  const size_t slot_bytes = (size_t)max_tiles * kSplitWaves * 1024;
+  const int lds_stride = window * 4 * kSplitD * ch + 8;
+  const size_t lds_bytes = slot_bytes + (size_t)p.m * lds_stride * sizeof(half_t);
+  if (lds_bytes > kLdsPerWgMax) return false;
+  out->grid = groups * r;
+  out->max_tiles = max_tiles;
+  out->phase_chunks = window * 4 * kSplitD;
+  out->lds_stride = lds_stride;
+  out->lds_bytes = lds_bytes;
+  *path = (int64_t)max_tiles * ((window + kSplitWaves - 1) / kSplitWaves);
+  return true;
+}
+
+// Whether, and how many ways, to split K across workgroups.  What the split buys was measured on MI355X
+// by timing problems of the same bytes with K cut and N multiplied: a shorter critical path where the
+// tile count leaves CUs idle for whole rounds (5120 rows = 320 tiles on 256 CUs), and less activation
+// staging where one tile per CU makes every workgroup stage all of a large x.  What it costs: the last
+// workgroup's chain of three trips to the memory side of the L2s (partials out, count, partials in),
+// 2 - 3 us.  A super step of a wavefront takes about 0.7 us, so the split must save at least five of
+// them on the critical path (5120 x 13824 int8: 28 -> 20, 21.8 -> 19.9 us at batch 1, 31.0 -> 22.8 us
+// at 16 rows), or spare a problem with one tile per CU the K phases that activations beyond the LDS
+// need (4096 x 11008 int4: 13.0 -> 11.7 us at 8 rows, 16.6 -> 13.7 us at 16).  On tile-major weights
+// the register-activation kernel already covers the small batches of these shapes: there only from
+// 12 rows on.  Measured and excluded: 4096 x 4096 at 8 - 16 rows (5.7 -> 7.3 us), 5120 x 5120 (10.4 -> 12.1 us).
+template <int BITS>
+bool choose_split(const Problem& p, int gs, SplitPlan* out) {
+  constexpr int ch = 128 / BITS;
+  if (p.m < 1 || p.m > 16 || p.k % (4 * kSplitD * ch) != 0) return false;
+  if (p.tiled ? !((BITS == 4 && gs == 0) || (BITS == 8 && gs == 3)) : !(gs == 0 || (1 << gs) >= kSplitD)) return false;
+  if (p.tiled && p.m < 12) return false;
+  const int64_t tiles = (p.n + 15) / 16, cu = cu_count();
+  const int nsuper = (int)(p.k / ch) / (4 * kSplitD);
+  const int64_t path1 = ((tiles + std::min(tiles, cu) - 1) / std::min(tiles, cu)) * ((nsuper + kSplitWaves - 1) / kSplitWaves);
+  int best = 1;
+  int64_t best_path = path1;
+  Plan best_plan{};
+  for (int r = 2; r <= kSplitMaxR; ++r) {
+    Plan plan;
+    int64_t path;
+    if (!split_plan_for<BITS>(p, r, &plan, &path)) continue;
+    if (path < best_path) {
+      best = r;
+      best_path = path;
+      best_plan = plan;
+    }
+  }
+  if (best == 1 || path1 - best_path < 5) {
+    best = 1;
+    if (p.m * p.k * 2 > 160 * 1024 && tiles <= cu) {
+      // the fewest windows whose activations fit, each wavefront keeping at least one super step
+      for (int r = 2; r <= kSplitMaxR && best == 1; ++r) {
+        Plan plan;
+        int64_t path;
+        if ((nsuper + r - 1) / r >= kSplitWaves && split_plan_for<BITS>(p, r, &plan, &path)) {
+          best = r;
+          best_plan = plan;
+        }
+      }
+    }
+  }
+  if (best == 1) return false;
+  out->r = best;
+  out->plan = best_plan;
+  out->workspace_bytes = tiles * best * 1024 + tiles * 4;
+  return true;
+}
+
+bool choose_split_any(const Problem& p, SplitPlan* out, int* gs_out) {
+  const int ch = 128 / p.bits;
+  int ratio = p.group / ch, gs = 0;
+  while ((1 << gs) < ratio) ++gs;
+  if (ratio < 1 || (1 << gs) != ratio || p.group % ch != 0) return false;
+  *gs_out = gs;
+  return p.bits == 4 ? choose_split<4>(p, gs, out) : choose_split<8>(p, gs, out);
+}
+
+}  // namespace
+
+int64_t gemv_split_workspace_bytes(const Problem& p) {
+  SplitPlan sp;
+  int gs;
+  return choose_split_any(p, &sp, &gs) ? sp.workspace_bytes : 0;
+}
+
+// 1 = launched with the K split, 0 = the split does not apply or the workspace is too small (nothing
+// launched), -1 = failure
+int launch_gemv_split(const Problem& p, void* workspace, int64_t workspace_bytes) {
+  SplitPlan sp;
+  int gs;
+  if (!choose_split_any(p, &sp, &gs) || workspace == nullptr || workspace_bytes < sp.workspace_bytes) return 0;
+  int ok;
+  if (p.bits == 4) {
+    if (p.tiled) ok = launch_one<4, kSplitWaves, kSplitD, 2, true, true>(p, gs, sp.plan, sp.r, workspace);
+    else if (gs == 0) ok = launch_one<4, kSplitWaves, kSplitD, kSplitD, false, true>(p, gs, sp.plan, sp.r, workspace);
+    else ok = launch_one<4, kSplitWaves, kSplitD, 1, false, true>(p, gs, sp.plan, sp.r, workspace);
+  } else {
+    if (p.tiled) ok = launch_one<8, kSplitWaves, kSplitD, 1, true, true>(p, gs, sp.plan, sp.r, workspace);
+    else if (gs == 0) ok = launch_one<8, kSplitWaves, kSplitD, kSplitD, false, true>(p, gs, sp.plan, sp.r, workspace);
+    else ok = launch_one<8, kSplitWaves, kSplitD, 1, false, true>(p, gs, sp.plan, sp.r, workspace);
+  }
+  if (ok != kLaunched) return -1;
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("gemv kernel (K split) launch failed: %s", hipGetErrorString(e));
+    return -1;
+  }
+  return 1;
 }
 
 }  // namespace wq

@@ -25,6 +25,12 @@ struct Problem {
 // (only reachable through mi355x_wq_matmul_ex; used by sweeps).
 int launch_gemv(const Problem& p, int variant);
 bool gemv_applicable(const Problem& p);  // M <= 16 and a default variant's LDS plan (slots + activations) fits
+// Cross-workgroup K split of the decode kernel (M <= 16): bytes of caller workspace it needs for `p`
+// (0 = no split for this problem), and the launch (1 launched, 0 not applicable / workspace too small,
+// -1 failure).  The workspace holds float32 partial tiles and per-tile arrival counters; the counters
+// must be zero before the first use and are zero again when the kernel has finished.
+int64_t gemv_split_workspace_bytes(const Problem& p);
+int launch_gemv_split(const Problem& p, void* workspace, int64_t workspace_bytes);
 int launch_skinny(const Problem& p, int variant);
 int launch_gemm(const Problem& p, int variant);
 bool gemm_pipe_applicable(const Problem& p);  // K % 64 == 0, operands below 1 GiB

@@ -30,6 +30,7 @@ struct Dtype {
 };
 constexpr Dtype kF16{2, 16, "float16"};
 constexpr Dtype kU32{1, 32, "uint32"};
+constexpr Dtype kU8{1, 8, "uint8"};
 
 // Checks one tensor argument; on success stores the (byte_offset adjusted) pointer.
 // `vector_ok`: the tensor may be 1-d [N] (reported as rows = 1, cols = N).
@@ -361,6 +362,60 @@ MI355X_TILED_ENTRY(mi355x_q4f16_matmul_tiled, true, 4, 7)
 MI355X_TILED_ENTRY(mi355x_q8f16_matmul_tiled, true, 8, 0)
 #undef MI355X_TILED_ENTRY
 
+// ---- decode with a workspace tensor: matmul_ws(x[M,K], wq[N,...], scales[N,...], workspace[bytes] u8, y[M,N])
+static int packed_ws(int bits, int zero_point, mi355x_tvm_value* args, int* type_codes, int num_args) {
+  if (num_args != 5 || args == nullptr || type_codes == nullptr) {
+    wq::set_error("matmul_ws expects 5 tensor arguments (x, wq, scales, workspace, y), got %d", num_args);
+    return fail();
+  }
+  const mi355x_dl_tensor *tx = nullptr, *tw = nullptr, *ts = nullptr, *tk = nullptr, *ty = nullptr;
+  void *px = nullptr, *pw = nullptr, *ps = nullptr, *pk = nullptr, *py = nullptr;
+  if (!take_tensor(args, type_codes, 1, "wq", kU32, -1, &tw, &pw)) return fail();
+  const int dev = tw->device.device_id;
+  int64_t wr = 0, wbytes = 0;
+  if (!take_tensor(args, type_codes, 0, "x", kF16, dev, &tx, &px) ||
+      !take_tensor(args, type_codes, 2, "scales", kF16, dev, &ts, &ps) ||
+      !take_tensor(args, type_codes, 3, "workspace", kU8, dev, &tk, &pk, true, &wr, &wbytes) ||
+      !take_tensor(args, type_codes, 4, "y", kF16, dev, &ty, &py))
+    return fail();
+  mi355x_wq_desc d;
+  memset(&d, 0, sizeof(d));
+  d.bits = bits;
+  d.zero_point = zero_point;
+  d.n = tw->shape[0];
+  d.k = tw->shape[1] * (32 / bits);
+  const int64_t m = tx->shape[0];
+  if (ts->shape[0] != d.n || ts->shape[1] <= 0 || d.k % ts->shape[1] != 0 || tx->shape[1] != d.k ||
+      ty->shape[0] != m || ty->shape[1] != d.n) {
+    wq::set_error("matmul_ws: x (%lld, %lld), wq of %lld rows and K=%lld, scales (%lld, %lld), y (%lld, %lld) do not fit",
+                  (long long)tx->shape[0], (long long)tx->shape[1], (long long)d.n, (long long)d.k,
+                  (long long)ts->shape[0], (long long)ts->shape[1], (long long)ty->shape[0], (long long)ty->shape[1]);
+    return fail();
+  }
+  d.group = (int32_t)(d.k / ts->shape[1]);
+  if (mi355x_wq_check(&d, m) != 0) return fail();
+  if (d.n == 0 || m == 0) return 0;
+  int cur = -1;
+  if (hipGetDevice(&cur) != hipSuccess) {
+    (void)hipGetLastError();
+    wq::set_error("no usable HIP device in this process");
+    return fail();
+  }
+  if (cur != dev) {
+    wq::set_error("tensors live on ROCm device %d but the current HIP device is %d", dev, cur);
+    return fail();
+  }
+  return mi355x_wq_matmul_ws(&d, px, pw, ps, nullptr, py, m, g_stream, 0, wr * wbytes > 0 ? pk : nullptr, wr * wbytes) == 0
+             ? 0
+             : fail();
+}
+int mi355x_q4f16_matmul_ws(mi355x_tvm_value* args, int* type_codes, int num_args, mi355x_tvm_value*, int*, void*) {
+  return packed_ws(4, 7, args, type_codes, num_args);
+}
+int mi355x_q8f16_matmul_ws(mi355x_tvm_value* args, int* type_codes, int num_args, mi355x_tvm_value*, int*, void*) {
+  return packed_ws(8, 0, args, type_codes, num_args);
+}
+
 // ---- registration in TVM's global table through its C API -----------------------
 typedef int (*backend_fn_t)(mi355x_tvm_value*, int*, int, mi355x_tvm_value*, int*, void*);
 
@@ -399,7 +454,9 @@ int mi355x_wq_register_tvm_globals(int allow_override) {
                            {"mi355x.q4f16_tile_weights", mi355x_q4f16_tile_weights},
                            {"mi355x.q8f16_tile_weights", mi355x_q8f16_tile_weights},
                            {"mi355x.q4f16_matmul_tiled", mi355x_q4f16_matmul_tiled},
-                           {"mi355x.q8f16_matmul_tiled", mi355x_q8f16_matmul_tiled}};
+                           {"mi355x.q8f16_matmul_tiled", mi355x_q8f16_matmul_tiled},
+                           {"mi355x.q4f16_matmul_ws", mi355x_q4f16_matmul_ws},
+                           {"mi355x.q8f16_matmul_ws", mi355x_q8f16_matmul_ws}};
   int count = 0;
   for (const Entry& e : entries) {
     void* handle = nullptr;

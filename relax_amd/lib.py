@@ -17,12 +17,14 @@ EXPORTED_SYMBOLS = (
     "mi355x_wq_matmul", "mi355x_wq_matmul_ex", "mi355x_wq_matmul_fused", "mi355x_wq_matmul_fused_ex",
     "mi355x_wq_dequantize", "mi355x_wq_check",
     "mi355x_wq_tiled_sizes", "mi355x_wq_tile_weights", "mi355x_wq_untile_weights", "mi355x_wq_matmul_tiled", "mi355x_wq_matmul_tiled_ex",
+    "mi355x_wq_workspace_bytes", "mi355x_wq_matmul_ws",
     "mi355x_wq_select_kernel", "mi355x_wq_last_error", "mi355x_wq_version",
     "mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_matmul_bias", "mi355x_q8f16_matmul_bias",
     "mi355x_q4f16_matmul_bias_relu", "mi355x_q8f16_matmul_bias_relu", "mi355x_q4f16_matmul_residual",
     "mi355x_q8f16_matmul_residual", "mi355x_q4f16_dequantize",
     "mi355x_q8f16_dequantize", "mi355x_q4f16_tile_weights", "mi355x_q8f16_tile_weights",
-    "mi355x_q4f16_matmul_tiled", "mi355x_q8f16_matmul_tiled", "mi355x_wq_packed_call", "mi355x_wq_packed_set_stream",
+    "mi355x_q4f16_matmul_tiled", "mi355x_q8f16_matmul_tiled", "mi355x_q4f16_matmul_ws", "mi355x_q8f16_matmul_ws",
+    "mi355x_wq_packed_call", "mi355x_wq_packed_set_stream",
     "mi355x_wq_packed_get_stream", "mi355x_wq_register_tvm_globals",
 )
 PACKED_ENTRIES = tuple(s for s in EXPORTED_SYMBOLS if s.startswith(("mi355x_q4f16_", "mi355x_q8f16_")))
@@ -80,6 +82,9 @@ def load() -> C.CDLL:
     L.mi355x_wq_untile_weights.argtypes = [dp, vp, vp, vp, vp, vp]
     L.mi355x_wq_matmul_tiled.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp]
     L.mi355x_wq_matmul_tiled_ex.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp, ci]
+    L.mi355x_wq_workspace_bytes.argtypes = [dp, i64, ci]
+    L.mi355x_wq_workspace_bytes.restype = i64
+    L.mi355x_wq_matmul_ws.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp, ci, vp, i64]
     L.mi355x_wq_check.argtypes = [dp, i64]
     L.mi355x_wq_select_kernel.argtypes = [dp, i64]
     L.mi355x_wq_last_error.restype = C.c_char_p

@@ -22,14 +22,22 @@ def wq_matmul(x: torch.Tensor, wq: torch.Tensor, scales: torch.Tensor, bits: int
               zero_point: int | None = None, out: torch.Tensor | None = None, kernel: int = 0,
               variant: int = 0, stream=None, bias: torch.Tensor | None = None,
               activation: str | None = None, residual: torch.Tensor | None = None,
-              tiled_n: int | None = None) -> torch.Tensor:
+              tiled_n: int | None = None, workspace: torch.Tensor | None = None) -> torch.Tensor:
     """y[M,N] = f16(x[M,K] @ dequant(wq, scales)^T) on the current HIP device (asynchronous).
 
     Optional fused epilogue, each step one float16 operation: ``+ bias[N]``, then ``activation``
     ("relu"), then ``+ residual[M,N]`` (``residual`` may be ``out`` itself).
 
     ``tiled_n=N``: ``wq`` and ``scales`` are the tile-major buffers `wq_tile_weights` returns
-    for an N-row matrix (their row count is N rounded up to 16)."""
+    for an N-row matrix (their row count is N rounded up to 16).
+
+    ``workspace``: a device buffer from `wq_workspace` (zeroed once, then reusable by calls that do
+    not overlap in time); lets the decode kernel split K across workgroups where that pays."""
+    if workspace is not None:
+        if kernel != 0 or variant != 0:
+            raise ValueError("a workspace goes with the library's own kernel choice")
+        return _wq_matmul_ws(x, wq, scales, bits, group, tiled_n, zero_point, out, stream, bias, activation,
+                             residual, workspace)
     if tiled_n is not None:
         return _wq_matmul_tiled(x, wq, scales, bits, group, tiled_n, zero_point, out, stream, bias,
                                 activation, residual, kernel | (variant << 8))
@@ -145,6 +153,53 @@ def _wq_matmul_tiled(x, wq_t, s_t, bits, group, n, zero_point, out, stream, bias
                          _lib.ACTIVATIONS[activation], 0)
     _lib.check(L.mi355x_wq_matmul_tiled_ex(desc, x.data_ptr(), wq_t.data_ptr(), s_t.data_ptr(), ep, out.data_ptr(),
                                            m, _stream_ptr(stream), kernel))
+    return out
+
+
+def wq_workspace_bytes(bits: int, group: int, n: int, k: int, m: int, tiled: bool = False,
+                       zero_point: int | None = None) -> int:
+    """Bytes of workspace `wq_matmul(..., workspace=)` needs to split K for this problem; 0 = it would not."""
+    L = _lib.load()
+    nbytes = L.mi355x_wq_workspace_bytes(_lib.make_desc(bits, group, n, k, zero_point), m, 1 if tiled else 0)
+    if nbytes < 0:
+        raise _lib.WqError(_lib.last_error())
+    return int(nbytes)
+
+
+def wq_workspace(nbytes: int, device="cuda") -> torch.Tensor | None:
+    """A zeroed workspace of `nbytes` (None for 0).  Size it for the largest problem that will use it."""
+    return torch.zeros(nbytes, dtype=torch.uint8, device=device) if nbytes > 0 else None
+
+
+def _wq_matmul_ws(x, wq, scales, bits, group, tiled_n, zero_point, out, stream, bias, activation, residual, workspace):
+    L = _lib.load()
+    if not (x.is_cuda and wq.is_cuda and scales.is_cuda and workspace.is_cuda):
+        raise ValueError("x, wq, scales and workspace must be device tensors")
+    if x.dtype != torch.float16 or scales.dtype != torch.float16 or not x.is_contiguous():
+        raise TypeError("x and scales must be float16, x compact")
+    if not (wq.is_contiguous() and scales.is_contiguous() and workspace.is_contiguous()):
+        raise ValueError("wq, scales and workspace must be compact")
+    m, k = x.shape
+    n = tiled_n if tiled_n is not None else wq.shape[0]
+    desc = _lib.make_desc(bits, group, n, k, zero_point)
+    if tiled_n is not None:
+        wb, sb = _tiled_sizes(L, desc)
+        if wq.numel() * wq.element_size() != wb or scales.numel() * scales.element_size() != sb:
+            raise ValueError(f"tile-major buffers must hold {wb} and {sb} bytes for N={n}, K={k}")
+    elif wq.shape[1] * (32 // bits) != k or tuple(scales.shape) != (n, k // group):
+        raise ValueError("wq / scales do not match x's K")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    elif tuple(out.shape) != (m, n) or out.dtype != torch.float16 or not out.is_contiguous():
+        raise ValueError("out must be a compact float16 [M, N] tensor")
+    if activation not in _lib.ACTIVATIONS:
+        raise ValueError(f"unsupported activation {activation!r}")
+    ep = _lib.WqEpilogue(bias.data_ptr() if bias is not None else None,
+                         residual.data_ptr() if residual is not None else None,
+                         _lib.ACTIVATIONS[activation], 0)
+    _lib.check(L.mi355x_wq_matmul_ws(desc, x.data_ptr(), wq.data_ptr(), scales.data_ptr(), ep, out.data_ptr(), m,
+                                     _stream_ptr(stream), 1 if tiled_n is not None else 0, workspace.data_ptr(),
+                                     workspace.numel() * workspace.element_size()))
     return out
 
 

@@ -27,7 +27,7 @@ def declared_symbols():
 def test_library_exports_every_declared_symbol():
     L = lib.load()
     names = declared_symbols()
-    assert len(names) == 32 and set(names) == set(lib.EXPORTED_SYMBOLS)
+    assert len(names) == 36 and set(names) == set(lib.EXPORTED_SYMBOLS)
     for n in names:
         assert hasattr(L, n), n
     assert L.mi355x_wq_version() >= 100
@@ -54,6 +54,27 @@ def test_tile_major_layout_entry_checks_without_a_gpu():
     assert L.mi355x_wq_untile_weights(d, None, ok, ok, ok, None) == -1 and "wq_tiled is NULL" in lib.last_error()
     assert L.mi355x_wq_matmul_tiled(lib.make_desc(4, 32, 64, 320), ok, ok, ok, None, ok, 4, None) == -1 \
         and "tile-major layout" in lib.last_error()
+
+
+def test_workspace_size_query_without_a_gpu():
+    """mi355x_wq_workspace_bytes: partial tiles (1 KB per 16-row tile and K window) plus one counter per
+    tile where the decode kernel would split K, 0 where it would not, -1 on an invalid descriptor.
+    (The rule reads the CU count; without a GPU the library assumes the 256 CUs of an MI355X.)"""
+    L = lib.load()
+    q = L.mi355x_wq_workspace_bytes
+    assert q(lib.make_desc(8, 128, 5120, 13824), 1, 0) == 320 * 3 * 1024 + 320 * 4      # three windows
+    assert q(lib.make_desc(8, 128, 5120, 13824), 16, 0) == 320 * 4 * 1024 + 320 * 4     # 16 rows: four fit the LDS
+    assert q(lib.make_desc(4, 32, 4096, 11008), 8, 0) == 256 * 2 * 1024 + 256 * 4       # activations beyond the LDS
+    assert q(lib.make_desc(4, 32, 4096, 11008), 1, 0) == 0
+    assert q(lib.make_desc(4, 32, 12288, 4096), 8, 0) == 0 and q(lib.make_desc(4, 32, 4096, 4096), 16, 0) == 0
+    assert q(lib.make_desc(8, 128, 5120, 13824), 4, 1) == 0                              # tile-major: from 12 rows on
+    assert q(lib.make_desc(8, 128, 5120, 13824), 16, 1) == 320 * 4 * 1024 + 320 * 4
+    assert q(lib.make_desc(4, 32, 4096, 11008), 32, 0) == 0                              # not a decode batch
+    assert q(lib.make_desc(4, 32, 4096, 320), 8, 1) == 0                                 # layout not defined: no split
+    assert q(lib.make_desc(5, 32, 4096, 4096), 8, 0) == -1 and "bits" in lib.last_error()
+    ok = 0x10000
+    assert L.mi355x_wq_matmul_ws(lib.make_desc(4, 32, 64, 256), ok, ok, ok, None, ok, 4, None, 0, ok + 4, 1 << 20) == -1 \
+        and "workspace" in lib.last_error() and "16-byte aligned" in lib.last_error()
 
 
 def test_measurement_probe_library_is_built_and_separate():
@@ -308,7 +329,7 @@ assert L.mi355x_wq_register_tvm_globals(0) == -1 and "no TVM runtime" in lib.las
 fake = C.CDLL({fake!r}, mode=C.RTLD_GLOBAL)
 fake.fake_tvm_name.restype = C.c_char_p
 fake.fake_tvm_last_error.restype = C.c_char_p
-assert L.mi355x_wq_register_tvm_globals(0) == 14
+assert L.mi355x_wq_register_tvm_globals(0) == 16
 names = sorted(fake.fake_tvm_name(i).decode() for i in range(fake.fake_tvm_count()))
 assert names == sorted("mi355x." + s[len("mi355x_"):] for s in lib.PACKED_ENTRIES), names
 # call a registered function the way the registry would, with host tensors: it must fail and the

@@ -1,0 +1,160 @@
+"""GPU parity of the decode kernel's cross-workgroup K split (mi355x_wq_matmul_ws, caller workspace).
+
+Bar as for the other matmul tests: float16 outputs within max-abs 1e-2 and relative 1e-2 of the oracle;
+beyond that the split is deterministic (the partial tiles are added in the order of their K windows,
+whichever workgroup arrives last), leaves its workspace ready for the next call, and a call whose
+workspace is missing or too small is the plain call bit for bit."""
+import numpy as np
+import pytest
+
+from oracle import c_oracle, wq_oracle as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+from tests.test_gpu_parity import _dev, assert_close, assert_fused, _fused_operands  # noqa: E402
+
+# (bits, M, N, K): shapes the library splits -- long K with one tile per CU, or 320 tiles on 256 CUs
+CASES = [(4, 8, 4096, 11008), (4, 16, 4096, 11008), (8, 1, 5120, 13824), (8, 4, 5120, 13824),
+         (8, 16, 5120, 13824), (4, 8, 4090, 11008), (8, 3, 5115, 13824), (4, 12, 2048, 22016)]
+
+
+@pytest.mark.parametrize("bits,m,n,k", CASES)
+def test_k_split_matches_the_oracle_and_is_deterministic(bits, m, n, k):
+    import relax_amd
+
+    x, wq, s, g = O.make_case(41, m, n, k, bits)
+    need = relax_amd.wq_workspace_bytes(bits, g, n, k, m)
+    assert need > 0, "the case is meant to split"
+    ws = relax_amd.wq_workspace(need)
+    dx, dwq, ds = _dev(x), _dev(wq), _dev(s)
+    y1 = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws)
+    torch.cuda.synchronize()
+    tiles = (n + 15) // 16
+    assert int(ws[need - 4 * tiles:].view(torch.int32).abs().sum()) == 0, "arrival counters are back at zero"
+    want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
+    # (K of 11008 - 22016: the float32 accumulation error is absolute and grows with the length of the
+    # sum, so a few more outputs than elsewhere land two float16 ulp away; the tolerance is unchanged)
+    assert_close(y1.cpu().numpy(), want, ("k split", bits, m, n, k), ulp_fraction=0.005)
+    for _ in range(3):  # same workspace, back to back: same bits
+        y2 = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y1.view(torch.int16), y2.view(torch.int16))
+    # tile-major weights: the same windows in the same order where the library splits there too
+    wq_t, s_t = relax_amd.wq_tile_weights(dwq, ds, bits, g)
+    y3 = relax_amd.wq_matmul(dx, wq_t, s_t, bits, g, tiled_n=n, workspace=ws)
+    torch.cuda.synchronize()
+    if relax_amd.wq_workspace_bytes(bits, g, n, k, m, tiled=True) > 0:
+        assert torch.equal(y1.view(torch.int16), y3.view(torch.int16))
+    else:
+        assert_close(y3.cpu().numpy(), want, ("tile-major, no split", bits, m, n, k), ulp_fraction=0.005)
+
+
+@pytest.mark.parametrize("bits,m,n,k", [(4, 8, 4096, 11008), (8, 16, 5120, 13824)])
+def test_k_split_applies_the_fused_tail_once(bits, m, n, k):
+    """bias + relu + residual behind the sum of the partial tiles: applied by the workgroup that adds them."""
+    import relax_amd
+
+    x, wq, s, g = O.make_case(43, m, n, k, bits)
+    bias, res = _fused_operands(43, m, n)
+    ws = relax_amd.wq_workspace(relax_amd.wq_workspace_bytes(bits, g, n, k, m))
+    assert ws is not None
+    dx, dwq, ds = _dev(x), _dev(wq), _dev(s)
+    plain = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws)
+    fused = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws, bias=_dev(bias), activation="relu",
+                                residual=_dev(res))
+    torch.cuda.synchronize()
+    want_plain = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
+    assert_fused(fused.cpu().numpy(), plain.cpu().numpy(), want_plain, bias, "relu", res, (bits, m, n, k))
+    # in place on the residual: y = h + W x written over h
+    h = _dev(res).clone()
+    relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws, residual=h, out=h)
+    torch.cuda.synchronize()
+    assert_fused(h.cpu().numpy(), plain.cpu().numpy(), want_plain, None, None, res, ("in place", bits, m))
+
+
+def test_missing_or_small_workspace_is_the_plain_call():
+    import relax_amd
+    from relax_amd import lib
+
+    bits, m, n, k = 8, 4, 5120, 13824
+    x, wq, s, g = O.make_case(47, m, n, k, bits)
+    dx, dwq, ds = _dev(x), _dev(wq), _dev(s)
+    plain = relax_amd.wq_matmul(dx, dwq, ds, bits, g)
+    need = relax_amd.wq_workspace_bytes(bits, g, n, k, m)
+    small = torch.zeros(need - 16, dtype=torch.uint8, device="cuda")
+    y = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=small)
+    torch.cuda.synchronize()
+    assert torch.equal(plain.view(torch.int16), y.view(torch.int16))
+    assert int(small.sum()) == 0, "a workspace that is too small is not touched"
+    # problems the library does not split ignore the workspace: 33 rows, and a wide projection
+    for m2, n2, k2 in ((33, 5120, 13824), (8, 12288, 4096)):
+        x2, wq2, s2, _ = O.make_case(48, m2, n2, k2, 4)
+        assert relax_amd.wq_workspace_bytes(4, 32, n2, k2, m2) == 0
+        a = relax_amd.wq_matmul(_dev(x2), _dev(wq2), _dev(s2), 4, 32)
+        b = relax_amd.wq_matmul(_dev(x2), _dev(wq2), _dev(s2), 4, 32, workspace=small)
+        torch.cuda.synchronize()
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16)) and int(small.sum()) == 0
+    # a forced kernel family and a workspace do not go together
+    with pytest.raises(ValueError, match="own kernel choice"):
+        relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=small, kernel=lib.KERNEL_GEMV)
+
+
+def test_k_split_in_a_hip_graph_replays_like_eager():
+    """The down projection of a decoder layer at 8 rows with its residual, captured once with the
+    workspace and replayed with eager work in between: every replay gives the eager bits, and a second
+    projection sharing the workspace in the same graph does not disturb the first."""
+    import relax_amd
+
+    m, n, k = 8, 4096, 11008
+    x, wq, s, g = O.make_case(53, m, n, k, 4)
+    x2, wq2, s2, _ = O.make_case(54, m, n, k, 4)
+    dx, dwq, ds, dx2, dwq2, ds2 = _dev(x), _dev(wq), _dev(s), _dev(x2), _dev(wq2), _dev(s2)
+    ws = relax_amd.wq_workspace(relax_amd.wq_workspace_bytes(4, g, n, k, m))
+    eager1 = relax_amd.wq_matmul(dx, dwq, ds, 4, g, workspace=ws)
+    eager2 = relax_amd.wq_matmul(dx2, dwq2, ds2, 4, g, workspace=ws)
+    torch.cuda.synchronize()
+    y1 = torch.empty_like(eager1)
+    y2 = torch.empty_like(eager2)
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=st):
+            relax_amd.wq_matmul(dx, dwq, ds, 4, g, workspace=ws, out=y1)
+            relax_amd.wq_matmul(dx2, dwq2, ds2, 4, g, workspace=ws, out=y2)
+    torch.cuda.synchronize()
+    for rep in range(4):
+        y1.zero_()
+        y2.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y1.view(torch.int16), eager1.view(torch.int16)), rep
+        assert torch.equal(y2.view(torch.int16), eager2.view(torch.int16)), rep
+        # the program's own eager work between replays, on the same workspace
+        again = relax_amd.wq_matmul(dx, dwq, ds, 4, g, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(again.view(torch.int16), eager1.view(torch.int16))
+
+
+def test_workspace_entry_called_vm_style():
+    """matmul_ws as a destination-passing extern with a 1-d uint8 workspace tensor."""
+    from relax_amd import vm_harness
+    import relax_amd
+
+    vm_harness.set_stream()
+    for bits, m, n, k in [(8, 2, 5120, 13824), (4, 16, 4096, 11008), (4, 8, 50, 512)]:
+        x, wq, s, g = O.make_case(60 + m, m, n, k, bits)
+        need = relax_amd.wq_workspace_bytes(bits, g, n, k, m)
+        ws = torch.zeros(max(need, 64), dtype=torch.uint8, device="cuda")
+        y = vm_harness.call_dps("mi355x_q%df16_matmul_ws" % bits, [_dev(x), _dev(wq), _dev(s), ws], (m, n))
+        torch.cuda.synchronize()
+        assert_close(y.cpu().numpy(), c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16), (bits, m, n, k),
+                     ulp_fraction=0.005)
+        if need:
+            direct = relax_amd.wq_matmul(_dev(x), _dev(wq), _dev(s), bits, g, workspace=ws)
+            torch.cuda.synchronize()
+            assert torch.equal(direct.view(torch.int16), y.view(torch.int16))
+    with pytest.raises(vm_harness.PackedError, match="5 tensor arguments"):
+        vm_harness.call_dps("mi355x_q4f16_matmul_ws", [_dev(x), _dev(wq), _dev(s)], (m, n))
+    with pytest.raises(vm_harness.PackedError, match="workspace"):
+        vm_harness.call_dps("mi355x_q4f16_matmul_ws", [_dev(x), _dev(wq), _dev(s), ws.view(torch.int8)], (m, n))
