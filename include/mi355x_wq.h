@@ -153,7 +153,9 @@ MI355X_WQ_API int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const vo
  * allocates per call (python/tvm/contrib/cutlass/build.py:335, conv2d_operation.py:417-418); here the
  * caller owns it, so that nothing is allocated under a stream capture or in a serving loop.
  *
- * mi355x_wq_workspace_bytes: the size mi355x_wq_matmul_ws needs to split K for (desc, m, layout); 0 if it
+ * mi355x_wq_workspace_bytes: the size mi355x_wq_matmul_ws needs to split K for (desc, m, layout) -- 16 KB of
+ * arrival counters at the head, then 1 KB per 16-row tile and K window, so one workspace sized for the
+ * largest projection serves projections of every shape; 0 if it
  * would not split (then the call equals mi355x_wq_matmul_fused / _tiled), -1 on an invalid descriptor.
  * Workspace rules: device memory, 16-byte aligned, all zero before its first use (the kernel leaves it
  * ready for the next call); calls that share a workspace must not overlap in time (one stream, or

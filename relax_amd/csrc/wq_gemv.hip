@@ -402,6 +402,8 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
 namespace {
 
 constexpr size_t kLdsPerCu = 160 * 1024;
+constexpr int64_t kSplitMaxTiles = 4096;                 // row tiles a K split handles (N <= 65536)
+constexpr int64_t kSplitCounterBytes = kSplitMaxTiles * 4;  // head of the workspace
 constexpr size_t kLdsPerWgMax = 159 * 1024;  // of the 160 KB a workgroup can address
 
 struct Plan {
@@ -458,9 +460,11 @@ int launch_one(const Problem& p, int group_shift, const Plan& plan, int ksplit =
   a.max_tiles = plan.max_tiles;
   a.phase_chunks = plan.phase_chunks;
   a.ep = Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation};
-  // workspace of the K split: [tiles][ksplit][256] float partial tiles, then [tiles] counters
-  float* const partials = static_cast<float*>(workspace);
-  unsigned int* const counters = reinterpret_cast<unsigned int*>(partials + (size_t)a.tiles * ksplit * 256);
+  // workspace of the K split: kSplitMaxTiles arrival counters at a fixed place -- a workspace shared by
+  // projections of different shapes keeps them apart from the partial tiles, whose leftovers are not
+  // zero -- then [tiles][ksplit][256] float partial tiles
+  unsigned int* const counters = static_cast<unsigned int*>(workspace);
+  float* const partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kSplitCounterBytes);
   // two builds of the kernel, by the way the activations are staged: flat index / a column per thread
   auto go = [&](auto rows) -> int {
     constexpr bool ROWS = decltype(rows)::value;
@@ -673,6 +677,7 @@ bool choose_split(const Problem& p, int gs, SplitPlan* out) {
   if (p.tiled ? !((BITS == 4 && gs == 0) || (BITS == 8 && gs == 3)) : !(gs == 0 || (1 << gs) >= kSplitD)) return false;
   if (p.tiled && p.m < 12) return false;
   const int64_t tiles = (p.n + 15) / 16, cu = cu_count();
+  if (tiles > kSplitMaxTiles) return false;
   const int nsuper = (int)(p.k / ch) / (4 * kSplitD);
   const int64_t path1 = ((tiles + std::min(tiles, cu) - 1) / std::min(tiles, cu)) * ((nsuper + kSplitWaves - 1) / kSplitWaves);
   int best = 1;
@@ -705,7 +710,7 @@ bool choose_split(const Problem& p, int gs, SplitPlan* out) {
   if (best == 1) return false;
   out->r = best;
   out->plan = best_plan;
-  out->workspace_bytes = tiles * best * 1024 + tiles * 4;
+  out->workspace_bytes = kSplitCounterBytes + tiles * best * 1024;
   return true;
 }
 

@@ -57,18 +57,18 @@ def test_tile_major_layout_entry_checks_without_a_gpu():
 
 
 def test_workspace_size_query_without_a_gpu():
-    """mi355x_wq_workspace_bytes: partial tiles (1 KB per 16-row tile and K window) plus one counter per
-    tile where the decode kernel would split K, 0 where it would not, -1 on an invalid descriptor.
+    """mi355x_wq_workspace_bytes: 16 KB of arrival counters plus the partial tiles (1 KB per 16-row tile
+    and K window) where the decode kernel would split K, 0 where it would not, -1 on an invalid descriptor.
     (The rule reads the CU count; without a GPU the library assumes the 256 CUs of an MI355X.)"""
     L = lib.load()
     q = L.mi355x_wq_workspace_bytes
-    assert q(lib.make_desc(8, 128, 5120, 13824), 1, 0) == 320 * 3 * 1024 + 320 * 4      # three windows
-    assert q(lib.make_desc(8, 128, 5120, 13824), 16, 0) == 320 * 4 * 1024 + 320 * 4     # 16 rows: four fit the LDS
-    assert q(lib.make_desc(4, 32, 4096, 11008), 8, 0) == 256 * 2 * 1024 + 256 * 4       # activations beyond the LDS
+    assert q(lib.make_desc(8, 128, 5120, 13824), 1, 0) == 16384 + 320 * 3 * 1024         # three windows
+    assert q(lib.make_desc(8, 128, 5120, 13824), 16, 0) == 16384 + 320 * 4 * 1024        # 16 rows: four fit the LDS
+    assert q(lib.make_desc(4, 32, 4096, 11008), 8, 0) == 16384 + 256 * 2 * 1024          # activations beyond the LDS
     assert q(lib.make_desc(4, 32, 4096, 11008), 1, 0) == 0
     assert q(lib.make_desc(4, 32, 12288, 4096), 8, 0) == 0 and q(lib.make_desc(4, 32, 4096, 4096), 16, 0) == 0
     assert q(lib.make_desc(8, 128, 5120, 13824), 4, 1) == 0                              # tile-major: from 12 rows on
-    assert q(lib.make_desc(8, 128, 5120, 13824), 16, 1) == 320 * 4 * 1024 + 320 * 4
+    assert q(lib.make_desc(8, 128, 5120, 13824), 16, 1) == 16384 + 320 * 4 * 1024
     assert q(lib.make_desc(4, 32, 4096, 11008), 32, 0) == 0                              # not a decode batch
     assert q(lib.make_desc(4, 32, 4096, 320), 8, 1) == 0                                 # layout not defined: no split
     assert q(lib.make_desc(5, 32, 4096, 4096), 8, 0) == -1 and "bits" in lib.last_error()
