@@ -148,8 +148,8 @@ MI355X_WQ_API int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const vo
  * whole rounds (5120 rows: 320 tiles on 256 CUs) or whose activations are large against one tile per CU,
  * the decode kernel splits K over two to four workgroups per tile; each writes a float32 partial tile
  * to the workspace, and the last to arrive adds them in the order of their K windows (the result does
- * not depend on the order of arrival), applies the epilogue and stores.  5120 x 13824 int8 at batch 1:
- * 22 -> 16 us.  The reference's counterpart is CUTLASS split-K, whose workspace the generated host code
+ * not depend on the order of arrival), applies the epilogue and stores.  5120 x 13824 int8: 22 -> 20 us
+ * at batch 1, 31 -> 23 us at 16 rows.  The reference's counterpart is CUTLASS split-K, whose workspace the generated host code
  * allocates per call (python/tvm/contrib/cutlass/build.py:335, conv2d_operation.py:417-418); here the
  * caller owns it, so that nothing is allocated under a stream capture or in a serving loop.
  *
