@@ -452,6 +452,15 @@ def main() -> int:
                 for (_, _, n, k), wd in zip(mats, dq):
                     torch.matmul(xg[k], wd.t(), out=yg[n])
 
+        # (and the same pass on tile-major copies of the weights, transformed outside the timing)
+        tiled_w = None if args.no_tiled else [[relax_amd.wq_tile_weights(wq, s, 4, 32) for wq, s, _, _ in mats]
+                                               for mats in use]
+
+        def prefill_pass_tiled():
+            for mats, tw in zip(use, tiled_w):
+                for (_, _, n, k), (wt, st) in zip(mats, tw):
+                    relax_amd.wq_matmul(xg[k], wt, st, 4, 32, out=yg[n], tiled_n=n)
+
         def timed(fn, reps):
             g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             g0.record(stream)
@@ -469,10 +478,15 @@ def main() -> int:
                 prefill_pass()
                 library_pass()
             torch.cuda.synchronize()
-            ours, theirs = [], []
+            if tiled_w is not None:
+                prefill_pass_tiled()
+                torch.cuda.synchronize()
+            ours, theirs, ours_tiled = [], [], []
             for _ in range(2):
                 ours.append(timed(prefill_pass, reps))
                 theirs.append(timed(library_pass, reps))
+                if tiled_w is not None:
+                    ours_tiled.append(timed(prefill_pass_tiled, reps))
         gms, lms = sum(ours) / len(ours), sum(theirs) / len(theirs)
         tflops = flops / (gms * 1e-3) / 1e12
         result["gemm"] = {"value": round(tflops, 1), "unit": "TFLOP/s", "ms_per_pass": round(gms, 4),
@@ -481,11 +495,13 @@ def main() -> int:
                           "library_f16_gemm_tflops": round(flops / (lms * 1e-3) / 1e12, 1),
                           "library_f16_gemm_note": "torch.matmul (hipBLASLt) on float16 weights dequantized "
                                                    "beforehand, same shapes and data, timed alternately"}
+        if ours_tiled:
+            result["gemm"]["tile_major_tflops"] = round(flops / (sum(ours_tiled) / len(ours_tiled) * 1e-3) / 1e12, 1)
         result["roofline_gemm"] = {"bound": "mfma", "achieved": round(tflops, 1),
                                    "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                    "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
                                    "kernel": "wq::wq_gemm_direct_kernel"}
-        del wds
+        del wds, tiled_w
 
     # ---- fused residual add: O and down projections of every layer, batch 1 and 8 -------------
     # h = h + x W^T as one launch against the matmul followed by a separate float16 add kernel.
