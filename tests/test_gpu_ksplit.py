@@ -179,3 +179,31 @@ def test_workspace_entry_called_vm_style():
         vm_harness.call_dps("mi355x_q4f16_matmul_ws", [_dev(x), _dev(wq), _dev(s)], (m, n))
     with pytest.raises(vm_harness.PackedError, match="workspace"):
         vm_harness.call_dps("mi355x_q4f16_matmul_ws", [_dev(x), _dev(wq), _dev(s), ws.view(torch.int8)], (m, n))
+
+
+def test_k_split_is_stable_while_another_stream_keeps_the_gpu_busy():
+    """Two hundred split launches on one stream, each into its own output, while a second stream runs
+    prefill-sized GEMMs that change which workgroup of a tile arrives last: every output has the bits of
+    the first.  (The sum is taken in the order of the K windows, not in the order of arrival.)"""
+    import relax_amd
+
+    bits, m, n, k = 8, 4, 5120, 13824
+    x, wq, s, g = O.make_case(61, m, n, k, bits)
+    dx, dwq, ds = _dev(x), _dev(wq), _dev(s)
+    ws = relax_amd.wq_workspace(relax_amd.wq_workspace_bytes(bits, g, n, k, m))
+    ref = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws)
+    xb, wqb, sb, gb = O.make_case(62, 512, 4096, 4096, 4)
+    dxb, dwqb, dsb = _dev(xb), _dev(wqb), _dev(sb)
+    torch.cuda.synchronize()
+    outs = [torch.empty_like(ref) for _ in range(200)]
+    side, main = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _ in range(60):
+            relax_amd.wq_matmul(dxb, dwqb, dsb, 4, gb)
+    with torch.cuda.stream(main):
+        for y in outs:
+            relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws, out=y)
+    torch.cuda.synchronize()
+    bad = [i for i, y in enumerate(outs) if not torch.equal(y.view(torch.int16), ref.view(torch.int16))]
+    assert not bad, bad[:10]
+    assert int(ws[:16384].view(torch.int32).abs().sum()) == 0
