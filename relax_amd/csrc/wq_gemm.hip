@@ -226,12 +226,13 @@ int launch_gemm(const Problem& p, int variant) {
     bool ok = false;
     if (variant == 0)
       ok = (tiles64x128 <= cu_count() && launch_gemm_direct(p, group_shift, 5)) ||
+           (first == 2 && launch_gemm_direct(p, group_shift, 6)) ||
            launch_gemm_direct(p, group_shift, first) || launch_gemm_direct(p, group_shift, first - 1);
     else if (variant >= 21)
       ok = launch_gemm_direct(p, group_shift, variant - 20);
     if (!ok) {
       set_error("gemm kernel: tile-major weights need the direct-weight kernel (K %% 256 == 0, operands below "
-                "1 GiB; variant 0 or 21..25), got M=%lld N=%lld K=%lld variant=%d", (long long)p.m,
+                "1 GiB; variant 0 or 21..26), got M=%lld N=%lld K=%lld variant=%d", (long long)p.m,
                 (long long)p.n, (long long)p.k, variant);
       return -1;
     }
@@ -245,7 +246,10 @@ int launch_gemm(const Problem& p, int variant) {
     const int64_t tiles64x128 = ((p.m + 63) / 64) * ((p.n + 127) / 128);
     const int first = tiles128 <= cu_count() / 2 ? 4 : 2;
     // (and 64x128 tiles with four K groups while even those fit the CUs in one round)
+    // (a last round of 128-row tiles that is at most half full runs as 64-row tiles in a launch of its
+    // own: 2048 x 22016, 372 -> 346 us in isolation, unchanged under sustained load; never slower)
     if ((tiles64x128 <= cu_count() && launch_gemm_direct(p, group_shift, 5)) ||
+        (first == 2 && launch_gemm_direct(p, group_shift, 6)) ||
         launch_gemm_direct(p, group_shift, first) || launch_gemm_direct(p, group_shift, first - 1))
       variant = -1;
     else variant = p.m >= 1024 ? 11 : 12;

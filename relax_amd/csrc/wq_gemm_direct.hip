@@ -80,7 +80,7 @@ template <int BITS, int GROUPS, int TM, int WAVES, bool TILED>
 __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
     half_t* y, int M, int N, int K, int group_shift, int zero_point, int tiles_m, int tiles_n,
-    const Epilogue ep) {
+    const Epilogue ep, int tile_n0) {
   constexpr int BK = 64;
   static_assert(TM == 4 || TM == 2, "row blocks of 32 per wavefront: 128- or 64-row tile");
   static_assert(WAVES == 4 || WAVES == 2, "wavefronts per K group: 256 or 128 output columns");
@@ -114,7 +114,8 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   const int panel = min(in_full, full);
   const int width = panel < full ? PANEL : tiles_n - full * PANEL;
   const int rest = bid - panel * tiles_m * PANEL;
-  const int tile_m = rest / width, tile_n = panel * PANEL + rest % width;
+  // (tile_n0: first column tile of this launch, when a matrix is covered by two launches)
+  const int tile_m = rest / width, tile_n = tile_n0 + panel * PANEL + rest % width;
   const int m0 = tile_m * BM, n0 = tile_n * (WAVES * 64);
 
   const int lane = threadIdx.x & 63;
@@ -519,11 +520,13 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
 
 namespace {
 
+// Column tiles [tile_n0, tile_n0 + tile_count) of the matrix (tile_count < 0: all of them).
 template <int BITS, int GROUPS, int TM, int WAVES, bool TILED>
-bool launch_direct(const Problem& p, int group_shift) {
+bool launch_direct(const Problem& p, int group_shift, int tile_n0 = 0, int tile_count = -1) {
   constexpr int BM = TM * 32, BN = WAVES * 64;
   const int tiles_m = (int)((p.m + BM - 1) / BM);
-  const int tiles_n = (int)((p.n + BN - 1) / BN);
+  const int tiles_n = tile_count >= 0 ? tile_count : (int)((p.n + BN - 1) / BN);
+  if (tiles_n == 0) return true;
   dim3 grid(tiles_m * tiles_n), block(GROUPS * WAVES * 64);
   // four activation stages per K group; the K-group exchange needs 16 KB per wavefront of a group
   constexpr size_t stages = (size_t)GROUPS * 4 * BM * 128, exchange = GROUPS > 1 ? (size_t)WAVES * 16384 : 0;
@@ -535,17 +538,17 @@ bool launch_direct(const Problem& p, int group_shift) {
   hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
-                     tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
+                     tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation}, tile_n0);
   return true;
 }
 
 template <int GROUPS, int TM, int WAVES>
-bool launch_bits(const Problem& p, int group_shift) {
+bool launch_bits(const Problem& p, int group_shift, int tile_n0 = 0, int tile_count = -1) {
   if (p.tiled)
-    return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES, true>(p, group_shift)
-                       : launch_direct<8, GROUPS, TM, WAVES, true>(p, group_shift);
-  return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES, false>(p, group_shift)
-                     : launch_direct<8, GROUPS, TM, WAVES, false>(p, group_shift);
+    return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES, true>(p, group_shift, tile_n0, tile_count)
+                       : launch_direct<8, GROUPS, TM, WAVES, true>(p, group_shift, tile_n0, tile_count);
+  return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES, false>(p, group_shift, tile_n0, tile_count)
+                     : launch_direct<8, GROUPS, TM, WAVES, false>(p, group_shift, tile_n0, tile_count);
 }
 
 }  // namespace
@@ -554,7 +557,7 @@ bool launch_bits(const Problem& p, int group_shift) {
 // two K groups (two per SIMD), each group accumulating half of K; 3 / 4: the same with 64 rows per
 // workgroup -- twice the tiles and about half the time per K step, for M too small to give every CU
 // a 128-row tile; 5: 64 x 128 tile, eight wavefronts in four K groups, for problems that leave CUs
-// idle even with 64 x 256 tiles.
+// idle even with 64 x 256 tiles; 6: variant 2 for whole rounds of tiles plus variant 4 for the rest.
 bool launch_gemm_direct(const Problem& p, int group_shift, int variant) {
   if (!gemm_pipe_applicable(p)) return false;
   // scales are fetched per 256 k: the kernel is laid out for the two benchmark quantizations
@@ -567,6 +570,22 @@ bool launch_gemm_direct(const Problem& p, int group_shift, int variant) {
     case 3: return launch_bits<1, 2, 4>(p, group_shift);
     case 4: return launch_bits<2, 2, 4>(p, group_shift);
     case 5: return launch_bits<4, 2, 2>(p, group_shift);
+    case 6: {
+      // 128 x 256 tiles for the column tiles that fill whole rounds of the CUs, 64 x 256 tiles for the
+      // rest, as a second launch: the last, partly filled round then takes about half as long
+      // (2048 x 22016: 1376 tiles = 5.4 rounds of 256 -> five rounds and 192 half tiles: 372 -> 346 us
+      // when launches come with pauses, no difference when they run back to back for milliseconds --
+      // the part is power limited then, and CUs that idle in a last round let the others clock higher;
+      // 512 x 22016: 2 - 7 % either way).  Applies when the rest is at most half a round and its
+      // 64-row tiles fit one.
+      if (p.k < 512) return false;
+      const int64_t cu = cu_count(), tm128 = (p.m + 127) / 128, tm64 = (p.m + 63) / 64, tn = (p.n + 255) / 256;
+      const int64_t full_cols = (tm128 * tn / cu) * cu / tm128;  // column tiles inside whole rounds
+      const int64_t rest_cols = tn - full_cols;
+      if (full_cols < 1 || rest_cols < 1 || rest_cols * tm128 * 2 > cu || rest_cols * tm64 > cu) return false;
+      return launch_bits<2, 4, 4>(p, group_shift, 0, (int)full_cols) &&
+             launch_bits<2, 2, 4>(p, group_shift, (int)full_cols, (int)rest_cols);
+    }
     default: return false;
   }
 }

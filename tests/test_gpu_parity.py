@@ -230,6 +230,31 @@ def test_gemm_direct_weight_variants_match_oracle(variant, bits, m, n, k):
     assert_close(got, want, (variant, bits, m, n, k))
 
 
+@pytest.mark.parametrize("bits,m,n,k", [(4, 600, 15323, 512), (8, 1000, 8200, 768)])
+def test_gemm_whole_rounds_plus_half_height_rest(bits, m, n, k):
+    """Variant 26, the default when it applies: the column tiles that fill whole rounds of the CUs as
+    128 x 256 tiles, the rest as 64 x 256 tiles in a second launch.  Same arithmetic per output as
+    variant 22 (bit-equal), ragged M and N, canonical and tile-major weights."""
+    import relax_amd
+    from relax_amd import lib
+
+    x, wq, s, g = O.make_case(600 + m, m, n, k, bits)
+    dx, dwq, ds = _dev(x), _dev(wq), _dev(s)
+    y26 = relax_amd.wq_matmul(dx, dwq, ds, bits, g, kernel=lib.KERNEL_GEMM, variant=26)
+    y22 = relax_amd.wq_matmul(dx, dwq, ds, bits, g, kernel=lib.KERNEL_GEMM, variant=22)
+    auto = relax_amd.wq_matmul(dx, dwq, ds, bits, g)
+    wq_t, s_t = relax_amd.wq_tile_weights(dwq, ds, bits, g)
+    t26 = relax_amd.wq_matmul(dx, wq_t, s_t, bits, g, kernel=lib.KERNEL_GEMM, variant=26, tiled_n=n)
+    torch.cuda.synchronize()
+    for other in (y22, auto, t26):
+        assert torch.equal(y26.view(torch.int16), other.view(torch.int16))
+    assert_close(y26.cpu().numpy(), c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16), (26, bits, m, n, k))
+    # where the rest would be more than half a round the variant declines
+    x2, wq2, s2, _ = O.make_case(601, 256, 256, 512, bits)
+    with pytest.raises(lib.WqError, match="does not apply"):
+        run_matmul(x2, wq2, s2, bits, g, kernel=lib.KERNEL_GEMM, variant=26)
+
+
 def test_gemm_direct_weight_variant_refuses_other_layouts():
     """K not a multiple of 256 or a non-default group size: the variant refuses, the default dispatch
     falls back to another GEMM kernel with the same result."""
