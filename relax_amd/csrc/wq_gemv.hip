@@ -33,6 +33,14 @@
 // TILED: weights and scales are in the tile-major layout (wq_tiled.hip), whose blocks are
 // exactly what a wavefront reads per instruction (D = 2): every load of the weight stream
 // is 1 KB contiguous.  Same lanes, same chunks, same order: bit-identical results.
+//
+// ROWS: how the activations reach LDS.  false: a flat index over (row, 16-byte column), two requests
+// per thread ahead of the first weights (batch 1 - 2, or rows longer than the workgroup has
+// threads); true: a thread stages its own column of four or eight rows, all requested ahead of
+// the first weights.
+//
+// KSPLIT: K is split over R workgroups per tile list as well (caller workspace): each writes a
+// float32 partial tile, the last to arrive adds them in the order of the K windows and stores.
 #include <algorithm>
 #include <type_traits>
 
