@@ -284,6 +284,7 @@ def main() -> int:
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--no-epilogue", action="store_true", help="skip the fused-residual leg")
     ap.add_argument("--no-ksplit", action="store_true", help="skip the caller-workspace (K split) leg")
+    ap.add_argument("--no-read-floor", action="store_true", help="skip the read-only floor measurement")
     ap.add_argument("--no-tiled", action="store_true", help="skip the tile-major-weights decode leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times (a kernel of known HBM "
@@ -543,6 +544,58 @@ def main() -> int:
             "us_per_projection_separate_add": round(times[False] * 1e3 / pairs, 3),
             "us_per_projection_fused": round(times[True] * 1e3 / pairs, 3),
             "speedup": round(times[False] / times[True], 3)}
+
+    if not args.no_read_floor:
+        # Context for the HBM fraction: a kernel that only reads -- the same packed weights and scales,
+        # one launch per matrix, the same number of launches in one HIP graph -- i.e. what launch, ramp
+        # and tail leave of the 8 TB/s for these byte counts with no arithmetic, staging or reduction.
+        import ctypes
+
+        so = os.path.join(ROOT, "relax_amd", "csrc", "libmi355x_probe.so")
+        if not os.path.exists(so):
+            raise ImportError(f"{so} is missing: build it with `make -C relax_amd/csrc all`")
+        rd = ctypes.CDLL(so).mi355x_probe_stream_read
+        rd.argtypes = [ctypes.c_void_p, ctypes.c_longlong, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_void_p,
+                       ctypes.c_int, ctypes.c_void_p]
+        best = None
+        for blocks in (256, 512, 1024):
+            sink = torch.empty(blocks * 512, dtype=torch.int32, device=dev)
+
+            def read_pass():
+                sp = int(stream.cuda_stream)
+                for _ in DECODE_BATCHES:
+                    for mats in layers:
+                        for wq, s, n, k in mats:
+                            rc = rd(wq.data_ptr(), wq.numel() * 4, s.data_ptr(), s.numel() * 2, sink.data_ptr(), blocks, sp)
+                            if rc != 0:
+                                raise RuntimeError("stream-read probe: HIP error %d" % rc)
+
+            with torch.cuda.stream(stream):
+                read_pass()
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=stream):
+                    read_pass()
+                gr.replay()
+                torch.cuda.synchronize()
+                r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                r0.record(stream)
+                for _ in range(args.steps):
+                    gr.replay()
+                r1.record(stream)
+                torch.cuda.synchronize()
+            rms = r0.elapsed_time(r1) / args.steps
+            if best is None or rms < best[0]:
+                best = (rms, blocks)
+        weight_bytes = len(DECODE_BATCHES) * sum(wq.numel() * 4 + s.numel() * 2 for mats in layers for wq, s, _, _ in mats)
+        result["read_only_floor"] = {
+            "value": round(weight_bytes / (best[0] * 1e-3) / 1e9, 1), "unit": "GB/s",
+            "frac_of_peak": round(weight_bytes / (best[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 3),
+            "ms_per_step": round(best[0], 4), "workgroups": best[1],
+            "workload": "a kernel that only reads the same weights and scales, one launch per matrix, the "
+                        "same %d launches in one HIP graph (best of 256 / 512 / 1024 workgroups of 512 threads)"
+                        % (len(DECODE_BATCHES) * len(LLAMA7B) * args.layers),
+            "decode_vs_floor": round(best[0] / ms_per_step, 3)}
 
     if not args.no_ksplit:
         # the down projection (4096 x 11008) of every layer at 8 rows: the one case of this step where a

@@ -1,7 +1,14 @@
-// Measurement aid, not part of the quantized-matmul path: a loop of 32x32x16 float16 MFMAs on
+// Measurement aids, not part of the quantized-matmul path.
+//
+// (1) A loop of 32x32x16 float16 MFMAs on
 // operands that stay in registers (no memory, LDS or other VALU work inside the loop).  What it
 // sustains depends only on the operand values, which is how the matrix-pipe rate that the GEMM
 // kernels can be held against on real data (as opposed to zeros) is measured.
+//
+// (2) A kernel that only reads: two buffers streamed once with 16-byte loads, four in flight per lane,
+// and folded into one word per thread.  Launched like a decode GEMV (one launch per weight matrix), it
+// gives the time that launch, ramp and tail take for a given byte count on this part with no arithmetic,
+// staging or reduction at all -- the floor the decode kernels are held against.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -48,7 +55,43 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(const half8_t* __restri
   }
 }
 
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(512) void probe_stream_read_kernel(const u32x4_t* __restrict__ a, long long na,
+                                                                const u32x4_t* __restrict__ b, long long nb,
+                                                                unsigned int* __restrict__ out) {
+  const long long stride = (long long)gridDim.x * 512, t = (long long)blockIdx.x * 512 + threadIdx.x;
+  u32x4_t f = {0u, 0u, 0u, 0u};
+  auto sweep = [&](const u32x4_t* __restrict__ p, long long n) {
+    long long i = t;
+    for (; i + 3 * stride < n; i += 4 * stride) {
+      const u32x4_t v0 = __builtin_nontemporal_load(p + i), v1 = __builtin_nontemporal_load(p + i + stride),
+                    v2 = __builtin_nontemporal_load(p + i + 2 * stride),
+                    v3 = __builtin_nontemporal_load(p + i + 3 * stride);
+      f ^= v0 ^ v1 ^ v2 ^ v3;
+    }
+    for (; i < n; i += stride) f ^= __builtin_nontemporal_load(p + i);
+  };
+  sweep(a, na);
+  sweep(b, nb);
+  out[t] = f[0] ^ f[1] ^ f[2] ^ f[3];
+}
+
 }  // namespace
+
+// Reads `bytes_a` bytes at `a` and `bytes_b` at `b` (16-byte aligned, multiples of 16) once, with
+// `blocks` workgroups of eight wavefronts; `out` receives blocks * 512 words.  Returns 0 or the HIP
+// error code of the launch.
+extern "C" __attribute__((visibility("default"))) int mi355x_probe_stream_read(const void* a, long long bytes_a,
+                                                                             const void* b, long long bytes_b,
+                                                                             void* out, int blocks, void* stream) {
+  if (a == nullptr || out == nullptr || blocks <= 0 || bytes_a < 0 || bytes_b < 0 || (bytes_a | bytes_b) % 16 != 0)
+    return -1;
+  hipLaunchKernelGGL(probe_stream_read_kernel, dim3((unsigned)blocks), dim3(512), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const u32x4_t*>(a), bytes_a / 16, static_cast<const u32x4_t*>(b), bytes_b / 16,
+                     static_cast<unsigned int*>(out));
+  return (int)hipGetLastError();
+}
 
 // Launches `blocks` workgroups of four wavefronts (one workgroup per CU fills every SIMD with one
 // wavefront), each wavefront issuing 16 * iters MFMAs

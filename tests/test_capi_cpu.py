@@ -78,13 +78,14 @@ def test_workspace_size_query_without_a_gpu():
 
 
 def test_measurement_probe_library_is_built_and_separate():
-    """bench.py --probe-mfma loads its kernel from a library of its own; the product library has
-    no symbol of it."""
+    """bench.py's measurement aids (the MFMA rate probe and the read-only floor kernel) live in a library
+    of their own; the product library has no symbol of them."""
     probe = os.path.join(os.path.dirname(lib.SO_PATH), "libmi355x_probe.so")
     assert os.path.exists(probe), "make -C relax_amd/csrc all"
     out = subprocess.run(["nm", "-D", "--defined-only", probe], capture_output=True, text=True).stdout
-    assert [l.split()[-1] for l in out.splitlines() if " T " in l] == ["mi355x_probe_mfma_f16"]
-    assert not hasattr(lib.load(), "mi355x_probe_mfma_f16")
+    assert sorted(l.split()[-1] for l in out.splitlines() if " T " in l) == ["mi355x_probe_mfma_f16",
+                                                                              "mi355x_probe_stream_read"]
+    assert not hasattr(lib.load(), "mi355x_probe_mfma_f16") and not hasattr(lib.load(), "mi355x_probe_stream_read")
 
 
 @pytest.mark.parametrize("kw,msg", [
