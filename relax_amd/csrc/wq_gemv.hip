@@ -70,13 +70,20 @@ struct GemvArgs {
 };
 
 template <int BITS, int WAVES, int D, int SPL, bool TILED, bool ROWS, bool KSPLIT>
-// (scalar kernel arguments instead of one struct: the first 16 dwords -- the operand pointers
-// and the shape -- are preloaded into SGPRs at wavefront launch, which takes the argument fetch
-// out of the start-up latency of a 5 - 15 us kernel)
+// Scalar kernel arguments instead of one struct, and in this order: the first 14 dwords of the
+// argument segment are preloaded into SGPRs at wavefront launch (16 user SGPRs less the segment
+// pointer); anything after them is fetched by a scalar load from host-visible memory.
+// Everything the staging and the weight stream need -- the three input pointers, the shape, the
+// plan and the grid size (gridDim.x is itself a load from the end of the segment), 14 dwords --
+// therefore comes first, and what only the final store needs (y, the epilogue, the K split's
+// workspace) after it.
 __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
-    const half_t* x_, const uint32_t* wq_, const half_t* scales_, half_t* y_, int M_, int N_, int K_,
-    int group_shift_, int zero_point_, int lds_stride_, int tiles_, int max_tiles_, int phase_chunks_,
-    const Epilogue ep_, int ksplit_, float* partials_, unsigned int* counters_) {
+    const half_t* x_, const uint32_t* wq_, const half_t* scales_, int M_, int N_, int K_,
+    int shift_and_zero_, int max_tiles_, int phase_chunks_, int ksplit_, int grid_, half_t* y_, const Epilogue ep_,
+    float* partials_, unsigned int* counters_) {
+  const int group_shift_ = shift_and_zero_ & 0xFF, zero_point_ = shift_and_zero_ >> 8;
+  const int tiles_ = (N_ + 15) >> 4;
+  const int lds_stride_ = phase_chunks_ * (128 / BITS) + 8;  // halves per staged row (launch_one's plan)
   GemvArgs a;
   a.x = x_;
   a.wq = wq_;
@@ -120,12 +127,13 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
 
   // Tiles of this workgroup: tile0, tile0 + tstride, ...  With the K split, R consecutive workgroups
   // share a tile list and each walks its own window of K (phase_chunks chunks from kr * phase_chunks).
-  const int G = gridDim.x;
+  const int G = grid_;
   const int R = KSPLIT ? ksplit_ : 1;
   const int kr = KSPLIT ? (int)blockIdx.x % R : 0;
   const int tile0 = KSPLIT ? (int)blockIdx.x / R : (int)blockIdx.x;
   const int tstride = KSPLIT ? G / R : G;
-  const int my_tiles = (a.tiles - tile0 + tstride - 1) / tstride;
+  // (= ceil((tiles - tile0) / tstride) without the division: max_tiles is the ceiling for tile0 = 0)
+  const int my_tiles = a.max_tiles - (tile0 + (a.max_tiles - 1) * tstride >= a.tiles ? 1 : 0);
 
   const Q4Consts qc = make_q4_consts(a.zero_point);
   const half_t* xrow = xs + (size_t)(col < M ? col : 0) * a.lds_stride;
@@ -217,8 +225,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     acc = float4_t{0.f, 0.f, 0.f, 0.f};
   };
 
-  const int nphases = KSPLIT ? 1 : (nchunks + a.phase_chunks - 1) / a.phase_chunks;
-  for (int ph = 0; ph < nphases; ++ph) {
+  for (int ph = 0; KSPLIT ? ph < 1 : ph * a.phase_chunks < nchunks; ++ph) {
     const int chunk_base = (KSPLIT ? kr : ph) * a.phase_chunks;
     const int ph_chunks = min(a.phase_chunks, nchunks - chunk_base);
     const int nsuper = (ph_chunks + 4 * D - 1) / (4 * D);
@@ -265,12 +272,34 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
           const int m = idx / vec_per_row, kv = idx - m * vec_per_row;
           *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = permute_x(v);
         };
-        const u32x4 x0 = x_load(tid), x1 = x_load(tid + NT);
+        // (the first two vectors without the division when a row has at least as many vectors as the
+        // workgroup has threads -- K >= 4096: they are in row 0 or 1; the start-up of a 5 us kernel is
+        // a few hundred instructions, and a division is forty of them)
+        int m0, kv0, m1, kv1;
+        if (vec_per_row >= NT) {
+          m0 = 0;
+          kv0 = tid;
+          m1 = tid + NT >= vec_per_row ? 1 : 0;
+          kv1 = tid + NT - m1 * vec_per_row;
+        } else {
+          m0 = tid / vec_per_row;
+          kv0 = tid - m0 * vec_per_row;
+          m1 = (tid + NT) / vec_per_row;
+          kv1 = tid + NT - m1 * vec_per_row;
+        }
+        auto x_load_at = [&](int m, int kv) -> u32x4 {
+          const bool ok = m < M && kbase + kv * 8 < K;
+          return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
+        };
+        auto x_store_at = [&](int m, int kv, u32x4 v) {
+          if (m < M) *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = permute_x(v);
+        };
+        const u32x4 x0 = x_load_at(m0, kv0), x1 = x_load_at(m1, kv1);
         __builtin_amdgcn_sched_barrier(0);
         load_super(b0, 0, ss_begin, chunk_base, ss_end);
         __builtin_amdgcn_sched_barrier(0);
-        x_store(tid, x0);
-        x_store(tid + NT, x1);
+        x_store_at(m0, kv0, x0);
+        x_store_at(m1, kv1, x1);
         for (int idx = tid + 2 * NT; idx < total; idx += 4 * NT) {
           const u32x4 v0 = x_load(idx), v1 = x_load(idx + NT), v2 = x_load(idx + 2 * NT), v3 = x_load(idx + 3 * NT);
           x_store(idx, v0);
@@ -481,8 +510,8 @@ int launch_one(const Problem& p, int group_shift, const Plan& plan, int ksplit =
                             lds_ok))
       return kFailed;
     hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT>), dim3(plan.grid), dim3(WAVES * 64),
-                       plan.lds_bytes, p.stream, a.x, a.wq, a.scales, a.y, a.M, a.N, a.K, a.group_shift,
-                       a.zero_point, a.lds_stride, a.tiles, a.max_tiles, a.phase_chunks, a.ep, ksplit, partials,
+                       plan.lds_bytes, p.stream, a.x, a.wq, a.scales, a.M, a.N, a.K,
+                       a.group_shift | (a.zero_point << 8), a.max_tiles, a.phase_chunks, ksplit, plan.grid, a.y, a.ep, partials,
                        counters);
     return kLaunched;
   };
