@@ -79,8 +79,11 @@ struct RawB {
 template <int BITS, int GROUPS, int TM, int WAVES, bool TILED>
 __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
-    half_t* y, int M, int N, int K, int group_shift, int zero_point, int tiles_m, int tiles_n,
-    const Epilogue ep, int tile_n0) {
+    int M, int N, int K, int shift_and_zero, int tiles_m, int tiles_n, int tile_n0, half_t* y,
+    const Epilogue ep) {
+  // (argument order: the first 14 dwords are preloaded into SGPRs at wavefront launch, later ones are
+  // a scalar load at the start of the kernel; what the K loop needs comes first, y and the epilogue last)
+  const int group_shift = shift_and_zero & 0xFF, zero_point = shift_and_zero >> 8;
   constexpr int BK = 64;
   static_assert(TM == 4 || TM == 2, "row blocks of 32 per wavefront: 128- or 64-row tile");
   static_assert(WAVES == 4 || WAVES == 2, "wavefronts per K group: 256 or 128 output columns");
@@ -536,9 +539,9 @@ bool launch_direct(const Problem& p, int group_shift, int tile_n0 = 0, int tile_
   if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED>, (int)lds_bytes, lds_ok))
     return false;
   hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED>), grid, block, lds_bytes, p.stream,
-                     (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
-                     (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point, tiles_m,
-                     tiles_n, Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation}, tile_n0);
+                     (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales, (int)p.m, (int)p.n,
+                     (int)p.k, group_shift | (p.zero_point << 8), tiles_m, tiles_n, tile_n0, (half_t*)p.y,
+                     Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
   return true;
 }
 
