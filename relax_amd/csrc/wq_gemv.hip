@@ -567,17 +567,16 @@ namespace {
 
 // The variants the default dispatch tries, in order (see launch_gemv).
 const int* default_order(const Problem& p) {
-  // Measured on MI355X (Llama-2-7B shapes): up to 4 rows run best with two 8-wave
-  // workgroups per CU, larger batches (more LDS per workgroup) with one.  Two-chunk
-  // super steps first, single chunks (any K) as the fallback.
-  // (rows of more than 2 KB -- int8 weights, long K -- already give one workgroup per CU
-  // enough bytes in flight: two per CU measured 8-11 % slower there)
+  // Measured on MI355X (Llama-2-7B and 13B shapes): one or two rows of int4 weights run best with two
+  // 8-wave workgroups per CU (4096 x 11008 at batch 1: 8.7 against 9.3 us), everything else with one
+  // (12288 x 4096 at 4 rows: 8.7 against 9.0 us; int8 15360 x 5120 at batch 1: 18.2 against 19.6 us).
+  // Two-chunk super steps first, single chunks (any K) as the fallback.
   static const int small[] = {25, 15, 24, 14}, large[] = {15, 14, 15, 14};
   // (between one and two row tiles per CU a second workgroup per CU only unbalances them:
   // 5120 x 5120, 9.9 against 8.7 us)
-  const int64_t row_bytes = p.k * p.bits / 8, tiles = (p.n + 15) / 16;
+  const int64_t tiles = (p.n + 15) / 16;
   const bool fills = tiles <= cu_count() || tiles >= 2 * cu_count();
-  return (p.m <= 4 && row_bytes <= 2048 && fills) ? small : large;
+  return (p.m <= 2 && p.bits == 4 && fills) ? small : large;
 }
 
 // Whether `variant` can be launched for p: K divisibility and an LDS plan (partial-tile slots of
