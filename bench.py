@@ -379,6 +379,15 @@ def main() -> int:
     gbs = bytes_per_step / (ms_per_step * 1e-3) / 1e9
     avg_launch_us = ms_per_step * 1e3 / launches_per_step
 
+    # which kernel family the library's own choice runs for each of the eight shape/batch cases
+    fam = {lib.KERNEL_GEMV: "wq::wq_gemv_kernel", lib.KERNEL_SKINNY: "wq::wq_skinny_kernel", lib.KERNEL_GEMM: "gemm"}
+    chosen = {}
+    for m in DECODE_BATCHES:
+        for _, n, k in LLAMA7B:
+            chosen.setdefault(fam[lib.load().mi355x_wq_select_kernel(lib.make_desc(4, 32, n, k), m)], []).append(
+                "%dx%d at batch %d" % (n, k, m))
+    decode_kernels = "; ".join("%s (%d of the 8 shape/batch cases%s)" % (
+        name, len(cs), "" if len(cs) > 2 else ": " + ", ".join(cs)) for name, cs in sorted(chosen.items(), key=lambda kv: -len(kv[1])))
     result = {
         "metric": "q4f16 GEMV GB/s + GEMM TFLOP/s (% roofline), Llama-7B shapes, 1 GPU",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -391,7 +400,7 @@ def main() -> int:
                    "launches_per_step": launches_per_step, "bytes_per_step": bytes_per_step},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "wq::wq_gemv_kernel (7 of the 8 shape/batch cases; batch 8 on 4096x11008 runs wq::wq_skinny_kernel)",
+                     "kernel": decode_kernels,
                      "bytes_per_launch": bytes_per_step // launches_per_step,
                      "avg_launch_us": round(avg_launch_us, 3)},
     }

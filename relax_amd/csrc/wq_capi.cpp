@@ -125,21 +125,19 @@ bool check_ptr(const void* p, const char* name, size_t align) {
 int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
   Problem p{nullptr, nullptr, nullptr, nullptr, m, d->n, d->k, d->bits, d->group, d->zero_point, nullptr};
   if (gemv_applicable(p)) {
-    // The GEMV kernel stages the activations in LDS.  Measured on MI355X: once they no longer fit
-    // there in one piece (more than 144 KB beside the partial-tile slots, so that K is walked in
-    // phases) and there is at most one row tile per CU to amortise the staging, the
-    // register-activation kernel is faster.  (16 rows of K = 4096, 128 KB, still fit: 7.7 against 8.8 us.)
-    const int64_t x_bytes = m * d->k * 2, tiles = (d->n + 15) / 16;
-    // (for rows of 16384 and more the staging kernel wins again: 4096 x 16384 at 4 rows 13.7 against
-    // 17.4 us; and with at most 2048 columns of K and 256 row tiles the matrix is so small -- 4 MB --
-    // that the staging kernel's start-up costs more than it saves: 4096 x 2048, 5.6 against 4.9 us)
-    const bool big_x = x_bytes > 144 * 1024 && tiles <= 256 && d->k < 16384;
+    // The GEMV kernel stages the activations in LDS, in K phases when they do not fit in one piece.
+    // (A rule that sent such problems with at most one row tile per CU to the register-activation
+    // kernel dated from a slower staging path: 16 rows on 4096 x 11008 now take 15.5 against 16.7 us,
+    // 8 rows 12.7 against 12.8 us.)
+    const int64_t tiles = (d->n + 15) / 16;
+    // (with at most 2048 columns of K and 256 row tiles the matrix is so small -- 4 MB -- that the
+    // staging kernel's start-up costs more than it saves: 4096 x 2048, 5.6 against 4.9 us)
     const bool tiny = tiles <= 256 && d->k <= 2048;
     // Tile-major weights, at most two row tiles per CU: the staging is spread over so few tiles that the
     // register-activation kernel, whose loads are as contiguous on this layout, wins -- int8 at every
     // batch (5120 x 5120: 8.0 - 10.6 us against 9.4 - 12.6 us; 5120 x 13824 at 8 rows: 19.2 against
     // 24.1 us); int4 with rows of up to 2 KB at up to 8 rows (4096 x 4096: 4.3 against 4.6 us at batch 1)
-    // or once there is more than one tile per CU; int4 with longer rows from 8 rows on, from 4 with more
+    // or once there is more than one tile per CU; int4 with longer rows at 8 - 12 rows, from 4 with more
     // than one tile per CU.  From 640 tiles on the staging kernel is ahead again (10240 x 4096: 7.9
     // against 8.8 us).
     bool few_tiles = false;
@@ -147,7 +145,7 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
       const bool long_rows = d->k * d->bits / 8 > 4096, over_one = tiles > cu_count();
       few_tiles = (d->bits == 8 && !(m <= 2 && tiles > cu_count() + cu_count() / 2)) ||
                   (d->bits == 4 && !long_rows && (m <= 8 || over_one)) ||
-                  (d->bits == 4 && long_rows && (m >= 8 || (m >= 4 && over_one)));
+                  (d->bits == 4 && long_rows && ((m >= 8 && m <= 12) || (m >= 4 && over_one)));
     }
     // (and int4 with up to four tiles per CU at 12 rows or more, where the staging kernel's time has grown with
     // the rows and the other's has not: 16384 x 4096 at 16 rows, 11.4 against 13.4 us)
@@ -156,7 +154,7 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
     // (rows of 16384 and more, one tile per CU: the staging kernel at batch 1 - 4, 17.7 against 19.8 us, the
     // other at 8 - 12 rows, 14.7 against 16.7 us)
     if (tiled && d->k >= 16384 && tiles <= cu_count() && m >= 8 && m <= 12) few_tiles = true;
-    if (!big_x && !tiny && !few_tiles) return MI355X_WQ_KERNEL_GEMV;
+    if (!tiny && !few_tiles) return MI355X_WQ_KERNEL_GEMV;
   }
   if (m > kSkinnyMaxM) return MI355X_WQ_KERNEL_GEMM;
   // 17..64 rows.  The skinny kernel re-reads the activations from L2 once per 16-row weight tile, so

@@ -467,7 +467,18 @@ bool make_plan(const Problem& p, int wgs_per_cu, Plan* out) {
   int phase_chunks = (int)(max_k / ch) / unit * unit;
   if (phase_chunks <= 0) return false;
   const int whole = (nchunks + 4 * D - 1) / (4 * D) * (4 * D);  // K as one phase, padded to a super step
-  if (phase_chunks >= whole) phase_chunks = whole;
+  if (phase_chunks >= whole) {
+    phase_chunks = whole;
+  } else if (p.m > 2) {
+    // K is walked in phases anyway: phases of equal length, and of at most one 16-byte vector per
+    // thread and row where that costs at most one phase more, so that the staging takes the
+    // column-per-thread path
+    const int per_vec = WAVES * 64 * 8 / ch;  // chunks whose vectors one pass of the workgroup covers
+    int nph = (nchunks + phase_chunks - 1) / phase_chunks;
+    const int capped = per_vec / unit * unit;
+    if (capped > 0 && (nchunks + capped - 1) / capped <= nph + 1) nph = (nchunks + capped - 1) / capped;
+    phase_chunks = std::min(phase_chunks, ((nchunks + nph - 1) / nph + unit - 1) / unit * unit);
+  }
   out->grid = grid;
   out->max_tiles = max_tiles;
   out->phase_chunks = phase_chunks;

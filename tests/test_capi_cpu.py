@@ -122,11 +122,12 @@ def test_kernel_selection_by_rows():
     assert L.mi355x_wq_select_kernel(d, 8) == lib.KERNEL_GEMV
     # 16 rows x 4096 = 128 KB of activations still fit the LDS in one piece
     assert L.mi355x_wq_select_kernel(d, 16) == lib.KERNEL_GEMV
-    # 16 rows x 8192 = 256 KB for only 256 row tiles: staging them in phases per workgroup does not pay
-    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 8192), 16) == lib.KERNEL_SKINNY
+    # 16 rows x 8192 = 256 KB: staged in K phases
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 8192), 16) == lib.KERNEL_GEMV
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 22016, 4096), 16) == lib.KERNEL_GEMV
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 11008), 2) == lib.KERNEL_GEMV
-    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 11008), 8) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 11008), 8) == lib.KERNEL_GEMV
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 2048), 8) == lib.KERNEL_SKINNY  # a 4 MB matrix
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 22016, 11008), 8) == lib.KERNEL_GEMV
     # a vocabulary-sized projection: too many row tiles per workgroup for the GEMV kernel's LDS slots
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 152064, 4096), 1) == lib.KERNEL_SKINNY
