@@ -225,7 +225,10 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     acc = float4_t{0.f, 0.f, 0.f, 0.f};
   };
 
-  for (int ph = 0; KSPLIT ? ph < 1 : ph * a.phase_chunks < nchunks; ++ph) {
+  // One K phase: stage its activations, stream every tile of the workgroup over it.  The first phase
+  // is a copy of its own ahead of the loop over the others: inside a loop the compiler hoists the
+  // stream's constants in front of it, i.e. in front of the kernel's first requests.
+  auto run_phase = [&](const int ph) {
     const int chunk_base = (KSPLIT ? kr : ph) * a.phase_chunks;
     const int ph_chunks = min(a.phase_chunks, nchunks - chunk_base);
     const int nsuper = (ph_chunks + 4 * D - 1) / (4 * D);
@@ -378,7 +381,10 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     // a wavefront without work in this phase still owns slots that the epilogue sums
     if (cnt == 0 && ph == 0)
       for (int i = 0; i < my_tiles; ++i) flush_tile(i, true);
-  }
+  };
+  run_phase(0);
+  if constexpr (!KSPLIT)
+    for (int ph = 1; ph * a.phase_chunks < nchunks; ++ph) run_phase(ph);
 
   // ---- sum the wavefronts' partial tiles, convert, store -----------------------------
   __syncthreads();
