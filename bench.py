@@ -33,7 +33,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
 # HBM bytes per GEMV launch of this workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (mean per dispatch, scaled by a 256 MiB copy: FETCH_SIZE reads half the true KiB, WRITE_SIZE
 # the true KiB); measurement and commands in profiles/gemv_decode_llama7b.md.
-GEMV_HBM_TRAFFIC_PER_LAUNCH = int((14165.4 * 2.0 + 93.4 * 1.0) * 1024)
+GEMV_HBM_TRAFFIC_PER_LAUNCH = int((14170.0 * 2.0 + 93.4 * 1.0) * 1024)
 
 
 def algorithmic_bytes(bits: int, group: int, m: int, n: int, k: int) -> int:

@@ -133,24 +133,18 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
     // (with at most 2048 columns of K and 256 row tiles the matrix is so small -- 4 MB -- that the
     // staging kernel's start-up costs more than it saves: 4096 x 2048, 5.6 against 4.9 us)
     const bool tiny = tiles <= 256 && d->k <= 2048;
-    // Tile-major weights, at most two row tiles per CU: the staging is spread over so few tiles that the
-    // register-activation kernel, whose loads are as contiguous on this layout, wins -- int8 at every
-    // batch (5120 x 5120: 8.0 - 10.6 us against 9.4 - 12.6 us; 5120 x 13824 at 8 rows: 19.2 against
-    // 24.1 us); int4 with rows of up to 2 KB at up to 8 rows (4096 x 4096: 4.3 against 4.6 us at batch 1)
-    // or once there is more than one tile per CU; int4 with longer rows at 8 - 12 rows, from 4 with more
-    // than one tile per CU.  From 640 tiles on the staging kernel is ahead again (10240 x 4096: 7.9
-    // against 8.8 us).
+    // Tile-major weights, at most two row tiles per CU (N <= 8192): the staging is spread over so few
+    // tiles that the register-activation kernel, whose loads are as contiguous on this layout, wins for
+    // int8 from 4 rows on, from 2 with more than one tile per CU (5120 x 5120: 7.9 - 10.7 us against
+    // 8.7 - 11.6 us; 5120 x 13824 at 8 rows: 19.3 against 22.7 us), and for int4 with rows of at least
+    // 4 KB at 8 rows and more with more than one tile per CU (5120 x 11008 at 8 rows: 13.7 against
+    // 14.7 us).  Everywhere else the staging kernel is ahead or level since its start-up was shortened
+    // (int4 4096 x 4096: 4.2 - 5.4 us against 4.3 - 6.5 us; from 640 tiles on always).
     bool few_tiles = false;
     if (tiled && tiles <= 2 * cu_count() && d->k < 16384) {
-      const bool long_rows = d->k * d->bits / 8 > 4096, over_one = tiles > cu_count();
-      few_tiles = (d->bits == 8 && !(m <= 2 && tiles > cu_count() + cu_count() / 2)) ||
-                  (d->bits == 4 && !long_rows && (m <= 8 || over_one)) ||
-                  (d->bits == 4 && long_rows && ((m >= 8 && m <= 12) || (m >= 4 && over_one)));
+      const bool long_rows = d->k * d->bits / 8 >= 4096, over_one = tiles > cu_count();
+      few_tiles = (d->bits == 8 && (m >= 4 || (m >= 2 && over_one))) || (d->bits == 4 && long_rows && m >= 8 && over_one);
     }
-    // (and int4 with up to four tiles per CU at 12 rows or more, where the staging kernel's time has grown with
-    // the rows and the other's has not: 16384 x 4096 at 16 rows, 11.4 against 13.4 us)
-    if (tiled && d->bits == 4 && m >= 12 && tiles > 2 * cu_count() && tiles <= 4 * cu_count() && d->k < 16384)
-      few_tiles = true;
     // (rows of 16384 and more, one tile per CU: the staging kernel at batch 1 - 4, 17.7 against 19.8 us, the
     // other at 8 - 12 rows, 14.7 against 16.7 us)
     if (tiled && d->k >= 16384 && tiles <= cu_count() && m >= 8 && m <= 12) few_tiles = true;
@@ -169,9 +163,11 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
     // On tile-major weights the skinny kernel's loads are contiguous and it holds out longer
     // (N = 12288, 32 rows: 14 us against the GEMM's 22 us): for int4 the GEMM takes over from 40 rows
     // with 160 or more column tiles and from 57 rows with 64 or more; int8 stays with the skinny
-    // kernel up to 64 rows (27648 x 5120 at 48 rows: 44 against 50 us).
+    // kernel up to 56 rows (27648 x 5120 at 48 rows: 44 against 50 us) and goes to the GEMM beyond
+    // with 160 or more column tiles (32000 x 4096 at 64 rows: 42 against 48 us).
     if (direct_small_tile && d->bits == 4 && ((tiles128 >= 160 && m >= 40) || (m > 56 && tiles128 >= 64)))
       return MI355X_WQ_KERNEL_GEMM;
+    if (direct_small_tile && d->bits == 8 && tiles128 >= 160 && m > 56) return MI355X_WQ_KERNEL_GEMM;
     return MI355X_WQ_KERNEL_SKINNY;
   }
   if (direct_small_tile && ((m >= 24 && tiles128 >= 160) || (d->bits == 4 && m > 32 && tiles128 >= 96) ||
