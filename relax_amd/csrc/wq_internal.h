@@ -61,3 +61,15 @@ bool ensure_dynamic_lds(const void* kernel, int bytes, bool* done);
 int cu_count();
 
 }  // namespace wq
+
+// The packed boundary's pieces that the subgraph module (wq_module.cpp) shares.
+struct mi355x_wq_callspec;
+union mi355x_tvm_value;
+namespace wq {
+// mi355x_wq_packed_call; when `wq_tiled` is given, a matmul reads these tile-major copies instead of
+// the canonical tensors in the wq / scales slots (which are still validated and give N, K and group).
+int packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes, int num_args,
+                             const void* wq_tiled, const void* scales_tiled);
+// Forwards the recorded error to TVM's error slot when the process has one; returns -1.
+int packed_fail();
+}  // namespace wq

@@ -125,6 +125,15 @@ void* mi355x_wq_packed_get_stream(void) { return g_stream; }
 
 int mi355x_wq_packed_call(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes,
                           int num_args) {
+  return wq::packed_call_with_weights(spec, args, type_codes, num_args, nullptr, nullptr);
+}
+
+}  // extern "C"
+
+int wq::packed_fail() { return fail(); }
+
+int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes,
+                                 int num_args, const void* wq_tiled, const void* scales_tiled) {
   if (spec == nullptr) {
     wq::set_error("call spec is NULL");
     return fail();
@@ -259,10 +268,14 @@ int mi355x_wq_packed_call(const mi355x_wq_callspec* spec, mi355x_tvm_value* args
     wq::set_error("tensors live on ROCm device %d but the current HIP device is %d", dev, cur);
     return fail();
   }
+  if (wq_tiled != nullptr && is_matmul)
+    return mi355x_wq_matmul_tiled(&d, px, wq_tiled, scales_tiled, &ep, po, m, g_stream) == 0 ? 0 : fail();
   const int rc = is_matmul ? mi355x_wq_matmul_fused(&d, px, pw, ps, &ep, po, m, g_stream)
                            : mi355x_wq_dequantize(&d, pw, ps, po, g_stream);
   return rc == 0 ? 0 : fail();
 }
+
+extern "C" {
 
 // Fixed-name entries: arguments in the canonical order x, wq, scales, [bias | residual], out.
 #define MI355X_FIXED_ENTRY(NAME, OP, BITS, ZP, BIAS, RES, ACT)                                      \

@@ -12,7 +12,7 @@ KERNEL_AUTO, KERNEL_GEMV, KERNEL_GEMM, KERNEL_SKINNY = 0, 1, 2, 3
 ACT_NONE, ACT_RELU = 0, 1
 ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "relax.nn.relu": ACT_RELU}
 
-# every symbol include/mi355x_wq.h and include/mi355x_wq_packed.h declare
+# every symbol include/mi355x_wq.h, include/mi355x_wq_packed.h and include/mi355x_wq_module.h declare
 EXPORTED_SYMBOLS = (
     "mi355x_wq_matmul", "mi355x_wq_matmul_ex", "mi355x_wq_matmul_fused", "mi355x_wq_matmul_fused_ex",
     "mi355x_wq_dequantize", "mi355x_wq_check",
@@ -26,6 +26,11 @@ EXPORTED_SYMBOLS = (
     "mi355x_q4f16_matmul_tiled", "mi355x_q8f16_matmul_tiled", "mi355x_q4f16_matmul_ws", "mi355x_q8f16_matmul_ws",
     "mi355x_wq_packed_call", "mi355x_wq_packed_set_stream",
     "mi355x_wq_packed_get_stream", "mi355x_wq_register_tvm_globals",
+    "mi355x_wq_module_type_key", "mi355x_wq_module_create", "mi355x_wq_module_destroy", "mi355x_wq_module_symbol",
+    "mi355x_wq_module_num_consts", "mi355x_wq_module_const_name", "mi355x_wq_module_json",
+    "mi355x_wq_module_initialized", "mi355x_wq_module_get_function", "mi355x_wq_module_init",
+    "mi355x_wq_module_call", "mi355x_wq_module_save_to_binary", "mi355x_wq_module_load_from_binary",
+    "mi355x_wq_module_create_from_json",
 )
 PACKED_ENTRIES = tuple(s for s in EXPORTED_SYMBOLS if s.startswith(("mi355x_q4f16_", "mi355x_q8f16_")))
 
@@ -94,6 +99,25 @@ def load() -> C.CDLL:
     for name in PACKED_ENTRIES:
         getattr(L, name).argtypes = [vp, C.POINTER(ci), ci, vp, C.POINTER(ci), vp]
     L.mi355x_wq_packed_call.argtypes = [vp, vp, C.POINTER(ci), ci]
+    i32 = C.c_int32
+    L.mi355x_wq_module_type_key.restype = C.c_char_p
+    L.mi355x_wq_module_create.argtypes = [C.c_char_p, vp, C.POINTER(C.c_char_p), C.POINTER(i32), i32, i32, C.POINTER(vp)]
+    L.mi355x_wq_module_destroy.argtypes = [vp]
+    L.mi355x_wq_module_destroy.restype = None
+    for name in ("symbol", "json"):
+        getattr(L, "mi355x_wq_module_" + name).argtypes = [vp]
+        getattr(L, "mi355x_wq_module_" + name).restype = C.c_char_p
+    L.mi355x_wq_module_const_name.argtypes = [vp, i32]
+    L.mi355x_wq_module_const_name.restype = C.c_char_p
+    L.mi355x_wq_module_num_consts.argtypes = [vp]
+    L.mi355x_wq_module_initialized.argtypes = [vp]
+    L.mi355x_wq_module_get_function.argtypes = [vp, C.c_char_p, C.POINTER(vp), C.POINTER(vp)]
+    L.mi355x_wq_module_init.argtypes = [vp, C.POINTER(vp), i32]
+    L.mi355x_wq_module_call.argtypes = [vp, vp, C.POINTER(ci), ci]
+    L.mi355x_wq_module_save_to_binary.argtypes = [vp, vp, i64]
+    L.mi355x_wq_module_save_to_binary.restype = i64
+    L.mi355x_wq_module_load_from_binary.argtypes = [vp, i64, C.POINTER(i64), C.POINTER(vp)]
+    L.mi355x_wq_module_create_from_json.argtypes = [C.c_char_p, C.c_char_p, C.POINTER(C.c_char_p), i32, C.POINTER(vp)]
     _lib = L
     return L
 

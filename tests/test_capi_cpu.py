@@ -18,7 +18,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def declared_symbols():
     names = []
-    for h in ("mi355x_wq.h", "mi355x_wq_packed.h"):
+    for h in ("mi355x_wq.h", "mi355x_wq_packed.h", "mi355x_wq_module.h"):
         text = open(os.path.join(ROOT, "include", h)).read()
         names += re.findall(r"MI355X_WQ_API\s+[\w\s\*]+?\b(mi355x_\w+)\s*\(", text)
     return names
@@ -27,7 +27,7 @@ def declared_symbols():
 def test_library_exports_every_declared_symbol():
     L = lib.load()
     names = declared_symbols()
-    assert len(names) == 36 and set(names) == set(lib.EXPORTED_SYMBOLS)
+    assert len(names) == 50 and set(names) == set(lib.EXPORTED_SYMBOLS)
     for n in names:
         assert hasattr(L, n), n
     assert L.mi355x_wq_version() >= 100
@@ -369,6 +369,7 @@ C_CLIENT = r"""
 #include <string.h>
 #include "mi355x_wq.h"
 #include "mi355x_wq_packed.h"
+#include "mi355x_wq_module.h"
 
 int main(void) {
   mi355x_wq_desc d = {4, 32, 7, 0, 4096, 4096};
@@ -385,6 +386,30 @@ int main(void) {
   if (strstr(mi355x_wq_last_error(), "x is NULL") == NULL) return 6;
   if (mi355x_wq_packed_call(&spec, NULL, NULL, 4) != -1) return 7;
   if (sizeof(mi355x_dl_tensor) != 48 || sizeof(mi355x_tvm_value) != 8) return 8;  /* DLPack / TVMValue ABI sizes */
+  {
+    /* the subgraph module from plain C: create, look a function up, save, load, destroy */
+    const char* names[2] = {"w", "s"};
+    int32_t slots[2] = {1, 2};
+    mi355x_wq_module *mod = NULL, *back = NULL;
+    mi355x_wq_packed_cfunc fn = NULL;
+    void* res = NULL;
+    char buf[512];
+    int64_t used = 0, n;
+    if (mi355x_wq_module_create("sym0", &spec, names, slots, 2, 0, &mod) != 0) return 9;
+    if (mi355x_wq_module_get_function(mod, "__init_sym0", &fn, &res) != 0 || fn == NULL || res != (void*)mod) return 10;
+    if (mi355x_wq_module_get_function(mod, "other", &fn, &res) != 0 || fn != NULL) return 11;
+    n = mi355x_wq_module_save_to_binary(mod, buf, (int64_t)sizeof(buf));
+    if (n <= 0 || n > (int64_t)sizeof(buf)) return 12;
+    if (mi355x_wq_module_load_from_binary(buf, n, &used, &back) != 0 || used != n) return 13;
+    if (strcmp(mi355x_wq_module_symbol(back), "sym0") != 0 || mi355x_wq_module_num_consts(back) != 2) return 14;
+    if (strcmp(mi355x_wq_module_json(back), mi355x_wq_module_json(mod)) != 0) return 15;
+    mi355x_wq_module_destroy(back);
+    if (mi355x_wq_module_create_from_json("sym1", mi355x_wq_module_json(mod), names, 2, &back) != 0) return 16;
+    if (strcmp(mi355x_wq_module_symbol(back), "sym1") != 0 || mi355x_wq_module_initialized(back) != 0) return 17;
+    mi355x_wq_module_destroy(back);
+    if (mi355x_wq_module_create_from_json("sym1", "{}", names, 2, &back) != -1 || back != NULL) return 18;
+    mi355x_wq_module_destroy(mod);
+  }
   puts("c client ok");
   return 0;
 }

@@ -1,0 +1,196 @@
+"""GPU tests of the subgraph runtime module: constants bound through `__init_<symbol>` (device
+tensors borrowed, host arrays copied), the call with the remaining arguments, the one-off tile-major
+conversion, and the export -> load -> run round trip
+(the shape of tests/python/relax/test_transform_codegen_pass.py:57-65)."""
+import numpy as np
+import pytest
+
+from oracle import c_oracle, wq_oracle as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+from relax_amd import lib, module as M, vm_harness  # noqa: E402
+from relax_amd.vm_harness import CallSpec, PackedError  # noqa: E402
+from tests.test_gpu_parity import _dev, assert_close  # noqa: E402
+
+
+def spec_for(bits, order, op=0, **kw):
+    slots = {r: i for i, r in enumerate(order)}
+    return CallSpec(op=op, bits=bits, group=0, zero_point=7 if bits == 4 else 0, arg_x=slots.get("x", 0),
+                    arg_wq=slots["wq"], arg_scales=slots["scales"], arg_out=slots["out"], num_args=len(order),
+                    arg_bias=slots.get("bias", -1), arg_residual=slots.get("residual", -1), **kw)
+
+
+def plain(bits, x, wq, s):
+    return vm_harness.call_dps("mi355x_q%df16_matmul" % bits, [x, wq, s], (x.shape[0], wq.shape[0]))
+
+
+@pytest.mark.parametrize("bits, m, n, k", [(4, 1, 4096, 4096), (4, 8, 200, 352), (4, 200, 136, 256), (8, 16, 5120, 5120),
+                                           (8, 3, 72, 384), (4, 64, 1024, 2048)])
+def test_bound_device_constants_give_the_plain_call_bit_for_bit(bits, m, n, k):
+    vm_harness.set_stream()
+    x, wq, s, g = O.make_case(31, m, n, k, bits)
+    dx, dw, ds = _dev(x), _dev(wq), _dev(s)
+    mod = M.SubgraphModule.create("f", spec_for(bits, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1])
+    init, run = mod.get_function("__init_f"), mod.get_function("f")
+    init(dw, ds)
+    assert mod.initialized
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    run(dx, y)
+    torch.cuda.synchronize()
+    assert torch.equal(y, plain(bits, dx, dw, ds))
+    assert_close(y.cpu().numpy(), c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16), (bits, m, n, k))
+    # init is once only: a second call with other tensors returns and changes nothing (json_runtime.h:91-98)
+    init(torch.zeros_like(dw), torch.zeros_like(ds))
+    y2 = torch.empty_like(y)
+    run(dx, y2)
+    assert torch.equal(y2, y)
+
+
+def test_host_constants_are_copied_to_the_device_at_init():
+    """After load_module the const loader holds host arrays (NDArrays are saved as CPU arrays)."""
+    vm_harness.set_stream()
+    for bits, m, n, k in [(4, 4, 512, 1024), (8, 1, 320, 640)]:
+        x, wq, s, g = O.make_case(32, m, n, k, bits)
+        mod = M.SubgraphModule.create("f", spec_for(bits, ("x", "wq", "scales", "out")), ["w", "s"], [1, 2])
+        mod.get_function("__init_f")(wq, s)  # numpy arrays
+        y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+        mod.get_function("f")(_dev(x), y)
+        torch.cuda.synchronize()
+        assert torch.equal(y, plain(bits, _dev(x), _dev(wq), _dev(s)))
+        mod.close()  # frees the module's device copies
+
+
+@pytest.mark.parametrize("bits, n, k", [(4, 4096, 4096), (8, 5120, 5120), (4, 200, 512)])
+def test_tile_major_conversion_at_init(bits, n, k):
+    """With the flag the module keeps its own tile-major copy and runs every call on it; results
+    equal mi355x_wq_matmul_tiled on weights tiled by hand, and the canonical path within tolerance."""
+    from relax_amd import wq_matmul, wq_tile_weights
+
+    vm_harness.set_stream()
+    group = 32 if bits == 4 else 128
+    for m in (1, 8, 48, 256):
+        x, wq, s, g = O.make_case(33, m, n, k, bits)
+        dx, dw, ds = _dev(x), _dev(wq), _dev(s)
+        mod = M.SubgraphModule.create("f", spec_for(bits, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1], M.TILE_WEIGHTS)
+        mod.get_function("__init_f")(wq if m == 8 else dw, s if m == 8 else ds)
+        y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+        mod.get_function("f")(dx, y)
+        torch.cuda.synchronize()
+        wt, st = wq_tile_weights(dw, ds, bits=bits, group=group)
+        assert torch.equal(y, wq_matmul(dx, wt, st, bits=bits, group=group, tiled_n=n))
+        assert_close(y.cpu().numpy(), c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16), (bits, m, n, k))
+
+
+def test_fused_operands_bias_constant_residual_argument():
+    vm_harness.set_stream()
+    bits, m, n, k = 4, 8, 1024, 1024
+    x, wq, s, g = O.make_case(34, m, n, k, bits)
+    rng = np.random.default_rng(5)
+    bias = rng.standard_normal(n).astype(np.float16)
+    res = rng.standard_normal((m, n)).astype(np.float16)
+    order = ("wq", "scales", "bias", "x", "residual", "out")
+    mod = M.SubgraphModule.create("g", spec_for(bits, order, activation=1), ["w", "s", "b"], [0, 1, 2], M.TILE_WEIGHTS)
+    mod.get_function("__init_g")(_dev(wq), _dev(s), bias)
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    mod.get_function("g")(_dev(x), _dev(res), y)
+    torch.cuda.synchronize()
+    want = c_oracle.wq_matmul_fused(x, wq, s, bits, g, bias=bias, activation="relu", residual=res)
+    assert_close(y.cpu().numpy(), want, "bias + relu + residual through the module")
+
+
+def test_dequantize_module():
+    vm_harness.set_stream()
+    x, wq, s, g = O.make_case(35, 1, 96, 256, 4)
+    mod = M.SubgraphModule.create("d", spec_for(4, ("wq", "scales", "out"), op=1), ["w", "s"], [0, 1])
+    mod.get_function("__init_d")(wq, s)
+    wd = torch.empty((96, 256), dtype=torch.float16, device="cuda")
+    mod.get_function("d")(wd)
+    torch.cuda.synchronize()
+    assert np.array_equal(wd.cpu().numpy().view(np.uint16), c_oracle.dequant(wq, s, 4, g, 8).view(np.uint16))
+
+
+def test_argument_errors():
+    vm_harness.set_stream()
+    x, wq, s, g = O.make_case(36, 2, 64, 128, 4)
+    mod = M.SubgraphModule.create("f", spec_for(4, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1])
+    with pytest.raises(PackedError, match="__init_f expects 2 constants, got 1"):
+        mod.get_function("__init_f")(_dev(wq))
+    assert not mod.initialized
+    y = torch.empty((2, 64), dtype=torch.float16, device="cuda")
+    with pytest.raises(PackedError, match="has not been initialized"):
+        mod.get_function("f")(_dev(x), y)
+    mod.get_function("__init_f")(_dev(wq), _dev(s))
+    with pytest.raises(PackedError, match="f expects 2 arguments .2 of the composite's 4 are bound constants., got 3"):
+        mod.get_function("f")(_dev(x), y, y)
+    with pytest.raises(PackedError, match="x has 64 columns but the weights have K=128"):
+        mod.get_function("f")(_dev(x[:, :64].copy()), y)
+    # constants of the wrong type are named when the call validates them
+    bad = M.SubgraphModule.create("f", spec_for(4, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1])
+    bad.get_function("__init_f")(_dev(s), _dev(s))
+    with pytest.raises(PackedError, match="wq.*expected dtype uint32"):
+        bad.get_function("f")(_dev(x), y)
+    tiled = M.SubgraphModule.create("f", spec_for(4, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1], M.TILE_WEIGHTS)
+    with pytest.raises(PackedError, match="wq must be uint32"):
+        tiled.get_function("__init_f")(_dev(s), _dev(s))
+    assert not tiled.initialized
+
+
+def test_export_load_run_round_trip(tmp_path):
+    """Two projections of a layer with bound weights: run, export, load the file in place of the
+    original, run again -- same bits (check_roundtrip, test_transform_codegen_pass.py:57-65)."""
+    vm_harness.set_stream()
+    cases = {"fused_q4_0": (4, 4096, 4096, ("wq", "scales", "x", "out"), M.TILE_WEIGHTS),
+             "fused_q8_1": (8, 1280, 5120, ("x", "wq", "scales", "out"), 0)}
+    consts, by_symbol, mods, inputs = {}, {}, [], {}
+    for i, (sym, (bits, n, k, order, flags)) in enumerate(cases.items()):
+        x, wq, s, g = O.make_case(40 + i, 8, n, k, bits)
+        names = [f"{sym}_const_0", f"{sym}_const_1"]
+        consts[names[0]], consts[names[1]] = _dev(wq), _dev(s)
+        by_symbol[sym] = names
+        slots = [order.index("wq"), order.index("scales")]
+        mods.append(M.SubgraphModule.create(sym, spec_for(bits, order), names, slots, flags))
+        inputs[sym] = (x, wq, s, g, bits)
+    exec0 = M.ConstLoader(consts, by_symbol, mods)
+    path = tmp_path / "exec.bin"
+    path.write_bytes(M.export_library(exec0))
+    exec1 = M.load_module(path.read_bytes())
+    assert all(isinstance(v, np.ndarray) for v in exec1.const_var_ndarray.values())  # host arrays after a load
+    for sym, (x, wq, s, g, bits) in inputs.items():
+        outs = []
+        for ex in (exec0, exec1):
+            y = torch.empty((8, wq.shape[0]), dtype=torch.float16, device="cuda")
+            ex.get_function(sym)(_dev(x), y)  # the first lookup runs __init_<symbol>
+            torch.cuda.synchronize()
+            outs.append(y)
+        assert torch.equal(outs[0], outs[1])
+        assert_close(outs[1].cpu().numpy(), c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16), sym)
+    assert all(exec1.initialized.values()) and all(m.initialized for m in exec1.imports)
+
+
+def test_module_call_captured_in_a_hip_graph():
+    """Calls allocate nothing, so a module call can sit in a captured decode step."""
+    vm_harness.set_stream()
+    x, wq, s, g = O.make_case(44, 1, 4096, 4096, 4)
+    mod = M.SubgraphModule.create("f", spec_for(4, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1], M.TILE_WEIGHTS)
+    mod.get_function("__init_f")(wq, s)
+    dx = _dev(x)
+    y = torch.empty((1, 4096), dtype=torch.float16, device="cuda")
+    run = mod.get_function("f")
+    run(dx, y)
+    torch.cuda.synchronize()
+    eager = y.clone()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        vm_harness.set_stream(stream)
+        with torch.cuda.graph(graph, stream=stream):
+            run(dx, y)
+    vm_harness.set_stream()
+    for _ in range(3):
+        y.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager)
