@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -35,7 +36,7 @@ struct mi355x_wq_module {
   std::vector<int32_t> const_args;
   int32_t flags = 0;
   std::mutex mutex;
-  bool initialized = false;
+  std::atomic<bool> initialized{false};  // set last in init, read without the lock by calls
   std::vector<BoundConst> bound;
   void* wq_tiled = nullptr;
   void* scales_tiled = nullptr;
@@ -293,8 +294,12 @@ bool bind_constants(mi355x_wq_module* m, const mi355x_dl_tensor* const* consts, 
   for (int i = 0; i < num_consts; ++i) {
     const mi355x_dl_tensor* t = consts[i];
     const char* name = m->const_names[i].c_str();
-    if (t == nullptr || t->data == nullptr || t->shape == nullptr || t->ndim < 1 || t->ndim > 2) {
+    if (t == nullptr || t->shape == nullptr || t->ndim < 1 || t->ndim > 2) {
       wq::set_error("constant '%s': expected a 1-d or 2-d tensor", name);
+      return false;
+    }
+    if (t->data == nullptr && t->shape[0] != 0 && t->shape[t->ndim - 1] != 0) {
+      wq::set_error("constant '%s': NULL data pointer", name);
       return false;
     }
     if (t->strides != nullptr) {
@@ -374,7 +379,18 @@ bool bind_constants(mi355x_wq_module* m, const mi355x_dl_tensor* const* consts, 
   const void* pw = static_cast<const char*>(tw.data) + tw.byte_offset;
   const void* ps = static_cast<const char*>(ts.data) + ts.byte_offset;
   if (mi355x_wq_tile_weights(&d, pw, ps, m->wq_tiled, m->scales_tiled, nullptr) != 0) return false;
-  return hip_ok(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+  if (!hip_ok(hipStreamSynchronize(nullptr), "hipStreamSynchronize")) return false;
+  // The module's own canonical copies (of host constants) are not read again: calls take N, K and the
+  // group from the headers and the data from the tile-major buffers, which have at least as many rows.
+  for (int i = 0; i < num_consts; ++i) {
+    BoundConst& b = m->bound[i];
+    const bool is_wq = m->const_args[i] == m->spec.arg_wq, is_scales = m->const_args[i] == m->spec.arg_scales;
+    if (b.owned == nullptr || !(is_wq || is_scales)) continue;
+    (void)hipFree(b.owned);
+    b.owned = nullptr;
+    b.tensor.data = is_wq ? m->wq_tiled : m->scales_tiled;
+  }
+  return true;
 }
 
 void set_int_return(void* ret, int64_t v) {
@@ -448,7 +464,7 @@ const char* mi355x_wq_module_const_name(const mi355x_wq_module* mod, int32_t i) 
   return mod && i >= 0 && i < (int32_t)mod->const_names.size() ? mod->const_names[i].c_str() : nullptr;
 }
 const char* mi355x_wq_module_json(const mi355x_wq_module* mod) { return mod ? mod->json.c_str() : nullptr; }
-int32_t mi355x_wq_module_initialized(const mi355x_wq_module* mod) { return mod && mod->initialized ? 1 : 0; }
+int32_t mi355x_wq_module_initialized(const mi355x_wq_module* mod) { return mod && mod->initialized.load() ? 1 : 0; }
 
 int mi355x_wq_module_get_function(mi355x_wq_module* mod, const char* name, mi355x_wq_packed_cfunc* func,
                                   void** resource_handle) {

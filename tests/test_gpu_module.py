@@ -194,3 +194,22 @@ def test_module_call_captured_in_a_hip_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y, eager)
+
+
+def test_empty_batch_and_empty_projection():
+    """M = 0 and N = 0 are legal shapes: nothing is launched, nothing fails (host constants, tile flag)."""
+    vm_harness.set_stream()
+    x, wq, s, g = O.make_case(45, 2, 64, 256, 4)
+    mod = M.SubgraphModule.create("f", spec_for(4, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1], M.TILE_WEIGHTS)
+    mod.get_function("__init_f")(wq, s)
+    mod.get_function("f")(torch.empty((0, 256), dtype=torch.float16, device="cuda"),
+                          torch.empty((0, 64), dtype=torch.float16, device="cuda"))
+    y = torch.empty((2, 64), dtype=torch.float16, device="cuda")
+    mod.get_function("f")(_dev(x), y)  # and the module still computes afterwards
+    torch.cuda.synchronize()
+    assert_close(y.cpu().numpy(), c_oracle.wq_matmul(x, wq, s, 4, g), "after an empty call")
+    none = M.SubgraphModule.create("e", spec_for(4, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1], M.TILE_WEIGHTS)
+    none.get_function("__init_e")(torch.empty((0, 32), dtype=torch.int32, device="cuda"),
+                                  torch.empty((0, 8), dtype=torch.float16, device="cuda"))
+    none.get_function("e")(_dev(x), torch.empty((2, 0), dtype=torch.float16, device="cuda"))
+    torch.cuda.synchronize()
