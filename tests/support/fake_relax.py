@@ -26,6 +26,20 @@ class Var(Expr):
         return self is other
 
 
+class Constant(Expr):
+    """A bound parameter: data plus shape; hashable by identity like the real node."""
+
+    def __init__(self, shape, data=None):
+        self.struct_info = StructInfo(shape)
+        self.data = data
+
+    def __hash__(self):
+        return id(self)
+
+    def __eq__(self, other):
+        return self is other
+
+
 class GlobalVar(Expr):
     def __init__(self, name):
         self.name_hint = name
@@ -70,22 +84,26 @@ class Function(Expr):
 def as_module():
     """A module object usable as `tvm` with a `relax` attribute."""
     relax = types.ModuleType("tvm.relax")
-    for cls in (Var, Call, Function, Tuple, GlobalVar, SeqExpr, BindingBlock, VarBinding):
+    for cls in (Var, Call, Function, Tuple, GlobalVar, SeqExpr, BindingBlock, VarBinding, Constant):
         setattr(relax, cls.__name__, cls)
     tvm = types.ModuleType("tvm")
     tvm.relax = relax
     return tvm, relax
 
 
-def quantized_linear(decode="decode_q4f16", m=4, n=48, k=128, tail=(), outer_order=None):
+def quantized_linear(decode="decode_q4f16", m=4, n=48, k=128, tail=(), outer_order=None, bound=()):
     """The annotated function FuseOpsByPattern(annotate_codegen=True) produces for
     decode -> permute_dims -> matmul -> astype followed by `tail`, a sequence of
     ("add", shape) / ("relu",) steps.  Composite parameters are ordered by first use:
-    (wq, scales, x, <tail operands in order>).  `outer_order` permutes the outer parameters."""
+    (wq, scales, x, <tail operands in order>).  `outer_order` permutes the outer parameters.
+    `bound` names operands ("wq", "scales", "operand<i>") that BindParams turned into constants: they sit
+    inside the composite as Constant nodes and are no parameters."""
     per = 8 if "q4" in decode else 4
     group = 32 if "q4" in decode else 128
-    wq, s, x = Var("wq", [n, k // per]), Var("s", [n, k // group]), Var("x", [m, k])
-    params = [wq, s, x]
+    wq = Constant([n, k // per]) if "wq" in bound else Var("wq", [n, k // per])
+    s = Constant([n, k // group]) if "scales" in bound else Var("s", [n, k // group])
+    x = Var("x", [m, k])
+    params = [p for p in (wq, s, x) if isinstance(p, Var)]
     binds = []
     wd = Var("wd", [n, k])
     binds.append(VarBinding(wd, Call(Op("relax.call_tir"), [GlobalVar(decode), Tuple([wq, s])])))
@@ -98,8 +116,9 @@ def quantized_linear(decode="decode_q4f16", m=4, n=48, k=128, tail=(), outer_ord
     for i, step in enumerate(tail):
         nxt = Var(f"t{i}", [m, n])
         if step[0] == "add":
-            operand = Var(f"operand{i}", step[1])
-            params.append(operand)
+            operand = Constant(step[1]) if f"operand{i}" in bound else Var(f"operand{i}", step[1])
+            if isinstance(operand, Var):
+                params.append(operand)
             args = [cur, operand] if len(step) < 3 or not step[2] else [operand, cur]
             binds.append(VarBinding(nxt, Call(Op("relax.add"), args)))
         else:

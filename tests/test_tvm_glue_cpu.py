@@ -183,3 +183,74 @@ def test_generated_fused_entry_forwards_all_roles(tmp_path):
         trampoline_source([("f", CallSpec(0, 4, 0, 7, 0, 1, 2, 3, -1, -1, 9))])
     with pytest.raises(ValueError, match="no fused operands"):
         trampoline_source([("f", CallSpec(1, 4, 0, 7, 0, 0, 1, 3, 2, -1, 0))])
+
+
+def constants_of(func):
+    """What RunCodegen's PostOrderVisit collects: every Constant of the function body, named
+    <symbol>_<codegen>_const_<i> in visiting order (src/relax/transform/run_codegen.cc:120-129)."""
+    from tests.support import fake_relax
+
+    found = []
+
+    def walk(e):
+        if isinstance(e, fake_relax.Constant) and e not in found:
+            found.append(e)
+        for child in getattr(e, "args", []) + getattr(e, "fields", []):
+            walk(child)
+        if isinstance(e, fake_relax.Function):
+            walk(e.body)
+        if isinstance(e, fake_relax.SeqExpr):
+            for block in e.blocks:
+                for b in block.bindings:
+                    walk(b.value)
+            walk(e.body)
+
+    walk(func)
+    return {c: f"fused_mi355x_mi355x_const_{i}" for i, c in enumerate(found)}
+
+
+def test_bound_weights_give_a_module_plan(fake_tvm):
+    from relax_amd import module as M
+    from relax_amd.tvm_glue.codegen import ACT_RELU, MODULE_TILE_WEIGHTS, module_plan, spec_from_function
+    from relax_amd.vm_harness import CallSpec as CSpec
+
+    n = 48
+    f = fake_tvm.quantized_linear(bound=("wq", "scales"))
+    assert [p.name_hint for p in f.params] == ["x_outer"]
+    with pytest.raises(ValueError, match="use module_plan"):
+        spec_from_function(f)
+    names = constants_of(f)
+    plan = module_plan(f, names)
+    s = plan.spec
+    assert plan.symbol == "fused_mi355x" and plan.flags == MODULE_TILE_WEIGHTS
+    assert plan.const_names == ("fused_mi355x_mi355x_const_0", "fused_mi355x_mi355x_const_1") and plan.const_args == (0, 1)
+    assert (s.arg_wq, s.arg_scales, s.arg_x, s.arg_out, s.num_args) == (0, 1, 2, 3, 4)  # the VM calls <symbol>(x, out)
+    # bias bound as well, residual a parameter, relu in between
+    f = fake_tvm.quantized_linear("decode_q8f16", tail=[("add", [n]), ("relu",), ("add", [4, n])],
+                                  bound=("wq", "scales", "operand0"))
+    plan = module_plan(f, constants_of(f))
+    s = plan.spec
+    assert plan.const_args == (0, 1, 2) and len(plan.const_names) == 3
+    assert (s.bits, s.arg_wq, s.arg_scales, s.arg_bias, s.arg_x, s.arg_residual, s.arg_out, s.activation) == \
+        (8, 0, 1, 2, 3, 4, 5, ACT_RELU)
+    # only the weights bound, scales a parameter: no tile-major conversion (it needs both)
+    f = fake_tvm.quantized_linear(bound=("wq",))
+    plan = module_plan(f, constants_of(f))
+    assert plan.flags == 0 and plan.const_args == (0,) and (plan.spec.arg_wq, plan.spec.arg_scales, plan.spec.arg_x) == (0, 1, 2)
+    # the plan is what the library's module accepts, and the module reports the same constants
+    f = fake_tvm.quantized_linear(tail=[("add", [n])], bound=("wq", "scales", "operand0"))
+    plan = module_plan(f, constants_of(f))
+    s = plan.spec
+    mod = M.SubgraphModule.create(plan.symbol, CSpec(op=s.op, bits=s.bits, group=s.group, zero_point=s.zero_point, arg_x=s.arg_x,
+                                                     arg_wq=s.arg_wq, arg_scales=s.arg_scales, arg_out=s.arg_out,
+                                                     num_args=s.num_args, arg_bias=s.arg_bias, arg_residual=s.arg_residual,
+                                                     activation=s.activation),
+                                  list(plan.const_names), list(plan.const_args), plan.flags)
+    assert mod.const_names == list(plan.const_names) and not mod.initialized
+    # a constant RunCodegen did not name
+    with pytest.raises(ValueError, match="has no name in constant_names"):
+        module_plan(f, {})
+    # an activation operand can not be a constant
+    f = fake_tvm.quantized_linear(tail=[("add", [4, n])], bound=("wq", "scales", "operand0"))
+    with pytest.raises(ValueError, match="residual of the composite is a constant"):
+        module_plan(f, constants_of(f))
