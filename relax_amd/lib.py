@@ -123,7 +123,8 @@ def load() -> C.CDLL:
 
 
 def last_error() -> str:
-    return load().mi355x_wq_last_error().decode()
+    # a message may quote bytes of a damaged module file, which need not be UTF-8
+    return load().mi355x_wq_last_error().decode(errors="backslashreplace")
 
 
 def make_desc(bits: int, group: int, n: int, k: int, zero_point: int | None = None) -> WqDesc:

@@ -163,3 +163,27 @@ def test_const_loader_and_module_blob_round_trip():
     unknown[24:36] = b"const_loadex"
     with pytest.raises(ValueError, match="a loader of that name is not registered"):
         M.load_module(bytes(unknown))
+
+
+def test_randomly_damaged_binaries_never_crash_the_loader():
+    """4000 single- and multi-byte corruptions of a good module: each either loads as a module that
+    passes the creation checks or is refused with a message; none reads outside the buffer."""
+    m = M.SubgraphModule.create("fused_q4_0", spec_matmul(order=("wq", "scales", "bias", "x", "out")), ["w", "s", "b"], [0, 1, 2],
+                                M.TILE_WEIGHTS)
+    good = bytearray(m.save_to_binary())
+    rng = np.random.default_rng(7)
+    loaded = refused = 0
+    for _ in range(4000):
+        bad = bytearray(good)
+        for _ in range(int(rng.integers(1, 4))):
+            bad[int(rng.integers(0, len(bad)))] = int(rng.integers(0, 256))
+        if rng.integers(0, 4) == 0:
+            bad = bad[:int(rng.integers(0, len(bad)))]
+        try:
+            back, used = M.SubgraphModule.load_from_binary(bytes(bad))
+            assert 0 < used <= len(bad) and back.json.startswith('{"version": 1')
+            loaded += 1
+        except lib.WqError as e:
+            assert str(e)
+            refused += 1
+    assert loaded + refused == 4000 and refused > 1000
