@@ -109,15 +109,34 @@ __device__ __forceinline__ void q4_word_natural(uint32_t w, half2_t s2, const Q4
   }
 }
 
-// int8: byte b (two's complement) xor 0x80 = b + 128 as an unsigned byte, so
-// 0x6400 | (byte ^ 0x80) is exactly 1152 + b.  One word -> 2 half2, natural order.
-// 8 VALU ops per word.
+// int8 -> float16 in one instruction per weight: v_cvt_f16_i16 with a sub-dword source select
+// (byte BYTE of the word, sign-extended) writing the low half (upper half zeroed) or the high half
+// (low half kept) of the destination.  Exact for every int8 value.
+template <int BYTE>
+__device__ __forceinline__ uint32_t cvt_i8_lo(uint32_t w) {
+  static_assert(BYTE >= 0 && BYTE < 4, "byte of a 32-bit word");
+  uint32_t d;
+  if constexpr (BYTE == 0) asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(d) : "v"(w));
+  else if constexpr (BYTE == 1) asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(d) : "v"(w));
+  else if constexpr (BYTE == 2) asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(d) : "v"(w));
+  else asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(d) : "v"(w));
+  return d;
+}
+template <int BYTE>
+__device__ __forceinline__ uint32_t cvt_i8_hi(uint32_t d, uint32_t w) {
+  static_assert(BYTE >= 0 && BYTE < 4, "byte of a 32-bit word");
+  if constexpr (BYTE == 0) asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_0" : "+v"(d) : "v"(w));
+  else if constexpr (BYTE == 1) asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_1" : "+v"(d) : "v"(w));
+  else if constexpr (BYTE == 2) asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_2" : "+v"(d) : "v"(w));
+  else asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3" : "+v"(d) : "v"(w));
+  return d;
+}
+
+// int8: one word -> 2 half2, natural order: two conversions and the scale multiply per pair.
+// 6 VALU ops per word.
 __device__ __forceinline__ void q8_word_natural(uint32_t w, half2_t s2, half2_t out[2]) {
-  const half2_t off = half2_t{(half_t)1152.0f, (half_t)1152.0f};
-  uint32_t t0 = __builtin_amdgcn_perm(0u, w, 0x0c010c00u) ^ 0x64806480u;
-  uint32_t t1 = __builtin_amdgcn_perm(0u, w, 0x0c030c02u) ^ 0x64806480u;
-  out[0] = (as_h2(t0) - off) * s2;
-  out[1] = (as_h2(t1) - off) * s2;
+  out[0] = as_h2(cvt_i8_hi<1>(cvt_i8_lo<0>(w), w)) * s2;
+  out[1] = as_h2(cvt_i8_hi<3>(cvt_i8_lo<2>(w), w)) * s2;
 }
 
 __device__ __forceinline__ half8_t pack_h8(half2_t a, half2_t b, half2_t c, half2_t d) {

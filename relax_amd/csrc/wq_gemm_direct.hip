@@ -243,7 +243,7 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   uint32_t s_step[2][2];  // [step parity][column tile]
 
   // The conversion of one pair of weights is a chain of four dependent VALU ops (byte
-  // permute, and-or, fma, scale multiply).  The chain is software-pipelined over four
+  // permute, and-or, fma, scale multiply; int8: convert low, convert high, scale multiply -- three).  The chain is software-pipelined over four
   // MFMA slots -- every slot advances four different pairs by one stage -- so no slot
   // contains dependent instructions.  Pair g (counted from the start of the K step)
   // belongs to B fragment g/4 = slice (g/8), column tile (g/4)%2, position g%4.
@@ -252,17 +252,21 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     if constexpr (BITS == 4) {
       return __builtin_amdgcn_perm(0u, b.w[j][0][kk], 0x0c000c00u | (uint32_t)pp | ((uint32_t)pp << 16));
     } else {
-      return __builtin_amdgcn_perm(0u, b.w[j][kk >> 1][(kk & 1) * 2 + (pp >> 1)],
-                                   (pp & 1) ? 0x0c030c02u : 0x0c010c00u);
+      // int8: the first weight of the pair, converted into the low half (upper half zero)
+      return cvt_i8_lo<(pp & 1) * 2>(b.w[j][kk >> 1][(kk & 1) * 2 + (pp >> 1)]);
     }
   };
-  auto stage_bits = [&](uint32_t v) -> uint32_t {
+  // (int8: the second weight of pair g of `b`, converted into the high half of v -- the chain reads the
+  // packed word in two consecutive slots, so a register set is reloaded no earlier than the slot after
+  // its last pair entered, and a slot converts before it loads)
+  auto stage_bits = [&](uint32_t v, const RawB<BITS>& b, auto gc) -> uint32_t {
+    constexpr int g = decltype(gc)::value, kk = (g / 8) & 3, j = (g / 4) & 1, pp = g & 3;
     if constexpr (BITS == 4) return and_or(v, 0x00F0000Fu, qc.magic);
-    else return v ^ 0x64806480u;
+    else return cvt_i8_hi<(pp & 1) * 2 + 1>(v, b.w[j][kk >> 1][(kk & 1) * 2 + (pp >> 1)]);
   };
   auto stage_center = [&](uint32_t v) -> half2_t {
     if constexpr (BITS == 4) return __builtin_elementwise_fma(as_h2(v), qc.mix_mul, -qc.mix_sub);
-    else return as_h2(v) - half2_t{(half_t)1152.0f, (half_t)1152.0f};
+    else return as_h2(v);  // the conversion is complete: this stage is empty for int8
   };
   auto stage_scale = [&](int parity, half2_t v, auto gc) -> uint32_t {
     constexpr int g = decltype(gc)::value, j = (g / 4) & 1;
@@ -339,12 +343,14 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   // three, two and one stage in
   static_for_d<0, PPS * LEAD>([&](auto gc) {
     constexpr int g = decltype(gc)::value;
-    fbq[g / 4][g & 3] = stage_scale(0, stage_center(stage_bits(stage_perm(rb[0], gc))), gc);
+    fbq[g / 4][g & 3] = stage_scale(0, stage_center(stage_bits(stage_perm(rb[0], gc), rb[0], gc)), gc);
   });
   static_for_d<0, PPS>([&](auto pc) {
     constexpr int pp = decltype(pc)::value;
-    t_center[pp] = stage_center(stage_bits(stage_perm(rb[0], std::integral_constant<int, PPS * LEAD + pp>{})));
-    t_bits[pp] = stage_bits(stage_perm(rb[0], std::integral_constant<int, PPS * (LEAD + 1) + pp>{}));
+    constexpr std::integral_constant<int, PPS * LEAD + pp> g1{};
+    constexpr std::integral_constant<int, PPS * (LEAD + 1) + pp> g2{};
+    t_center[pp] = stage_center(stage_bits(stage_perm(rb[0], g1), rb[0], g1));
+    t_bits[pp] = stage_bits(stage_perm(rb[0], g2), rb[0], g2);
     t_perm[pp] = stage_perm(rb[0], std::integral_constant<int, PPS * (LEAD + 2) + pp>{});
   });
 
@@ -377,11 +383,12 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
       // slots behind them (pairs 32.. belong to the next step's packed weights)
       static_for_d<0, PPS>([&](auto pc) {
         constexpr int pp = decltype(pc)::value;
-        constexpr int gd = PPS * (s + LEAD) + pp, ga = gd + 3 * PPS;
+        constexpr int gd = PPS * (s + LEAD) + pp, ga = gd + 3 * PPS, gb = ga - PPS;
         fbq[(gd / 4) & 3][gd & 3] = stage_scale(gd < 32 ? (P & 1) : ((P + 1) & 1), t_center[pp],
                                                 std::integral_constant<int, gd & 31>{});
         t_center[pp] = stage_center(t_bits[pp]);
-        t_bits[pp] = stage_bits(t_perm[pp]);
+        t_bits[pp] = gb < 32 ? stage_bits(t_perm[pp], bcur, std::integral_constant<int, gb & 31>{})
+                             : stage_bits(t_perm[pp], bnxt, std::integral_constant<int, gb & 31>{});
         t_perm[pp] = ga < 32 ? stage_perm(bcur, std::integral_constant<int, ga & 31>{})
                              : stage_perm(bnxt, std::integral_constant<int, ga & 31>{});
       });
