@@ -30,10 +30,37 @@ DECODE_BATCHES = (1, 8)
 PREFILL_M = 2048
 HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
-# HBM bytes per GEMV launch of this workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (mean per dispatch, scaled by a 256 MiB copy: FETCH_SIZE reads half the true KiB, WRITE_SIZE
-# the true KiB); measurement and commands in profiles/gemv_decode_llama7b.md.
-GEMV_HBM_TRAFFIC_PER_LAUNCH = int((14170.0 * 2.0 + 93.4 * 1.0) * 1024)
+GEMV_PROFILE = os.path.join(ROOT, "profiles", "gemv_decode_llama7b.md")
+GEMV_KERNEL_SOURCES = ("relax_amd/csrc/wq_gemv.hip", "relax_amd/csrc/wq_device.h")
+
+
+def kernel_sources_digest() -> str:
+    """sha256 over the decode kernel's source files (what a counter summary is valid for)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for rel in GEMV_KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def measured_traffic():
+    """HBM bytes per GEMV launch of this workload, from the tracked rocprofv3 counter summary
+    (FETCH_SIZE / WRITE_SIZE per dispatch, scaled by the copy of known size that runs first).
+    The summary names the digest of the kernel sources it was taken on; when the sources have
+    changed since, the figure is stale and None is returned."""
+    import re
+
+    try:
+        text = open(GEMV_PROFILE).read()
+    except OSError:
+        return None
+    traffic = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", text, re.M)
+    digest = re.search(r"^kernel_sources_sha256:\s*([0-9a-f]{64})", text, re.M)
+    if not traffic or not digest or digest.group(1) != kernel_sources_digest():
+        return None
+    return int(traffic.group(1))
 
 
 def algorithmic_bytes(bits: int, group: int, m: int, n: int, k: int) -> int:
@@ -144,136 +171,6 @@ def config_table(torch, dev, args) -> int:
     return 0
 
 
-def audit_dispatch(torch, dev, tiled: bool = False) -> int:
-    """Default kernel selection against every explicit (family, variant) for M <= 64: the tool the
-    selection rules were checked with.  One HIP graph over 2-6 distinct weight sets per timing.
-    `tiled`: the same on weights in the tile-major layout (their own selection rules)."""
-    import relax_amd
-    from relax_amd import lib
-
-    def graph_us(fn, launches):
-        st = torch.cuda.Stream()
-        with torch.cuda.stream(st):
-            fn()
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=st):
-                fn()
-        torch.cuda.synchronize()
-        ts = []
-        for _ in range(3):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            g.replay()
-            e1.record()
-            torch.cuda.synchronize()
-            ts.append(e0.elapsed_time(e1) * 1e3 / launches)
-        return sorted(ts)[1]
-
-    shapes = [(2048, 4096), (4096, 2048), (4096, 4096), (5120, 5120), (6144, 4096), (8192, 4096), (8192, 8192),
-              (11008, 4096), (16384, 4096), (32000, 4096), (4096, 16384)]
-    cands = [(lib.KERNEL_GEMV, v) for v in ((15, 25) if tiled else (14, 15, 24, 25))] \
-        + [(lib.KERNEL_SKINNY, v) for v in ((1, 2, 5, 7, 9, 11) if tiled else (1, 2, 5, 7, 9))] + [(lib.KERNEL_GEMM, 25)]
-    names = {lib.KERNEL_GEMV: "gemv", lib.KERNEL_SKINNY: "skinny", lib.KERNEL_GEMM: "gemm"}
-    behind = 0
-    for bits, group in ((4, 32), (8, 128)):
-        for n, k in shapes:
-            nsets = max(2, min(6, (400 << 20) // (n * k * bits // 8)))
-            sets = [(torch.randint(-2**31, 2**31 - 1, (n, k * bits // 32), dtype=torch.int32, device=dev),
-                     (torch.rand((n, k // group), device=dev) * 0.015 + 0.005).to(torch.float16)) for _ in range(nsets)]
-            if tiled:
-                sets = [relax_amd.wq_tile_weights(wq, sc, bits, group) for wq, sc in sets]
-            for m in (1, 4, 8, 16, 24, 32, 48, 64):
-                x = torch.randn((m, k), device=dev).to(torch.float16)
-                y = torch.empty((m, n), dtype=torch.float16, device=dev)
-
-                def run(fam, var):
-                    def f():
-                        for wq, sc in sets:
-                            relax_amd.wq_matmul(x, wq, sc, bits, group, out=y, kernel=fam, variant=var,
-                                                tiled_n=n if tiled else None)
-                    return graph_us(f, nsets)
-
-                run(0, 0)  # first use of a kernel on this device: code load, LDS attribute
-                base = run(0, 0)
-                best, best_name = base, "default"
-                for fam, var in cands:
-                    if fam == lib.KERNEL_GEMV and m > 16:
-                        continue
-                    try:
-                        t = run(fam, var)
-                    except lib.WqError:
-                        continue
-                    if t < best:
-                        best, best_name = t, "%s %d" % (names[fam], var)
-                base = min(base, run(0, 0))  # again after the candidates: clocks and caches have settled
-                line = {"case": "q%df16 M=%d N=%d K=%d%s" % (bits, m, n, k, " tile-major" if tiled else ""), "default_us": round(base, 2),
-                        "best_us": round(best, 2), "best": best_name, "behind": round(base / best - 1.0, 3)}
-                if base > 1.08 * best:
-                    behind += 1
-                    print(json.dumps(line), flush=True)
-            del sets
-    print(json.dumps({"layout": "tile-major" if tiled else "canonical", "cases": 2 * len(shapes) * 8,
-                      "more_than_8_percent_behind": behind}), flush=True)
-    return 0
-
-
-def probe_mfma(torch, dev) -> int:
-    """A loop of 32x32x16 float16 MFMAs whose operands never leave registers, one wavefront per
-    SIMD, about 10 - 15 ms per launch: the rate depends on the operand values only."""
-    import ctypes
-
-    so = os.path.join(ROOT, "relax_amd", "csrc", "libmi355x_probe.so")
-    if not os.path.exists(so):
-        raise ImportError(f"{so} is missing: build it with `make -C relax_amd/csrc all`")
-    fn = ctypes.CDLL(so).mi355x_probe_mfma_f16
-    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
-    blocks, iters = 256, 40000
-    shape = (blocks, 8, 256 * 8)  # [:, :4] A fragments, [:, 4:] B fragments
-    out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
-    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
-
-    def q4_like():
-        t = torch.randn(shape, device=dev)
-        w = torch.randint(0, 16, (blocks, 4, 256 * 8), device=dev).float() - 7.0
-        sc = (torch.rand((blocks, 4, 256 * 8), device=dev) * 0.015 + 0.005).half().float()
-        t[:, 4:] = w * sc
-        return t
-
-    cases = [
-        ("zeros", lambda: torch.zeros(shape, device=dev)),
-        ("ones", lambda: torch.ones(shape, device=dev)),
-        ("A ~ N(0,1), B = (u{0..15} - 7) * 2^-7", lambda: torch.cat(
-            [torch.randn((blocks, 4, 256 * 8), device=dev),
-             (torch.randint(0, 16, (blocks, 4, 256 * 8), device=dev).float() - 7.0) / 128.0], dim=1)),
-        ("A ~ N(0,1), B = (u{0..15} - 7) * s, s ~ U(0.005, 0.02): the benchmark's weights", q4_like),
-        ("A, B ~ N(0,1)", lambda: torch.randn(shape, device=dev)),
-    ]
-    flops = blocks * 4 * iters * 16 * 32768.0
-    for name, make in cases:
-        ops = make().to(torch.float16).contiguous()
-        rc = fn(ops.data_ptr(), out.data_ptr(), blocks, iters // 10, clocks.data_ptr(), None)  # warm-up
-        torch.cuda.synchronize()
-        best = None
-        for _ in range(3):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            rc |= fn(ops.data_ptr(), out.data_ptr(), blocks, iters, clocks.data_ptr(), None)
-            e1.record()
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1)
-            if best is None or ms < best:
-                best, (cyc, ref) = ms, clocks.tolist()
-        if rc != 0:
-            raise RuntimeError(f"probe launch failed with HIP error {rc}")
-        print(json.dumps({"probe": "mfma_f32_32x32x16_f16, operands in registers", "operands": name,
-                          "ms": round(best, 2), "tflops": round(flops / best / 1e9, 0),
-                          "frac_of_peak": round(flops / best / 1e9 / MFMA_F16_PEAK_TFLOPS, 3),
-                          "cycles_per_mfma": round(cyc / (iters * 16.0), 2),
-                          "shader_clock_ghz": round(cyc / (ref * 10.0), 3)}), flush=True)
-    return 0
-
-
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -284,25 +181,11 @@ def main() -> int:
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--no-epilogue", action="store_true", help="skip the fused-residual leg")
     ap.add_argument("--no-ksplit", action="store_true", help="skip the caller-workspace (K split) leg")
-    ap.add_argument("--no-read-floor", action="store_true", help="skip the read-only floor measurement")
     ap.add_argument("--no-tiled", action="store_true", help="skip the tile-major-weights decode leg")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run a plain 256 MiB device copy three times (a kernel of known HBM "
-                         "traffic, used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--configs", action="store_true",
                     help="instead of the benchmark: time every shape of the decode, prefill and q8f16 "
                          "configurations on its own (weights rotated through more than 512 MB, one HIP "
                          "graph per case) and print one line per case")
-    ap.add_argument("--audit-dispatch", action="store_true",
-                    help="instead of the benchmark: for 11 shapes x 8 row counts (1..64) per quantization, time the "
-                         "library's default kernel choice against every explicit variant of every family and print "
-                         "the cases where the default is more than 8 %% behind the best")
-    ap.add_argument("--audit-tile-major", action="store_true",
-                    help="the same audit on weights in the tile-major layout")
-    ap.add_argument("--probe-mfma", action="store_true",
-                    help="instead of the benchmark: time a register-resident float16 MFMA loop on operands "
-                         "of several distributions (what the matrix pipes sustain as a function of the data "
-                         "alone) and print one line per distribution")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the hot path is a single-GPU kernel and this build has no "
@@ -319,20 +202,18 @@ def main() -> int:
     torch.cuda.set_device(dev)
     torch.manual_seed(0)
 
-    if args.probe_mfma:
-        return probe_mfma(torch, dev)
     if args.configs:
         return config_table(torch, dev, args)
-    if args.audit_dispatch or args.audit_tile_major:
-        return audit_dispatch(torch, dev, tiled=args.audit_tile_major)
 
-    if args.calibrate_copy:
-        src = torch.ones(64 * 1024 * 1024, dtype=torch.int32, device=dev)  # 256 MiB read + 256 MiB written
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+    # A kernel of known HBM traffic ahead of everything else (256 MiB read, 256 MiB written, three
+    # times, outside every timing): under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its counts give
+    # the factor that turns the counters of the kernels below into bytes.
+    src = torch.ones(64 * 1024 * 1024, dtype=torch.int32, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
 
     # ---- synthetic weights: every bit pattern is a valid packed int4 row ------------------
     layers = []
@@ -404,7 +285,7 @@ def main() -> int:
                      "bytes_per_launch": bytes_per_step // launches_per_step,
                      "avg_launch_us": round(avg_launch_us, 3)},
     }
-    result["roofline"]["traffic"] = GEMV_HBM_TRAFFIC_PER_LAUNCH
+    result["roofline"]["traffic"] = measured_traffic()
 
     # ---- the same decode step on tile-major weights (the one-off layout transform applied at load) ----
     if not args.no_tiled:
@@ -553,58 +434,6 @@ def main() -> int:
             "us_per_projection_separate_add": round(times[False] * 1e3 / pairs, 3),
             "us_per_projection_fused": round(times[True] * 1e3 / pairs, 3),
             "speedup": round(times[False] / times[True], 3)}
-
-    if not args.no_read_floor:
-        # Context for the HBM fraction: a kernel that only reads -- the same packed weights and scales,
-        # one launch per matrix, the same number of launches in one HIP graph -- i.e. what launch, ramp
-        # and tail leave of the 8 TB/s for these byte counts with no arithmetic, staging or reduction.
-        import ctypes
-
-        so = os.path.join(ROOT, "relax_amd", "csrc", "libmi355x_probe.so")
-        if not os.path.exists(so):
-            raise ImportError(f"{so} is missing: build it with `make -C relax_amd/csrc all`")
-        rd = ctypes.CDLL(so).mi355x_probe_stream_read
-        rd.argtypes = [ctypes.c_void_p, ctypes.c_longlong, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_void_p,
-                       ctypes.c_int, ctypes.c_void_p]
-        best = None
-        for blocks in (256, 512, 1024):
-            sink = torch.empty(blocks * 512, dtype=torch.int32, device=dev)
-
-            def read_pass():
-                sp = int(stream.cuda_stream)
-                for _ in DECODE_BATCHES:
-                    for mats in layers:
-                        for wq, s, n, k in mats:
-                            rc = rd(wq.data_ptr(), wq.numel() * 4, s.data_ptr(), s.numel() * 2, sink.data_ptr(), blocks, sp)
-                            if rc != 0:
-                                raise RuntimeError("stream-read probe: HIP error %d" % rc)
-
-            with torch.cuda.stream(stream):
-                read_pass()
-                torch.cuda.synchronize()
-                gr = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gr, stream=stream):
-                    read_pass()
-                gr.replay()
-                torch.cuda.synchronize()
-                r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                r0.record(stream)
-                for _ in range(args.steps):
-                    gr.replay()
-                r1.record(stream)
-                torch.cuda.synchronize()
-            rms = r0.elapsed_time(r1) / args.steps
-            if best is None or rms < best[0]:
-                best = (rms, blocks)
-        weight_bytes = len(DECODE_BATCHES) * sum(wq.numel() * 4 + s.numel() * 2 for mats in layers for wq, s, _, _ in mats)
-        result["read_only_floor"] = {
-            "value": round(weight_bytes / (best[0] * 1e-3) / 1e9, 1), "unit": "GB/s",
-            "frac_of_peak": round(weight_bytes / (best[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 3),
-            "ms_per_step": round(best[0], 4), "workgroups": best[1],
-            "workload": "a kernel that only reads the same weights and scales, one launch per matrix, the "
-                        "same %d launches in one HIP graph (best of 256 / 512 / 1024 workgroups of 512 threads)"
-                        % (len(DECODE_BATCHES) * len(LLAMA7B) * args.layers),
-            "decode_vs_floor": round(best[0] / ms_per_step, 3)}
 
     if not args.no_ksplit:
         # the down projection (4096 x 11008) of every layer at 8 rows: the one case of this step where a

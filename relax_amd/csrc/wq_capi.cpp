@@ -1,6 +1,7 @@
 // C ABI of the library (include/mi355x_wq.h): argument validation, kernel-family
 // dispatch and the thread-local error string.  No kernel is launched unless every
 // shape, size and alignment assumption of the kernels has been checked here.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -28,32 +29,32 @@ int current_device_slot() {
   return dev >= 0 && dev < kMaxDevices ? dev : kMaxDevices - 1;
 }
 
-bool ensure_dynamic_lds(const void* kernel, int bytes, bool* done) {
+bool ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<bool>* done) {
   const int slot = current_device_slot();
-  if (done[slot]) return true;  // a race only repeats the same idempotent call
+  if (done[slot].load(std::memory_order_acquire)) return true;  // a race only repeats the same idempotent call
   const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
   if (e != hipSuccess) {
     (void)hipGetLastError();
     set_error("cannot reserve %d bytes of LDS for a kernel on this device: %s", bytes, hipGetErrorString(e));
     return false;
   }
-  done[slot] = true;
+  done[slot].store(true, std::memory_order_release);
   return true;
 }
 
 int cu_count() {
-  static int cached[kMaxDevices] = {0};  // same value for every caller of a device
+  static std::atomic<int> cached[kMaxDevices];  // same value for every caller of a device
   const int slot = current_device_slot();
-  if (cached[slot] == 0) {
+  if (cached[slot].load(std::memory_order_relaxed) == 0) {
     int dev = 0;
     hipDeviceProp_t prop;
     if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
         prop.multiProcessorCount > 0)
-      cached[slot] = prop.multiProcessorCount;
+      cached[slot].store(prop.multiProcessorCount, std::memory_order_relaxed);
     else
       return 256;
   }
-  return cached[slot];
+  return cached[slot].load(std::memory_order_relaxed);
 }
 
 namespace {
@@ -311,7 +312,7 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
     return -1;
   if (ep != nullptr && ep->bias != nullptr && !check_ptr(ep->bias, "bias", 2)) return -1;
   if (ep != nullptr && ep->residual != nullptr && !check_ptr(ep->residual, "residual", 2)) return -1;
-  const int family = kernel & 0xFF, variant = (kernel >> 8) & 0xFF;
+  const int family = kernel & 0xFF, variant = (kernel >> 8) & 0xFFFF;
   Problem p{x, wq_, scales, y, m, desc->n, desc->k, desc->bits, desc->group, desc->zero_point,
             static_cast<hipStream_t>(stream)};
   if (ep != nullptr) {

@@ -11,6 +11,7 @@
 //
 // LDS rows are padded by 16 bytes (row stride 144 B) so that the 16-byte operand
 // reads of 8 consecutive lanes cover all banks once.
+#include <atomic>
 #include "wq_device.h"
 #include "wq_internal.h"
 
@@ -199,7 +200,7 @@ bool launch_one(const Problem& p, int group_shift) {
   const int tiles_n = (int)((p.n + BN - 1) / BN);
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * (64 + 8) * sizeof(half_t);
-  static bool lds_ok[kMaxDevices] = {false};
+  static std::atomic<bool> lds_ok[kMaxDevices];
   if (!ensure_dynamic_lds((const void*)wq_gemm_kernel<BITS, BM, BN, WM, WN>, (int)lds_bytes, lds_ok)) return false;
   hipLaunchKernelGGL((wq_gemm_kernel<BITS, BM, BN, WM, WN>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,

@@ -50,6 +50,7 @@
 // Shape requirements (checked by the launcher): K a multiple of 256 (at least 512 for K
 // groups), group 32 (int4) or 128 (int8), operands < 1 GiB; other shapes use the other GEMM
 // kernels.
+#include <atomic>
 #include <type_traits>
 
 #include "wq_device.h"
@@ -542,7 +543,7 @@ bool launch_direct(const Problem& p, int group_shift, int tile_n0 = 0, int tile_
   constexpr size_t stages = (size_t)GROUPS * 4 * BM * 128, exchange = GROUPS > 1 ? (size_t)WAVES * 16384 : 0;
   constexpr size_t lds_bytes = stages > exchange ? stages : exchange;
   static_assert(lds_bytes <= 160 * 1024, "LDS per workgroup");
-  static bool lds_ok[kMaxDevices] = {false};
+  static std::atomic<bool> lds_ok[kMaxDevices];
   if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED>, (int)lds_bytes, lds_ok))
     return false;
   hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED>), grid, block, lds_bytes, p.stream,

@@ -25,6 +25,7 @@
 //
 // Shape requirements (checked by the launcher; other shapes use the generic GEMM
 // kernel): K a multiple of 64, every operand below 1 GiB.
+#include <atomic>
 #include <type_traits>
 
 #include "wq_device.h"
@@ -298,7 +299,7 @@ bool launch_pipe(const Problem& p, int group_shift) {
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   constexpr size_t lds_bytes = 3 * (size_t)(BM + BN) * 128;
   static_assert(lds_bytes <= 160 * 1024, "three stages must fit the 160 KB LDS");
-  static bool lds_ok[kMaxDevices] = {false};
+  static std::atomic<bool> lds_ok[kMaxDevices];
   if (!ensure_dynamic_lds((const void*)wq_gemm_pipe_kernel<BITS, BM, BN, WM, WN>, (int)lds_bytes, lds_ok)) return false;
   hipLaunchKernelGGL((wq_gemm_pipe_kernel<BITS, BM, BN, WM, WN>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,

@@ -1,5 +1,6 @@
 // Host-side contract between the C ABI (wq_capi.cpp) and the kernel launchers.
 #pragma once
+#include <atomic>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -55,7 +56,7 @@ int current_device_slot();
 // Raises a kernel's dynamic-LDS limit on the current device, once per device and kernel
 // (the attribute is per device; `done` is the kernel's own flag array of kMaxDevices
 // entries).  Returns false with the error set if the runtime refuses.
-bool ensure_dynamic_lds(const void* kernel, int bytes, bool* done);
+bool ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<bool>* done);
 
 // Compute units of the current device (cached per device).
 int cu_count();

@@ -77,17 +77,6 @@ def test_workspace_size_query_without_a_gpu():
         and "workspace" in lib.last_error() and "16-byte aligned" in lib.last_error()
 
 
-def test_measurement_probe_library_is_built_and_separate():
-    """bench.py's measurement aids (the MFMA rate probe and the read-only floor kernel) live in a library
-    of their own; the product library has no symbol of them."""
-    probe = os.path.join(os.path.dirname(lib.SO_PATH), "libmi355x_probe.so")
-    assert os.path.exists(probe), "make -C relax_amd/csrc all"
-    out = subprocess.run(["nm", "-D", "--defined-only", probe], capture_output=True, text=True).stdout
-    assert sorted(l.split()[-1] for l in out.splitlines() if " T " in l) == ["mi355x_probe_mfma_f16",
-                                                                              "mi355x_probe_stream_read"]
-    assert not hasattr(lib.load(), "mi355x_probe_mfma_f16") and not hasattr(lib.load(), "mi355x_probe_stream_read")
-
-
 @pytest.mark.parametrize("kw,msg", [
     (dict(bits=5), "bits must be 4 or 8"),
     (dict(group=48), "group must be 32 times a power of two"),

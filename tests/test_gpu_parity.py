@@ -185,7 +185,7 @@ def test_config2_llama7b_decode_projections(m, n, k):
 
 
 @pytest.mark.parametrize("m", [1, 16])
-@pytest.mark.parametrize("n,k", [(5120, 5120), (5120, 13824)])
+@pytest.mark.parametrize("n,k", [(15360, 5120), (5120, 5120), (27648, 5120), (5120, 13824)])
 def test_config4_q8_llama13b_skinny(m, n, k):
     x, wq, s, g = O.make_case(4, m, n, k, 8)
     got = run_matmul(x, wq, s, 8, g)
@@ -291,10 +291,15 @@ def test_gemm_pipelined_variant_refuses_k_not_multiple_of_64():
     assert_close(run_matmul(x, wq, s, 4, g, kernel=lib.KERNEL_GEMM), c_oracle.wq_matmul(x, wq, s, 4, g), "generic")
 
 
-@pytest.mark.parametrize("bits,m,n,k", [(4, 512, 4096, 4096), (4, 2048, 4096, 11008), (8, 256, 5120, 5120)])
+@pytest.mark.parametrize("bits,m,n,k",
+                         [(4, m, n, k) for m in (512, 2048)
+                          for n, k in ((12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008))] +
+                         [(8, 256, n, k) for n, k in ((15360, 5120), (5120, 5120), (27648, 5120), (5120, 13824))])
 def test_gemm_full_size_rows_against_oracle_and_all_tiles_against_torch(bits, m, n, k):
-    """Full-size prefill shapes: a sample of rows against the oracle (seconds on the host), and every
-    output tile against a float32 torch matmul of the bit-exact dequantized weights."""
+    """Every prefill shape of the q4f16 configuration (M = 512 and 2048 on the four Llama-2-7B
+    projections) and of the q8f16 configuration at M = 256 (the four Llama-2-13B projections), at full
+    size: a sample of rows against the oracle (seconds on the host), and every output tile against a
+    float32 torch matmul of the bit-exact dequantized weights."""
     import relax_amd
 
     x, wq, s, g = O.make_case(3, m, n, k, bits)
