@@ -165,6 +165,23 @@ MI355X_WQ_API int mi355x_wq_matmul_ws(const mi355x_wq_desc* desc, const void* x,
                                      const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int tiled,
                                      void* workspace, int64_t workspace_bytes);
 
+/* mi355x_wq_matmul_ws without a workspace argument and without any allocation: the partial tiles and
+ * arrival counters of the K split live in a device array that is part of the library's code object
+ * (mi355x_wq_static_ws_bytes() bytes: 16 KB of counters + 4 MB of partial tiles per GPU, held until the
+ * process ends).  It has no counterpart in the reference: it exists for callers that cannot allocate
+ * device memory or pass a buffer they own -- code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  The call itself calls no hipMalloc / hipFree or allocating library routine.
+ * Same results as mi355x_wq_matmul_ws with a sufficient workspace, bit for bit.  Where the split does not
+ * apply the call equals mi355x_wq_matmul_fused / _tiled; a problem whose split needs more than the array
+ * holds (mi355x_wq_workspace_bytes(...) > mi355x_wq_static_ws_bytes()) is refused with -1 -- use the
+ * caller-workspace form for it.  All calls on one GPU share that GPU's array: calls that overlap in time
+ * on one GPU (two streams, two threads) race; the kernel returns the counters to zero, so consecutive
+ * calls need no clearing. */
+MI355X_WQ_API int mi355x_wq_matmul_static_ws(const mi355x_wq_desc* desc, const void* x, const void* wq,
+                                            const void* scales, const mi355x_wq_epilogue* ep, void* y, int64_t m,
+                                            void* stream, int tiled);
+MI355X_WQ_API int64_t mi355x_wq_static_ws_bytes(void);
+
 /* Validates a descriptor and a row count without touching the GPU: 0 if
  * mi355x_wq_matmul would accept them. */
 MI355X_WQ_API int mi355x_wq_check(const mi355x_wq_desc* desc, int64_t m);

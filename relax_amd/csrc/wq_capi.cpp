@@ -199,7 +199,7 @@ namespace {
 
 int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
                       const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int kernel, bool tiled,
-                      void* workspace = nullptr, int64_t workspace_bytes = 0);
+                      void* workspace = nullptr, int64_t workspace_bytes = 0, bool library_scratch = false);
 
 }  // namespace
 
@@ -231,6 +231,14 @@ int mi355x_wq_matmul_ws(const mi355x_wq_desc* desc, const void* x, const void* w
   return matmul_any_layout(desc, x, wq_, scales, ep, y, m, stream, MI355X_WQ_KERNEL_AUTO, tiled != 0, workspace,
                            workspace_bytes);
 }
+
+int mi355x_wq_matmul_static_ws(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
+                               const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int tiled) {
+  return matmul_any_layout(desc, x, wq_, scales, ep, y, m, stream, MI355X_WQ_KERNEL_AUTO, tiled != 0, nullptr, 0,
+                           true);
+}
+
+int64_t mi355x_wq_static_ws_bytes(void) { return wq::gemv_static_scratch_bytes(); }
 
 int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const void* x, const void* wq_tiled,
                               const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y, int64_t m,
@@ -287,7 +295,7 @@ namespace {
 
 int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
                       const mi355x_wq_epilogue* ep, void* y, int64_t m, void* stream, int kernel, bool tiled,
-                      void* workspace, int64_t workspace_bytes) {
+                      void* workspace, int64_t workspace_bytes, bool library_scratch) {
   using namespace wq;
   if (!check_desc(desc, m)) return -1;
   if (ep != nullptr) {
@@ -332,6 +340,11 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
     // a caller workspace allows the decode kernel's K split where it pays; everything else is as without
     if (!check_ptr(workspace, "workspace", 16)) return -1;
     const int rc = launch_gemv_split(p, workspace, workspace_bytes);
+    if (rc != 0) return rc < 0 ? -1 : 0;
+  }
+  if (library_scratch) {
+    // the same split on the library's own device array: nothing is allocated, sizes beyond it are refused
+    const int rc = launch_gemv_split_static(p);
     if (rc != 0) return rc < 0 ? -1 : 0;
   }
   if (tiled) {

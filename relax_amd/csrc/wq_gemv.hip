@@ -783,4 +783,65 @@ int launch_gemv_split(const Problem& p, void* workspace, int64_t workspace_bytes
   return 1;
 }
 
+// ---- the K split on memory the library owns: an entry point that allocates nothing -------------------
+// For callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that forbid
+// hipMalloc): the partial tiles and arrival counters of the K split live in a file-scope device array
+// instead of a caller workspace.  Every GPU the library runs on holds its own copy of the array, at its
+// own address, until the process ends; the host-side name `scratch` is only a handle for
+// hipGetSymbolAddress, never an address a kernel may use.  The address is looked up once per device
+// (with that device current) and kept; kernels receive it as an argument, exactly as they receive a
+// caller's workspace.  The array starts zeroed (device variables are zero-initialised when the code
+// object is loaded) and every launch returns its counters to zero, so consecutive calls need no
+// clearing; partial tiles are written before they are read.  All calls on one GPU share the array:
+// calls that overlap in time on one GPU (different streams, different threads) race.
+static __device__ __align__(256) unsigned char scratch[kSplitCounterBytes + 4 * 1024 * 1024];
+
+namespace {
+
+constexpr int64_t kStaticScratchBytes = kSplitCounterBytes + 4 * 1024 * 1024;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of the current device's copy of `scratch`, or nullptr with the error set.
+void* static_scratch_address() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) {
+    (void)hipGetLastError();
+    set_error("no usable HIP device in this process");
+    return nullptr;
+  }
+  const bool cached = dev < kMaxDevices;  // beyond the table: looked up on every call
+  if (cached) {
+    void* known = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (known != nullptr) return known;
+  }
+  void* ptr = nullptr;
+  const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || ptr == nullptr) {
+    (void)hipGetLastError();
+    set_error("cannot resolve the library's scratch array on device %d: %s", dev, hipGetErrorString(e));
+    return nullptr;
+  }
+  if (cached) g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  return ptr;
+}
+
+}  // namespace
+
+int64_t gemv_static_scratch_bytes() { return kStaticScratchBytes; }
+
+// 1 = launched with the K split on the library's scratch array, 0 = the split does not apply to `p`
+// (nothing launched), -1 = failure: the split would need more than the array holds, or a runtime error
+int launch_gemv_split_static(const Problem& p) {
+  const int64_t need = gemv_split_workspace_bytes(p);
+  if (need == 0) return 0;
+  if (need > kStaticScratchBytes) {
+    set_error("the K split of this problem needs %lld bytes of scratch memory, the library's own array holds %lld: "
+              "use mi355x_wq_matmul_ws with a caller workspace", (long long)need, (long long)kStaticScratchBytes);
+    return -1;
+  }
+  void* const ptr = static_scratch_address();
+  if (ptr == nullptr) return -1;
+  return launch_gemv_split(p, ptr, kStaticScratchBytes);
+}
+
 }  // namespace wq

@@ -32,6 +32,10 @@ bool gemv_applicable(const Problem& p);  // M <= 16 and a default variant's LDS 
 // must be zero before the first use and are zero again when the kernel has finished.
 int64_t gemv_split_workspace_bytes(const Problem& p);
 int launch_gemv_split(const Problem& p, void* workspace, int64_t workspace_bytes);
+// The same split on the library's own file-scope device array (no caller workspace, no allocation):
+// 1 launched, 0 the split does not apply, -1 failure (also when the problem needs more than the array holds).
+int launch_gemv_split_static(const Problem& p);
+int64_t gemv_static_scratch_bytes();
 int launch_skinny(const Problem& p, int variant);
 int launch_gemm(const Problem& p, int variant);
 bool gemm_pipe_applicable(const Problem& p);  // K % 64 == 0, operands below 1 GiB

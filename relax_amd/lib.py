@@ -17,7 +17,7 @@ EXPORTED_SYMBOLS = (
     "mi355x_wq_matmul", "mi355x_wq_matmul_ex", "mi355x_wq_matmul_fused", "mi355x_wq_matmul_fused_ex",
     "mi355x_wq_dequantize", "mi355x_wq_check",
     "mi355x_wq_tiled_sizes", "mi355x_wq_tile_weights", "mi355x_wq_untile_weights", "mi355x_wq_matmul_tiled", "mi355x_wq_matmul_tiled_ex",
-    "mi355x_wq_workspace_bytes", "mi355x_wq_matmul_ws",
+    "mi355x_wq_workspace_bytes", "mi355x_wq_matmul_ws", "mi355x_wq_matmul_static_ws", "mi355x_wq_static_ws_bytes",
     "mi355x_wq_select_kernel", "mi355x_wq_last_error", "mi355x_wq_version",
     "mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_matmul_bias", "mi355x_q8f16_matmul_bias",
     "mi355x_q4f16_matmul_bias_relu", "mi355x_q8f16_matmul_bias_relu", "mi355x_q4f16_matmul_residual",
@@ -90,6 +90,8 @@ def load() -> C.CDLL:
     L.mi355x_wq_workspace_bytes.argtypes = [dp, i64, ci]
     L.mi355x_wq_workspace_bytes.restype = i64
     L.mi355x_wq_matmul_ws.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp, ci, vp, i64]
+    L.mi355x_wq_matmul_static_ws.argtypes = [dp, vp, vp, vp, ep, vp, i64, vp, ci]
+    L.mi355x_wq_static_ws_bytes.restype = i64
     L.mi355x_wq_check.argtypes = [dp, i64]
     L.mi355x_wq_select_kernel.argtypes = [dp, i64]
     L.mi355x_wq_last_error.restype = C.c_char_p
