@@ -81,7 +81,19 @@ MI355X_WQ_API int mi355x_wq_matmul_ex(const mi355x_wq_desc* desc, const void* x,
  * path cannot lower erf on float16 (src/target/intrin_rule.h:39-48), so there is nothing to match. */
 enum {
   MI355X_WQ_ACT_NONE = 0,
-  MI355X_WQ_ACT_RELU = 1
+  MI355X_WQ_ACT_RELU = 1,
+  /* Gated tail of a fused gate+up projection (rows 0 .. N/2-1 of the weights: gate, rows N/2 .. N-1: up):
+   *   y[M, N/2] = multiply(nn.silu(h[:, :N/2]), h[:, N/2:]),  h = f16(accumulator)
+   * with the float16 operation sequence of the CPU path -- nn.silu(x) = multiply(x, sigmoid(x))
+   * (python/tvm/relax/transform/legalize_ops.py:506-510), sigmoid(x) = 1 / (1 + exp(-x))
+   * (src/target/intrin_rule.cc:135-141), exp evaluated in float32 and rounded: five float16 roundings.
+   * Identical to the CPU result except where the last bit of the float32 exp differs between the two
+   * math libraries and survives the rounding to float16 (about one output in a few thousand, then a few
+   * float16 ulp).  The reference's counterpart is the activation member of its fused matmul patterns
+   * (python/tvm/relax/dpl/pattern.py:1049-1095, python/tvm/contrib/cutlass/gen_tensor_op.py:377-380).
+   * `y` is [M, N/2]; no bias, no residual, canonical weights, N even; M <= 16 runs the decode kernel,
+   * larger M needs K % 256 == 0 with group 32 (int4) / 128 (int8). */
+  MI355X_WQ_ACT_SILU_MUL = 2
 };
 typedef struct mi355x_wq_epilogue {
   const void* bias;     /* float16 [N] (device), or NULL */

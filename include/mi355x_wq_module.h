@@ -46,7 +46,8 @@ typedef int (*mi355x_wq_packed_cfunc)(mi355x_tvm_value* args, int* type_codes, i
                                       void* resource_handle);
 
 enum {
-  MI355X_WQ_MODULE_TILE_WEIGHTS = 1, /* convert bound weights to the tile-major layout at init */
+  MI355X_WQ_MODULE_TILE_WEIGHTS = 1, /* convert bound weights to the tile-major layout at init (where it is defined) */
+  MI355X_WQ_MODULE_LIBRARY_SCRATCH = 2, /* decode calls may split K on the library's scratch array (mi355x_wq_matmul_static_ws) */
   MI355X_DL_CPU = 1                  /* kDLCPU */
 };
 
@@ -57,7 +58,8 @@ MI355X_WQ_API const char* mi355x_wq_module_type_key(void);
 /* Creates the module of one composite function.  `spec` describes the full argument list;
  * `const_args[i]` is the slot bound by the constant named `const_names[i]` (slots of wq, scales or
  * bias; never x, the residual or the output).  A module without constants needs no init call.
- * MI355X_WQ_MODULE_TILE_WEIGHTS needs both wq and scales among the constants of a matmul.
+ * MI355X_WQ_MODULE_TILE_WEIGHTS needs both wq and scales among the constants of a matmul; for a
+ * (bits, group, K) the tile-major layout is not defined for, init keeps the canonical constants.
  * Returns 0 and the module in *out, or -1 (mi355x_wq_last_error). */
 MI355X_WQ_API int mi355x_wq_module_create(const char* symbol, const mi355x_wq_callspec* spec,
                                          const char* const* const_names, const int32_t* const_args,

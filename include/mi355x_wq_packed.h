@@ -70,6 +70,7 @@ enum {
  *   matmul     : x[M,K] f16, wq[N,K*bits/32] u32, scales[N,K/group] f16, y[M,N] f16 (output, last)
  *   matmul_bias / matmul_bias_relu : x, wq, scales, bias[N] f16, y
  *   matmul_residual                : x, wq, scales, residual[M,N] f16, y
+ *   matmul_silu_mul                : x, wq, scales, y[M,N/2] f16 (gate rows then up rows in wq: MI355X_WQ_ACT_SILU_MUL)
  *   dequantize : wq, scales, wd[N,K] f16 (output, last)
  * group is K / scales.shape[1]; the zero point is 7 (q4f16) or 0 (q8f16).
  * Return 0, or -1 after recording the message with TVMAPISetLastError (when the
@@ -94,6 +95,12 @@ MI355X_WQ_API int mi355x_q8f16_matmul_bias_relu(mi355x_tvm_value* args, int* typ
                                   mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
                                   void* resource_handle);
 MI355X_WQ_API int mi355x_q8f16_matmul_residual(mi355x_tvm_value* args, int* type_codes, int num_args,
+                                 mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
+                                 void* resource_handle);
+MI355X_WQ_API int mi355x_q4f16_matmul_silu_mul(mi355x_tvm_value* args, int* type_codes, int num_args,
+                                 mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
+                                 void* resource_handle);
+MI355X_WQ_API int mi355x_q8f16_matmul_silu_mul(mi355x_tvm_value* args, int* type_codes, int num_args,
                                  mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
                                  void* resource_handle);
 MI355X_WQ_API int mi355x_q4f16_dequantize(mi355x_tvm_value* args, int* type_codes, int num_args,
@@ -156,6 +163,14 @@ typedef struct mi355x_wq_callspec {
 /* The body every entry (fixed-name or generated trampoline) forwards to. */
 MI355X_WQ_API int mi355x_wq_packed_call(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes,
                           int num_args);
+/* The same body for entries generated with the hook's option {"workspace": true}: decode matmuls (M <= 16) may
+ * split K across workgroups on the library's own scratch array (mi355x_wq_matmul_static_ws in mi355x_wq.h:
+ * nothing is allocated; calls that overlap in time on one GPU must not both take this path).  The
+ * reference's counterpart is the per-backend options map RunCodegen hands to the hook
+ * (src/relax/transform/run_codegen.cc:155-162), which its cutlass backend reads for its split-K /
+ * tuning switches (python/tvm/contrib/cutlass/build.py:695-696). */
+MI355X_WQ_API int mi355x_wq_packed_call_scratch(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes,
+                                               int num_args);
 
 /* Stream used by the packed entries on the calling thread (hipStream_t as void*;
  * NULL = null stream, TVM's default: src/runtime/rocm/rocm_common.h:53-63). */

@@ -39,6 +39,8 @@ def lib() -> C.CDLL:
         L.wq_oracle_wq_matmul.argtypes = [C.c_int, i64, p, p, p, i64, i64, i64, p, p, p, C.c_int]
         L.wq_oracle_epilogue.argtypes = [p, i64, i64, p, C.c_int, p]
         L.wq_oracle_epilogue.restype = None
+        L.wq_oracle_silu_mul.argtypes = [p, i64, i64, p]
+        L.wq_oracle_silu_mul.restype = None
         _lib = L
     return _lib
 
@@ -119,6 +121,16 @@ def wq_matmul(x, wq, s, bits: int, group: int, nthreads: int = 1) -> np.ndarray:
 def epilogue(y, bias=None, activation=None, residual=None) -> np.ndarray:
     """Fused tail on a copy of y [M,N] float16: + bias[N], relu, + residual[M,N]."""
     L = lib()
+    if activation == "silu_mul":
+        if bias is not None or residual is not None:
+            raise ValueError("the gated tail takes no bias or residual")
+        src = np.ascontiguousarray(y, dtype=np.float16)
+        m, n = src.shape
+        if n % 2 != 0:
+            raise ValueError("the gated tail needs an even number of output columns")
+        gated = np.empty((m, n // 2), dtype=np.float16)
+        L.wq_oracle_silu_mul(_ptr(src), m, n, _ptr(gated))
+        return gated
     out = np.array(y, dtype=np.float16, order="C", copy=True)
     m, n = out.shape
     if activation not in (None, "none", "relu", "relax.nn.relu"):

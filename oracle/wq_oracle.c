@@ -24,6 +24,7 @@
  * Build: gcc -O2 -ffp-contract=off -fno-fast-math -fopenmp -shared -fPIC
  * (no reassociation, no fused multiply-add: the float32 sum must stay sequential).
  */
+#include <math.h>
 #include <stdint.h>
 #include <string.h>
 
@@ -180,6 +181,25 @@ void wq_oracle_epilogue(uint16_t* y, int64_t m_rows, int64_t n_rows, const uint1
       if (residual)
         h = wq_oracle_f32_to_f16(wq_oracle_f16_to_f32(h) + wq_oracle_f16_to_f32(residual[m * n_rows + n]));
       y[m * n_rows + n] = h;
+    }
+}
+
+/* ---- gated tail: out[m, j] = multiply(nn.silu(y[m, j]), y[m, j + n/2]) for j < n/2, the float16
+ * operation sequence of python/tvm/relax/transform/legalize_ops.py:506-510 and
+ * src/target/intrin_rule.cc:135-141: e = f16(expf(-g)), d = f16(1 + e), s = f16(1 / d),
+ * t = f16(g * s), out = f16(t * u).  Sum, quotient and products of float16 values rounded through
+ * float32 equal one rounding (24 >= 2*11 + 2 significand bits). ---- */
+void wq_oracle_silu_mul(const uint16_t* y, int64_t m_rows, int64_t n_rows, uint16_t* out) {
+  const int64_t half = n_rows / 2;
+  for (int64_t m = 0; m < m_rows; ++m)
+    for (int64_t j = 0; j < half; ++j) {
+      const float g = wq_oracle_f16_to_f32(y[m * n_rows + j]);
+      const float u = wq_oracle_f16_to_f32(y[m * n_rows + half + j]);
+      const float e = wq_oracle_f16_to_f32(wq_oracle_f32_to_f16(expf(-g)));
+      const float d = wq_oracle_f16_to_f32(wq_oracle_f32_to_f16(1.0f + e));
+      const float s = wq_oracle_f16_to_f32(wq_oracle_f32_to_f16(1.0f / d));
+      const float t = wq_oracle_f16_to_f32(wq_oracle_f32_to_f16(g * s));
+      out[m * half + j] = wq_oracle_f32_to_f16(t * u);
     }
 }
 

@@ -34,6 +34,16 @@ Reference semantics followed (file:line under the reference tree):
   emitted as select(t > 0, t, 0) with an ordered compare
   (src/target/llvm/codegen_llvm.cc:1500-1504): -0 and NaN both give +0.
 
+* gated tail (the gate+up projection of a Llama MLP followed by `multiply(nn.silu(gate), up)` on the two
+  halves of the output): `relax.nn.silu` legalizes to `multiply(x, sigmoid(x))`
+  (python/tvm/relax/transform/legalize_ops.py:506-510), `sigmoid` to `1 / (1 + exp(-x))` in the tensor's
+  dtype (src/target/intrin_rule.cc:135-141) and `exp` to the llvm.exp intrinsic
+  (src/target/llvm/intrin_rule_llvm.cc:41-42), which on a float16 operand is evaluated in float32
+  (extend, expf, truncate).  Every float16 operation rounds once: e = f16(expf(-g)), d = f16(1 + e),
+  s = f16(1 / d), t = f16(g * s), y = f16(t * u).  The one step that is not fixed by IEEE arithmetic is
+  the last bit of expf (the host libm's); rounded to float16 it differs between correct
+  implementations in about one operand in a few thousand.
+
 Layout decisions frozen by this build (the reference holds no quantized path):
 element k of a row lives in word k // per_word at bit offset
 (k % per_word) * bits, least-significant field first.
@@ -190,10 +200,41 @@ def relu_f16(t: np.ndarray) -> np.ndarray:
         return np.where(t > np.float16(0), t, np.float16(0)).astype(np.float16)
 
 
+def silu_mul_f16(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+    """multiply(nn.silu(gate), up) on float16 tensors, every operation rounded once to float16:
+    e = f16(expf(-g)); d = f16(1 + e); s = f16(1 / d); t = f16(g * s); y = f16(t * u).
+    expf is taken as the correctly rounded float32 exponential (float64 exp rounded to float32: what
+    glibc's expf returns in all but astronomically rare cases); sums and products of two float16 values
+    are exact in float64 before their single rounding."""
+    g = np.asarray(gate, dtype=np.float16)
+    u = np.asarray(up, dtype=np.float16)
+    with np.errstate(over="ignore", invalid="ignore", divide="ignore", under="ignore"):
+        e = np.exp(-g.astype(np.float64)).astype(np.float32).astype(np.float16)
+        d = (np.float64(1) + e.astype(np.float64)).astype(np.float16)
+        # 1 / d in float32 is correctly rounded and 24 >= 2 * 11 + 2 bits make the second rounding innocuous
+        s = (np.float32(1) / d.astype(np.float32)).astype(np.float16)
+        t = (g.astype(np.float64) * s.astype(np.float64)).astype(np.float16)
+        return (t.astype(np.float64) * u.astype(np.float64)).astype(np.float16)
+
+
+def gated_epilogue(y: np.ndarray) -> np.ndarray:
+    """y [M, N] = f16(accumulator) of a fused gate+up projection -> [M, N/2]:
+    multiply(nn.silu(y[:, :N/2]), y[:, N/2:])."""
+    y = np.asarray(y, dtype=np.float16)
+    if y.ndim != 2 or y.shape[1] % 2 != 0:
+        raise ValueError("the gated tail needs an even number of output columns")
+    half = y.shape[1] // 2
+    return silu_mul_f16(y[:, :half], y[:, half:])
+
+
 def epilogue(y: np.ndarray, bias=None, activation: str | None = None, residual=None) -> np.ndarray:
     """The fused tail of a composite applied to y = f16(accumulator):
     + bias[N], then relu, then + residual[M,N]; every step absent or one float16 op."""
     t = np.asarray(y, dtype=np.float16)
+    if activation == "silu_mul":
+        if bias is not None or residual is not None:
+            raise ValueError("the gated tail takes no bias or residual")
+        return gated_epilogue(t)
     if bias is not None:
         t = add_f16(t, np.asarray(bias, dtype=np.float16).reshape(1, -1))
     if activation in ("relu", "relax.nn.relu"):

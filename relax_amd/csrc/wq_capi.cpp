@@ -303,9 +303,25 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
       set_error("epilogue.reserved must be 0, got %d", ep->reserved);
       return -1;
     }
-    if (ep->activation != MI355X_WQ_ACT_NONE && ep->activation != MI355X_WQ_ACT_RELU) {
+    if (ep->activation != MI355X_WQ_ACT_NONE && ep->activation != MI355X_WQ_ACT_RELU &&
+        ep->activation != MI355X_WQ_ACT_SILU_MUL) {
       set_error("unknown epilogue activation %d", ep->activation);
       return -1;
+    }
+    if (ep->activation == MI355X_WQ_ACT_SILU_MUL) {
+      // y[M, N/2] = multiply(nn.silu(acc[:, :N/2]), acc[:, N/2:]): the whole tail of a gate+up projection
+      if (ep->bias != nullptr || ep->residual != nullptr) {
+        set_error("the gated tail (silu_mul) takes no bias and no residual");
+        return -1;
+      }
+      if (desc->n % 2 != 0) {
+        set_error("the gated tail (silu_mul) needs an even N (gate rows, then as many up rows), got N=%lld", (long long)desc->n);
+        return -1;
+      }
+      if (tiled) {
+        set_error("the gated tail (silu_mul) is computed on canonical weights only");
+        return -1;
+      }
     }
   }
   if (m == 0 || desc->n == 0) return 0;  // empty output
@@ -335,6 +351,16 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
       return -1;
     }
     p.tiled = true;
+  }
+  if (p.activation == MI355X_WQ_ACT_SILU_MUL) {
+    // Gated tail: the decode kernel (M <= 16, any of its variants) and the direct-weight GEMM walk the weight
+    // rows in the interleaved gate / up order; the K split, the skinny kernel and the LDS-staged GEMMs do not.
+    if (family == MI355X_WQ_KERNEL_SKINNY) {
+      set_error("the gated tail (silu_mul) is not implemented by the skinny kernel");
+      return -1;
+    }
+    const bool decode = family == MI355X_WQ_KERNEL_GEMV || (family == MI355X_WQ_KERNEL_AUTO && m <= 16 && gemv_applicable(p));
+    return decode ? launch_gemv(p, variant) : launch_gemm(p, variant);
   }
   if (workspace != nullptr && family == MI355X_WQ_KERNEL_AUTO) {
     // a caller workspace allows the decode kernel's K split where it pays; everything else is as without

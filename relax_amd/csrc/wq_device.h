@@ -149,8 +149,31 @@ __device__ __forceinline__ half8_t pack_h8(half2_t a, half2_t b, half2_t c, half
 struct Epilogue {
   const half_t* bias;      // [N], or nullptr
   const half_t* residual;  // [M,N], or nullptr; may be the output buffer itself
-  int activation;          // 0 none, 1 relu
+  int activation;          // 0 none, 1 relu, 2 gated: y[M, N/2] = multiply(nn.silu(gate), up), see store_gated
 };
+constexpr int kActGated = 2;
+
+// Gated tail of a fused gate+up projection.  The weight matrix holds the gate rows 0 .. N/2-1 and the up
+// rows N/2 .. N-1; kernels that fuse the tail walk the rows in the interleaved order
+// gate 0, up 0, gate 1, up 1, ... (logical row r = physical row r/2 + (r odd ? N/2 : 0)), so that the two
+// accumulators of an output land in one lane or in adjacent lanes.
+__device__ __forceinline__ int gated_physical_row(int logical, int N) { return (logical >> 1) + ((logical & 1) ? (N >> 1) : 0); }
+
+// multiply(nn.silu(g), u) on float16 values, every operation rounded once as the CPU path executes them:
+// e = f16(exp(-g)) (evaluated in float32), d = f16(1 + e), s = f16(1 / d), t = f16(g * s), y = f16(t * u).
+// The float32 quotient is correctly rounded and its second rounding to float16 is innocuous.
+__device__ __forceinline__ half_t silu_mul(half_t g, half_t u) {
+  const half_t e = (half_t)expf(-(float)g);
+  const half_t d = (half_t)1 + e;
+  const half_t s = (half_t)(1.0f / (float)d);
+  const half_t t = g * s;
+  return t * u;
+}
+
+// y[m, j] of the gated output [M, N/2] from the accumulators of gate row j and up row j
+__device__ __forceinline__ void store_gated(half_t* y, int m, int j, int half_n, float acc_gate, float acc_up) {
+  y[(size_t)m * half_n + j] = silu_mul((half_t)acc_gate, (half_t)acc_up);
+}
 
 __device__ __forceinline__ void store_out(const Epilogue& ep, half_t* y, int m, int n, int N, float acc) {
   half_t h = (half_t)acc;

@@ -255,6 +255,13 @@ int launch_gemm(const Problem& p, int variant) {
       variant = -1;
     else variant = p.m >= 1024 ? 11 : 12;
   }
+  if (p.activation == kActGated && variant != -1 && variant < 21) {
+    // only the direct-weight kernel walks the rows in the interleaved gate / up order
+    set_error("gemm kernel: the gated tail (silu_mul) needs the direct-weight kernel: K %% 256 == 0, group %d, operands "
+              "below 1 GiB; got M=%lld N=%lld K=%lld group=%d variant=%d", p.bits == 4 ? 32 : 128, (long long)p.m,
+              (long long)p.n, (long long)p.k, p.group, variant);
+    return -1;
+  }
   if (variant == -1) {
     // launched above
   } else if (variant >= 21) {

@@ -84,7 +84,8 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     const Epilogue ep) {
   // (argument order: the first 14 dwords are preloaded into SGPRs at wavefront launch, later ones are
   // a scalar load at the start of the kernel; what the K loop needs comes first, y and the epilogue last)
-  const int group_shift = shift_and_zero & 0xFF, zero_point = shift_and_zero >> 8;
+  const int group_shift = shift_and_zero & 0xFF, zero_point = (shift_and_zero >> 8) & 0xFF;
+  const bool gated = (shift_and_zero >> 16) & 1;  // fused multiply(nn.silu(gate), up): rows walked interleaved
   constexpr int BK = 64;
   static_assert(TM == 4 || TM == 2, "row blocks of 32 per wavefront: 128- or 64-row tile");
   static_assert(WAVES == 4 || WAVES == 2, "wavefronts per K group: 256 or 128 output columns");
@@ -162,7 +163,8 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   for (int j = 0; j < 2; ++j) {
     // column tile j of the MFMA holds the tile's columns of parity j (lane fr: column 2 fr + j), so
     // that a lane ends up with two adjacent outputs of a row and a wavefront stores whole 128-byte lines
-    const int n = min(n0 + wave * 64 + 2 * fr + j, (int)n_stored - 1);  // rows past N: computed, not stored
+    int n = min(n0 + wave * 64 + 2 * fr + j, (int)n_stored - 1);  // rows past N: computed, not stored
+    if (gated) n = gated_physical_row(n, N);  // column parity j: gate row / up row of output (n0 + wave*64)/2 + fr
     if constexpr (TILED) {
       // chunk c of row n sits at ((tile*S + c/8)*2 + c%2)*1024 + ((c%8)/2*16 + n%16)*16; the lane's chunks
       // of step kt are 2 kt + fh (int4) or 4 kt + 2 fh + v (int8), which leaves these lane constants
@@ -474,8 +476,19 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   }
 
   // ---- epilogue: lane holds columns 2 (lane % 32), + 1 and rows 8*(v/4) + 4*(lane/32) + v%4 ------
-  const bool paired = pair_store_ok(ep, y, N);
   const int n = n0 + wave * 64 + 2 * fr;
+  if (gated) {
+    // the lane's two columns are the gate and the up accumulator of output column n / 2
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
+        if (m < M && n + 1 < N) store_gated(y, m, n >> 1, N >> 1, acc[i][0][v], acc[i][1][v]);
+      }
+    return;
+  }
+  const bool paired = pair_store_ok(ep, y, N);
   if (paired && m0 + BM <= M && n0 + WAVES * 64 <= N) {
     // Tile inside the matrix, 4-byte accesses allowed: the tail's shape is decided once, outside the
     // unrolled stores (per-element tests of the three epilogue fields cost more than the stores).
@@ -548,7 +561,7 @@ bool launch_direct(const Problem& p, int group_shift, int tile_n0 = 0, int tile_
     return false;
   hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales, (int)p.m, (int)p.n,
-                     (int)p.k, group_shift | (p.zero_point << 8), tiles_m, tiles_n, tile_n0, (half_t*)p.y,
+                     (int)p.k, group_shift | (p.zero_point << 8) | (p.activation == kActGated ? 1 << 16 : 0), tiles_m, tiles_n, tile_n0, (half_t*)p.y,
                      Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
   return true;
 }

@@ -34,14 +34,10 @@
 // exactly what a wavefront reads per instruction (D = 2): every load of the weight stream
 // is 1 KB contiguous.  Same lanes, same chunks, same order: bit-identical results.
 //
-// Activations: a wavefront only ever multiplies its own K range, so it stages exactly that slice
-// of every activation row itself, into LDS columns of its own -- no workgroup barrier stands between
-// a wavefront and its weight stream.  (With a barrier there, the last wavefront's activation loads
-// queue in the CU's memory pipeline behind the weight requests of every wavefront launched before
-// it, and all of them wait for that.)  XB: activation vectors a lane requests ahead of its first
-// weights (1, 2, 4 or 8; a masked-off request still takes its turn in the memory pipeline, so the
-// launcher picks the smallest that covers the rows).  NS: register sets of the weight stream, all
-// requested before the first wait (two; three and four were measured 3 - 15 % slower at every shape).
+// ROWS: how the activations reach LDS.  false: a flat index over (row, 16-byte column), two requests
+// per thread ahead of the first weights (batch 1 - 2, or rows longer than the workgroup has
+// threads); true: a thread stages its own column of four or eight rows, all requested ahead of
+// the first weights.
 //
 // KSPLIT: K is split over R workgroups per tile list as well (caller workspace): each writes a
 // float32 partial tile, the last to arrive adds them in the order of the K windows and stores.
@@ -74,7 +70,7 @@ struct GemvArgs {
   Epilogue ep;
 };
 
-template <int BITS, int WAVES, int D, int SPL, bool TILED, int XB, int NS, bool KSPLIT>
+template <int BITS, int WAVES, int D, int SPL, bool TILED, bool ROWS, bool KSPLIT>
 // Scalar kernel arguments instead of one struct, and in this order: the first 14 dwords of the
 // argument segment are preloaded into SGPRs at wavefront launch (16 user SGPRs less the segment
 // pointer); anything after them is fetched by a scalar load from host-visible memory.
@@ -86,7 +82,8 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     const half_t* x_, const uint32_t* wq_, const half_t* scales_, int M_, int N_, int K_,
     int shift_and_zero_, int max_tiles_, int phase_chunks_, int ksplit_, int grid_, half_t* y_, const Epilogue ep_,
     float* partials_, unsigned int* counters_) {
-  const int group_shift_ = shift_and_zero_ & 0xFF, zero_point_ = shift_and_zero_ >> 8;
+  const int group_shift_ = shift_and_zero_ & 0xFF, zero_point_ = (shift_and_zero_ >> 8) & 0xFF;
+  const bool gated = (shift_and_zero_ >> 16) & 1;  // fused multiply(nn.silu(gate), up): rows walked interleaved
   const int tiles_ = (N_ + 15) >> 4;
   const int lds_stride_ = phase_chunks_ * (128 / BITS) + 8;  // halves per staged row (launch_one's plan)
   GemvArgs a;
@@ -142,11 +139,6 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
 
   const Q4Consts qc = make_q4_consts(a.zero_point);
   const half_t* xrow = xs + (size_t)(col < M ? col : 0) * a.lds_stride;
-  constexpr int VS = 4 * D * CH / 8;  // 16-byte vectors of one activation row per super step
-  // super steps of a wavefront in a full phase: the stride of the wavefronts' LDS columns
-  const int pw_full = ((a.phase_chunks + 4 * D - 1) / (4 * D) + WAVES - 1) / WAVES;
-  half_t* const xs_wave = xs + wave * pw_full * (4 * D * CH);
-  const half_t* const xrow_wave = xrow + wave * pw_full * (4 * D * CH);
 
   // weights of (tile index i, super step ss of the current phase) -> registers
   auto load_super = [&](GemvBuf<D, SPL>& b, int i, int ss, int chunk_base, int ss_end) {
@@ -165,7 +157,8 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
       else b.sc[0] = load_b32(rs, ok ? (item * 64u + (uint32_t)lane) * 4u : kOobOffset);
       return;
     }
-    const int n = min((tile0 + i * tstride) * 16 + col, N - 1);  // rows past N: computed, not stored
+    int n = min((tile0 + i * tstride) * 16 + col, N - 1);  // rows past N: computed, not stored
+    if (gated) n = gated_physical_row(n, N);  // even columns of a tile: gate rows, odd columns: their up rows
     const int chunk0 = chunk_base + ss * 4 * D + kq * D;
     // D > 1 is only launched when K is a multiple of 4*D chunks, so a lane's D
     // chunks are valid together; D == 1 checks its single chunk.
@@ -192,9 +185,9 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
 
   float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  // one super step of MFMAs; `ss_local` counts the wavefront's own super steps of this phase
+  // one super step of MFMAs; `ss_local` addresses the staged activations of this phase
   auto compute_super = [&](const GemvBuf<D, SPL>& b, int ss_local) {
-    const half_t* xp = xrow_wave + (ss_local * 4 * D + kq * D) * CH;
+    const half_t* xp = xrow + (ss_local * 4 * D + kq * D) * CH;
     half8_t av[2][NJ];  // activations of chunk d+1 are read from LDS while chunk d is consumed
 #pragma unroll
     for (int j = 0; j < NJ; ++j) av[0][j] = *reinterpret_cast<const half8_t*>(xp + j * 8);
@@ -235,10 +228,9 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     acc = float4_t{0.f, 0.f, 0.f, 0.f};
   };
 
-  // One K phase: every wavefront stages its own slice of the activations and streams every tile of the
-  // workgroup over it.  The first phase is a copy of its own ahead of the loop over the others: inside
-  // a loop the compiler hoists the stream's constants in front of it, i.e. in front of the kernel's
-  // first requests.
+  // One K phase: stage its activations, stream every tile of the workgroup over it.  The first phase
+  // is a copy of its own ahead of the loop over the others: inside a loop the compiler hoists the
+  // stream's constants in front of it, i.e. in front of the kernel's first requests.
   auto run_phase = [&](const int ph) {
     const int chunk_base = (KSPLIT ? kr : ph) * a.phase_chunks;
     const int ph_chunks = min(a.phase_chunks, nchunks - chunk_base);
@@ -248,26 +240,15 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     const int ss_end = min(ss_begin + per_wave, nsuper);
     const int cnt = max(ss_end - ss_begin, 0);  // super steps per tile for this wavefront
 
-    // the weight stream: a flat software pipeline over (tile, super step), NS register sets deep
-    const int items = my_tiles * cnt;
-    int ci = 0, cs = 0;  // tile / local super step of the item being consumed
-    int pi = 0, ps = 0;  // ... of the next item to request
-    auto advance = [&](int& i, int& s) {
-      if (++s >= cnt) {
-        s = 0;
-        ++i;
-      }
-    };
-    GemvBuf<D, SPL> buf[NS];
-
-    // ---- this wavefront's slice of the activations (zero padded to whole super steps) -------
-    // cnt * VS vectors per row from k_first on; lane l owns vectors l, l + 64, ... of every row.
-    // The first XB requests go out ahead of the first weights and are stored after them: loads
-    // of a wavefront retire in order, so they are back long before the weights.
+    // ---- stage this phase's activations (zero padded to a whole k-step) ---------------
+    // The first batch of vectors per thread is requested before the first weights and
+    // stored after them: global loads retire in order, so the LDS fill does not wait
+    // for the much slower first weight loads.
+    GemvBuf<D, SPL> b0, b1;
     {
-      const int k_first = (chunk_base + ss_begin * 4 * D) * CH;
-      const int vpr = cnt * VS;
-      const int J = (vpr + 63) >> 6;  // requests per row and lane
+      const int kbase = chunk_base * CH;
+      const int kpad = ((ph_chunks + 3) / 4) * 4 * CH;
+      const int vec_per_row = kpad / 8;
       auto permute_x = [&](u32x4 v) -> u32x4 {
         if constexpr (BITS == 4) {
           u32x4 p;
@@ -280,72 +261,125 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
           return v;
         }
       };
-      auto x_load = [&](int m, int j) -> u32x4 {
-        const int v = lane + 64 * j, k = k_first + v * 8;
-        const bool ok = m < M && v < vpr && k < K;
-        return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)k) * 2u : kOobOffset);
-      };
-      auto x_store = [&](int m, int j, u32x4 val) {
-        const int v = lane + 64 * j;
-        if (m < M && v < vpr) *reinterpret_cast<u32x4*>(xs_wave + (size_t)m * a.lds_stride + v * 8) = permute_x(val);
-      };
-      auto next = [&](int& m, int& j) {  // wave-uniform counters: scalar arithmetic
-        if (++j >= J) {
-          j = 0;
-          ++m;
+      if (ph > 0) __syncthreads();  // every wavefront is done reading the previous phase
+      if constexpr (!ROWS) {
+        // one or two rows, or rows longer than the workgroup has threads: a flat index over (row, column),
+        // two vectors per thread ahead of the weights
+        // (every extra request, even one that is masked off, takes its turn in the memory pipeline
+        // ahead of the first weights: the batch-1 start-up is kept as short as it can be)
+        const int total = M * vec_per_row;
+        auto x_load = [&](int idx) -> u32x4 {
+          const int m = idx / vec_per_row, kv = idx - m * vec_per_row;
+          const bool ok = idx < total && kbase + kv * 8 < K;
+          return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
+        };
+        auto x_store = [&](int idx, u32x4 v) {
+          if (idx >= total) return;
+          const int m = idx / vec_per_row, kv = idx - m * vec_per_row;
+          *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = permute_x(v);
+        };
+        // (the first two vectors without the division when a row has at least as many vectors as the
+        // workgroup has threads -- K >= 4096: they are in row 0 or 1; the start-up of a 5 us kernel is
+        // a few hundred instructions, and a division is forty of them)
+        int m0, kv0, m1, kv1;
+        if (vec_per_row >= NT) {
+          m0 = 0;
+          kv0 = tid;
+          m1 = tid + NT >= vec_per_row ? 1 : 0;
+          kv1 = tid + NT - m1 * vec_per_row;
+        } else {
+          m0 = tid / vec_per_row;
+          kv0 = tid - m0 * vec_per_row;
+          m1 = (tid + NT) / vec_per_row;
+          kv1 = tid + NT - m1 * vec_per_row;
         }
-      };
-      int lm = 0, lj = 0, sm = 0, sj = 0;
-      u32x4 xv[XB];
-#pragma unroll
-      for (int r = 0; r < XB; ++r) {
-        xv[r] = x_load(lm, lj);
-        next(lm, lj);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int q = 0; q < NS; ++q) {
-        load_super(buf[q], pi, ss_begin + ps, chunk_base, ss_end);
-        advance(pi, ps);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int r = 0; r < XB; ++r) {
-        x_store(sm, sj, xv[r]);
-        next(sm, sj);
-      }
-      while (lm < M) {  // more rows than the first batch covers: eight requests at a time
-        u32x4 xw[8];
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          xw[r] = x_load(lm, lj);
-          next(lm, lj);
+        auto x_load_at = [&](int m, int kv) -> u32x4 {
+          const bool ok = m < M && kbase + kv * 8 < K;
+          return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
+        };
+        auto x_store_at = [&](int m, int kv, u32x4 v) {
+          if (m < M) *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = permute_x(v);
+        };
+        const u32x4 x0 = x_load_at(m0, kv0), x1 = x_load_at(m1, kv1);
+        __builtin_amdgcn_sched_barrier(0);
+        load_super(b0, 0, ss_begin, chunk_base, ss_end);
+        __builtin_amdgcn_sched_barrier(0);
+        x_store_at(m0, kv0, x0);
+        x_store_at(m1, kv1, x1);
+        for (int idx = tid + 2 * NT; idx < total; idx += 4 * NT) {
+          const u32x4 v0 = x_load(idx), v1 = x_load(idx + NT), v2 = x_load(idx + 2 * NT), v3 = x_load(idx + 3 * NT);
+          x_store(idx, v0);
+          x_store(idx + NT, v1);
+          x_store(idx + 2 * NT, v2);
+          x_store(idx + 3 * NT, v3);
         }
+      } else {
+        // more rows, and a phase of at most one vector per thread and row (launch_one checks): a thread
+        // stages its column of RM rows per batch.  No address needs a division (with the flat index the
+        // divisions alone cost half a microsecond at eight rows), the RM requests of the first batch are
+        // in flight together and all go out before the first weights.  (Measured alternatives, all
+        // slower: part of the batch behind the weights -- it returns after them, i.e. after a cold trip
+        // to HBM; sixteen in flight; requests under per-vector branches, which the wait-count
+        // insertion serialises.)
+        auto x_load = [&](int m, int kv) -> u32x4 {
+          const bool ok = m < M && kv < vec_per_row && kbase + kv * 8 < K;
+          return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
+        };
+        auto x_store = [&](int m, int kv, u32x4 v) {
+          if (m >= M || kv >= vec_per_row) return;
+          *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = permute_x(v);
+        };
+        auto stage = [&](auto rmc) {
+          constexpr int RM = decltype(rmc)::value;
+          u32x4 xv[RM];
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          x_store(sm, sj, xw[r]);
-          next(sm, sj);
-        }
+          for (int r = 0; r < RM; ++r) xv[r] = x_load(r, tid);
+          __builtin_amdgcn_sched_barrier(0);
+          load_super(b0, 0, ss_begin, chunk_base, ss_end);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int r = 0; r < RM; ++r) x_store(r, tid, xv[r]);
+          for (int m0 = RM; m0 < M; m0 += RM) {
+#pragma unroll
+            for (int r = 0; r < RM; ++r) xv[r] = x_load(m0 + r, tid);
+#pragma unroll
+            for (int r = 0; r < RM; ++r) x_store(m0 + r, tid, xv[r]);
+          }
+        };
+        if (M <= 4) stage(std::integral_constant<int, 4>{});
+        else stage(std::integral_constant<int, 8>{});
       }
-      // the slice is read back by this wavefront only: LDS serves a wavefront's accesses in order
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
     }
+    __syncthreads();
 
-    // Items past the end load zeros from an out-of-range offset and are neither multiplied nor flushed.
-    for (int j = 0; j < items; j += NS) {
-#pragma unroll
-      for (int q = 0; q < NS; ++q) {
-        if (j + q < items) {
-          compute_super(buf[q], cs);
-          if (cs == cnt - 1) flush_tile(ci, ph == 0);
-          advance(ci, cs);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        load_super(buf[q], pi, ss_begin + ps, chunk_base, ss_end);
-        advance(pi, ps);
-        __builtin_amdgcn_sched_barrier(0);
+    // ---- the weight stream: a flat software pipeline over (tile, super step) ----------
+    // Two items per trip, unconditionally (with an early exit in between, the compiler
+    // sinks the prefetch below the compute).  Items past the end load zeros from an
+    // out-of-range offset and are not flushed.
+    const int items = my_tiles * cnt;
+    int ci = 0, cs = 0;  // tile / local super step of the item being consumed
+    int pi = 0, ps = 0;  // ... of the item being prefetched
+    auto advance = [&](int& i, int& s) {
+      if (++s >= cnt) {
+        s = 0;
+        ++i;
       }
+    };
+    for (int j = 0; j < items; j += 2) {
+      advance(pi, ps);
+      load_super(b1, pi, ss_begin + ps, chunk_base, ss_end);
+      __builtin_amdgcn_sched_barrier(0);
+      compute_super(b0, ss_begin + cs);
+      if (cs == cnt - 1) flush_tile(ci, ph == 0);
+      advance(ci, cs);
+      __builtin_amdgcn_sched_barrier(0);
+      advance(pi, ps);
+      load_super(b0, pi, ss_begin + ps, chunk_base, ss_end);
+      __builtin_amdgcn_sched_barrier(0);
+      compute_super(b1, min(ss_begin + cs, nsuper - 1));
+      if (ci < my_tiles && cs == cnt - 1) flush_tile(ci, ph == 0);
+      advance(ci, cs);
+      __builtin_amdgcn_sched_barrier(0);
     }
     // a wavefront without work in this phase still owns slots that the epilogue sums
     if (cnt == 0 && ph == 0)
@@ -366,7 +400,17 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) sum += slots[((size_t)(i * WAVES + w) * 4 + r) * 64 + l];
-        store_out(a.ep, a.y, m, n, N, sum);
+        if (gated) {
+          // adjacent columns of the tile hold a gate / up pair: the even lane also sums its neighbour's
+          if ((l & 1) == 0 && n + 1 < N) {
+            float up = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) up += slots[((size_t)(i * WAVES + w) * 4 + r) * 64 + l + 1];
+            store_gated(a.y, m, n >> 1, N >> 1, sum, up);
+          }
+        } else {
+          store_out(a.ep, a.y, m, n, N, sum);
+        }
       }
     }
   } else {
@@ -375,6 +419,12 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     // the order of their K windows -- whoever arrives last, the sum is the same -- applies the
     // epilogue, stores, and returns the counter to zero for the next launch.  Nobody waits for anybody.
     //
+    // Ordering.  In the language's memory model the count would be a release (and, for the workgroup
+    // that arrives last, an acquire) at agent scope.  On this part both are cache-wide operations -- a
+    // write-back and an invalidate of a whole L2 -- and were measured: with acquire-release on the one
+    // counter add per workgroup a launch takes 2.8 - 4.9 us longer (4096 x 11008 at 8 rows: 11.3 -> 14.1 us,
+    // 5120 x 13824 int8 at batch 1: 18.0 -> 22.9 us), more than the split saves.  The exchange therefore
+    // relies on what the hardware guarantees for the accesses it actually makes:
     // Visibility across the chip's eight L2s without cache-wide fences (a device-scope fence writes
     // back and invalidates a whole L2; one per wavefront cost 65 us per launch): the partial tiles and
     // the counters are only ever touched by device-scope atomic stores, loads and adds, which are
@@ -488,27 +538,23 @@ int launch_one(const Problem& p, int group_shift, const Plan& plan, int ksplit =
   // zero -- then [tiles][ksplit][256] float partial tiles
   unsigned int* const counters = static_cast<unsigned int*>(workspace);
   float* const partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kSplitCounterBytes);
-  // builds of the kernel by the number of activation requests a lane makes ahead of its first weights
-  auto go = [&](auto xb) -> int {
-    constexpr int XB = decltype(xb)::value, NS = 2;
+  // two builds of the kernel, by the way the activations are staged: flat index / a column per thread
+  auto go = [&](auto rows) -> int {
+    constexpr bool ROWS = decltype(rows)::value;
     static std::atomic<bool> lds_ok[kMaxDevices];
-    if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, XB, NS, KSPLIT>, (int)kLdsPerWgMax,
+    if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT>, (int)kLdsPerWgMax,
                             lds_ok))
       return kFailed;
-    hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, XB, NS, KSPLIT>), dim3(plan.grid), dim3(WAVES * 64),
+    hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT>), dim3(plan.grid), dim3(WAVES * 64),
                        plan.lds_bytes, p.stream, a.x, a.wq, a.scales, a.M, a.N, a.K,
-                       a.group_shift | (a.zero_point << 8), a.max_tiles, a.phase_chunks, ksplit, plan.grid, a.y, a.ep, partials,
+                       a.group_shift | (a.zero_point << 8) | (p.activation == kActGated ? 1 << 16 : 0), a.max_tiles, a.phase_chunks, ksplit, plan.grid, a.y, a.ep, partials,
                        counters);
     return kLaunched;
   };
-  // requests a lane makes for its wavefront's slice of the activations: rows x ceil(vectors per row / 64)
   constexpr int ch = 128 / BITS;
-  const int pw_full = ((plan.phase_chunks + 4 * D - 1) / (4 * D) + WAVES - 1) / WAVES;
-  const int64_t requests = p.m * ((pw_full * (4 * D * ch / 8) + 63) / 64);
-  if (requests <= 1) return go(std::integral_constant<int, 1>{});
-  if (requests <= 2) return go(std::integral_constant<int, 2>{});
-  if (requests <= 4) return go(std::integral_constant<int, 4>{});
-  return go(std::integral_constant<int, 8>{});
+  const int phase_vectors = (plan.phase_chunks + 3) / 4 * 4 * ch / 8;  // 16-byte vectors per staged row
+  if (p.m <= 2 || phase_vectors > WAVES * 64) return go(std::false_type{});
+  return go(std::true_type{});
 }
 
 // D chunks per lane need K to be a multiple of 4*D chunks, and the lane's D
@@ -557,17 +603,16 @@ namespace {
 
 // The variants the default dispatch tries, in order (see launch_gemv).
 const int* default_order(const Problem& p) {
-  // Measured on MI355X (Llama-2-7B and 13B shapes, every variant on the same part): one 8-wavefront
-  // workgroup per CU is within 3 % of the best variant everywhere except one or two rows of int4
-  // weights with several row tiles per CU, where 4-wavefront workgroups -- each wavefront then walks a
-  // quarter of K instead of an eighth, i.e. twice the super steps per tile -- run ahead: four per CU
-  // from four tiles per CU on (22016 x 4096 at batch 1: 11.9 against 13.3 us), two per CU from two on
-  // (12288 x 4096: 8.0 against 8.2 us).  Two-chunk super steps first, single chunks (any K) as the fallback.
-  static const int wide[] = {42, 15, 14, 14}, mid[] = {22, 15, 14, 14}, other[] = {15, 14, 15, 14};
-  const int64_t tiles = (p.n + 15) / 16, cu = cu_count();
-  if (p.m <= 2 && p.bits == 4 && tiles >= 4 * cu) return wide;
-  if (p.m <= 2 && p.bits == 4 && tiles >= 2 * cu) return mid;
-  return other;
+  // Measured on MI355X (Llama-2-7B and 13B shapes): one or two rows of int4 weights run best with two
+  // 8-wave workgroups per CU (4096 x 11008 at batch 1: 8.7 against 9.3 us), everything else with one
+  // (12288 x 4096 at 4 rows: 8.7 against 9.0 us; int8 15360 x 5120 at batch 1: 18.2 against 19.6 us).
+  // Two-chunk super steps first, single chunks (any K) as the fallback.
+  static const int small[] = {25, 15, 24, 14}, large[] = {15, 14, 15, 14};
+  // (between one and two row tiles per CU a second workgroup per CU only unbalances them:
+  // 5120 x 5120, 9.9 against 8.7 us)
+  const int64_t tiles = (p.n + 15) / 16;
+  const bool fills = tiles <= cu_count() || tiles >= 2 * cu_count();
+  return (p.m <= 2 && p.bits == 4 && fills) ? small : large;
 }
 
 // Whether `variant` can be launched for p: K divisibility and an LDS plan (partial-tile slots of

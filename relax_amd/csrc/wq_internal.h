@@ -73,8 +73,9 @@ union mi355x_tvm_value;
 namespace wq {
 // mi355x_wq_packed_call; when `wq_tiled` is given, a matmul reads these tile-major copies instead of
 // the canonical tensors in the wq / scales slots (which are still validated and give N, K and group).
+// `library_scratch`: decode matmuls go through mi355x_wq_matmul_static_ws (K split on the library's scratch array).
 int packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes, int num_args,
-                             const void* wq_tiled, const void* scales_tiled);
+                             const void* wq_tiled, const void* scales_tiled, bool library_scratch = false);
 // Forwards the recorded error to TVM's error slot when the process has one; returns -1.
 int packed_fail();
 }  // namespace wq

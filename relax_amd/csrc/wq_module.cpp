@@ -222,7 +222,7 @@ bool validate(const char* symbol, const mi355x_wq_callspec* spec, const int32_t*
     wq::set_error("module: between 0 and %d constants, got %d", (int)kMaxConsts, num_consts);
     return false;
   }
-  if ((flags & ~MI355X_WQ_MODULE_TILE_WEIGHTS) != 0) {
+  if ((flags & ~(MI355X_WQ_MODULE_TILE_WEIGHTS | MI355X_WQ_MODULE_LIBRARY_SCRATCH)) != 0) {
     wq::set_error("module: unknown flags 0x%x", flags);
     return false;
   }
@@ -372,8 +372,12 @@ bool bind_constants(mi355x_wq_module* m, const mi355x_dl_tensor* const* consts, 
     return false;
   }
   if (d.n == 0) return true;
+  // The flag is a request, not a promise: where the tile-major layout is not defined for this
+  // (bits, group, K) -- e.g. int4 with K not a multiple of 256 -- the canonical constants stay bound
+  // and calls run on them, exactly as they would without the flag.
+  if (!wq::tiled_layout_defined(d.bits, d.group, d.k)) return true;
   int64_t wq_bytes = 0, sc_bytes = 0;
-  if (mi355x_wq_tiled_sizes(&d, &wq_bytes, &sc_bytes) != 0) return false;  // no tile-major layout for this (bits, group, K)
+  if (mi355x_wq_tiled_sizes(&d, &wq_bytes, &sc_bytes) != 0) return false;
   if (!hip_ok(hipMalloc(&m->wq_tiled, wq_bytes), "hipMalloc") || !hip_ok(hipMalloc(&m->scales_tiled, sc_bytes), "hipMalloc"))
     return false;
   const void* pw = static_cast<const char*>(tw.data) + tw.byte_offset;
@@ -529,7 +533,8 @@ int mi355x_wq_module_call(mi355x_wq_module* mod, mi355x_tvm_value* args, int* ty
       ++next;
     }
   }
-  return wq::packed_call_with_weights(&mod->spec, full, codes, total, mod->wq_tiled, mod->scales_tiled);
+  return wq::packed_call_with_weights(&mod->spec, full, codes, total, mod->wq_tiled, mod->scales_tiled,
+                                      (mod->flags & MI355X_WQ_MODULE_LIBRARY_SCRATCH) != 0);
 }
 
 int64_t mi355x_wq_module_save_to_binary(const mi355x_wq_module* mod, void* buffer, int64_t capacity) {

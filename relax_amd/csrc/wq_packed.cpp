@@ -128,12 +128,17 @@ int mi355x_wq_packed_call(const mi355x_wq_callspec* spec, mi355x_tvm_value* args
   return wq::packed_call_with_weights(spec, args, type_codes, num_args, nullptr, nullptr);
 }
 
+int mi355x_wq_packed_call_scratch(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes,
+                                  int num_args) {
+  return wq::packed_call_with_weights(spec, args, type_codes, num_args, nullptr, nullptr, true);
+}
+
 }  // extern "C"
 
 int wq::packed_fail() { return fail(); }
 
 int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes,
-                                 int num_args, const void* wq_tiled, const void* scales_tiled) {
+                                 int num_args, const void* wq_tiled, const void* scales_tiled, bool library_scratch) {
   if (spec == nullptr) {
     wq::set_error("call spec is NULL");
     return fail();
@@ -218,9 +223,16 @@ int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_valu
                     (long long)d.k);
       return fail();
     }
-    if (to->shape[0] != m || to->shape[1] != d.n) {
+    // the gated tail halves the output: y[M, N/2] = multiply(nn.silu(gate), up)
+    const bool gated_out = spec->activation == MI355X_WQ_ACT_SILU_MUL;
+    if (gated_out && d.n % 2 != 0) {
+      wq::set_error("the gated tail (silu_mul) needs an even N, got %lld", (long long)d.n);
+      return fail();
+    }
+    const int64_t out_cols = gated_out ? d.n / 2 : d.n;
+    if (to->shape[0] != m || to->shape[1] != out_cols) {
       wq::set_error("y has shape (%lld, %lld), expected (%lld, %lld)", (long long)to->shape[0],
-                    (long long)to->shape[1], (long long)m, (long long)d.n);
+                    (long long)to->shape[1], (long long)m, (long long)out_cols);
       return fail();
     }
   } else if (to->shape[0] != d.n || to->shape[1] != d.k) {
@@ -268,6 +280,12 @@ int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_valu
     wq::set_error("tensors live on ROCm device %d but the current HIP device is %d", dev, cur);
     return fail();
   }
+  if (library_scratch && is_matmul) {
+    // decode calls may split K across workgroups on the library's own scratch array (no allocation)
+    const bool tiled = wq_tiled != nullptr;
+    return mi355x_wq_matmul_static_ws(&d, px, tiled ? wq_tiled : pw, tiled ? scales_tiled : ps, &ep, po, m, g_stream,
+                                      tiled ? 1 : 0) == 0 ? 0 : fail();
+  }
   if (wq_tiled != nullptr && is_matmul)
     return mi355x_wq_matmul_tiled(&d, px, wq_tiled, scales_tiled, &ep, po, m, g_stream) == 0 ? 0 : fail();
   const int rc = is_matmul ? mi355x_wq_matmul_fused(&d, px, pw, ps, &ep, po, m, g_stream)
@@ -294,6 +312,8 @@ MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_bias_relu, 0, 4, 7, 1, 0, MI355X_WQ_ACT_R
 MI355X_FIXED_ENTRY(mi355x_q8f16_matmul_bias_relu, 0, 8, 0, 1, 0, MI355X_WQ_ACT_RELU)
 MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_residual, 0, 4, 7, 0, 1, 0)
 MI355X_FIXED_ENTRY(mi355x_q8f16_matmul_residual, 0, 8, 0, 0, 1, 0)
+MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_silu_mul, 0, 4, 7, 0, 0, MI355X_WQ_ACT_SILU_MUL)
+MI355X_FIXED_ENTRY(mi355x_q8f16_matmul_silu_mul, 0, 8, 0, 0, 0, MI355X_WQ_ACT_SILU_MUL)
 MI355X_FIXED_ENTRY(mi355x_q4f16_dequantize, 1, 4, 7, 0, 0, 0)
 MI355X_FIXED_ENTRY(mi355x_q8f16_dequantize, 1, 8, 0, 0, 0, 0)
 #undef MI355X_FIXED_ENTRY
@@ -462,6 +482,8 @@ int mi355x_wq_register_tvm_globals(int allow_override) {
                            {"mi355x.q8f16_matmul_bias_relu", mi355x_q8f16_matmul_bias_relu},
                            {"mi355x.q4f16_matmul_residual", mi355x_q4f16_matmul_residual},
                            {"mi355x.q8f16_matmul_residual", mi355x_q8f16_matmul_residual},
+                           {"mi355x.q4f16_matmul_silu_mul", mi355x_q4f16_matmul_silu_mul},
+                           {"mi355x.q8f16_matmul_silu_mul", mi355x_q8f16_matmul_silu_mul},
                            {"mi355x.q4f16_dequantize", mi355x_q4f16_dequantize},
                            {"mi355x.q8f16_dequantize", mi355x_q8f16_dequantize},
                            {"mi355x.q4f16_tile_weights", mi355x_q4f16_tile_weights},

@@ -9,8 +9,8 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 SO_PATH = os.path.join(CSRC, "libmi355x_wq.so")
 
 KERNEL_AUTO, KERNEL_GEMV, KERNEL_GEMM, KERNEL_SKINNY = 0, 1, 2, 3
-ACT_NONE, ACT_RELU = 0, 1
-ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "relax.nn.relu": ACT_RELU}
+ACT_NONE, ACT_RELU, ACT_SILU_MUL = 0, 1, 2
+ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "relax.nn.relu": ACT_RELU, "silu_mul": ACT_SILU_MUL}
 
 # every symbol include/mi355x_wq.h, include/mi355x_wq_packed.h and include/mi355x_wq_module.h declare
 EXPORTED_SYMBOLS = (
@@ -21,10 +21,10 @@ EXPORTED_SYMBOLS = (
     "mi355x_wq_select_kernel", "mi355x_wq_last_error", "mi355x_wq_version",
     "mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_matmul_bias", "mi355x_q8f16_matmul_bias",
     "mi355x_q4f16_matmul_bias_relu", "mi355x_q8f16_matmul_bias_relu", "mi355x_q4f16_matmul_residual",
-    "mi355x_q8f16_matmul_residual", "mi355x_q4f16_dequantize",
+    "mi355x_q8f16_matmul_residual", "mi355x_q4f16_matmul_silu_mul", "mi355x_q8f16_matmul_silu_mul", "mi355x_q4f16_dequantize",
     "mi355x_q8f16_dequantize", "mi355x_q4f16_tile_weights", "mi355x_q8f16_tile_weights",
     "mi355x_q4f16_matmul_tiled", "mi355x_q8f16_matmul_tiled", "mi355x_q4f16_matmul_ws", "mi355x_q8f16_matmul_ws",
-    "mi355x_wq_packed_call", "mi355x_wq_packed_set_stream",
+    "mi355x_wq_packed_call", "mi355x_wq_packed_call_scratch", "mi355x_wq_packed_set_stream",
     "mi355x_wq_packed_get_stream", "mi355x_wq_register_tvm_globals",
     "mi355x_wq_module_type_key", "mi355x_wq_module_create", "mi355x_wq_module_destroy", "mi355x_wq_module_symbol",
     "mi355x_wq_module_num_consts", "mi355x_wq_module_const_name", "mi355x_wq_module_json",
@@ -101,6 +101,7 @@ def load() -> C.CDLL:
     for name in PACKED_ENTRIES:
         getattr(L, name).argtypes = [vp, C.POINTER(ci), ci, vp, C.POINTER(ci), vp]
     L.mi355x_wq_packed_call.argtypes = [vp, vp, C.POINTER(ci), ci]
+    L.mi355x_wq_packed_call_scratch.argtypes = [vp, vp, C.POINTER(ci), ci]
     i32 = C.c_int32
     L.mi355x_wq_module_type_key.restype = C.c_char_p
     L.mi355x_wq_module_create.argtypes = [C.c_char_p, vp, C.POINTER(C.c_char_p), C.POINTER(i32), i32, i32, C.POINTER(vp)]

@@ -29,6 +29,7 @@ from . import lib as _lib
 from .vm_harness import (K_TVM_NDARRAY_HANDLE, K_TVM_NULLPTR, CallSpec, PackedError, TensorArg, TVMValue)
 
 TILE_WEIGHTS = 1
+LIBRARY_SCRATCH = 2
 ND_ARRAY_MAGIC = 0xDD5E40F096B4A13F  # kTVMNDArrayMagic, include/tvm/runtime/ndarray.h:447
 _PACKED_CFUNC = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_void_p, C.c_void_p)
 

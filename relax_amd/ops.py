@@ -26,7 +26,8 @@ def wq_matmul(x: torch.Tensor, wq: torch.Tensor, scales: torch.Tensor, bits: int
     """y[M,N] = f16(x[M,K] @ dequant(wq, scales)^T) on the current HIP device (asynchronous).
 
     Optional fused epilogue, each step one float16 operation: ``+ bias[N]``, then ``activation``
-    ("relu"), then ``+ residual[M,N]`` (``residual`` may be ``out`` itself).
+    ("relu"), then ``+ residual[M,N]`` (``residual`` may be ``out`` itself); or ``activation="silu_mul"``
+    alone: the output is ``[M, N/2] = multiply(nn.silu(y[:, :N/2]), y[:, N/2:])``.
 
     ``tiled_n=N``: ``wq`` and ``scales`` are the tile-major buffers `wq_tile_weights` returns
     for an N-row matrix (their row count is N rounded up to 16).
@@ -55,10 +56,12 @@ def wq_matmul(x: torch.Tensor, wq: torch.Tensor, scales: torch.Tensor, bits: int
         raise ValueError(f"wq has {wq.shape[1]} words per row, expected {k * bits // 32} for K={k}")
     if tuple(scales.shape) != (n, k // group):
         raise ValueError(f"scales has shape {tuple(scales.shape)}, expected {(n, k // group)}")
+    # the gated tail ("silu_mul": multiply(nn.silu(gate), up) on the two halves of a gate+up projection) halves the output
+    out_cols = n // 2 if activation == "silu_mul" else n
     if out is None:
-        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
-    elif tuple(out.shape) != (m, n) or out.dtype != torch.float16 or not out.is_contiguous():
-        raise ValueError("out must be a compact float16 [M, N] tensor")
+        out = torch.empty((m, out_cols), dtype=torch.float16, device=x.device)
+    elif tuple(out.shape) != (m, out_cols) or out.dtype != torch.float16 or not out.is_contiguous():
+        raise ValueError(f"out must be a compact float16 [{m}, {out_cols}] tensor")
     desc = _lib.make_desc(bits, group, n, k, zero_point)
     if bias is None and residual is None and activation is None:
         rc = L.mi355x_wq_matmul_ex(desc, x.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(),

@@ -15,6 +15,12 @@ activation)` describes for its CUTLASS backend (python/tvm/relax/dpl/pattern.py:
     y = R.nn.relu(y)
     y = R.add(y, residual)        # residual [M, N]
 
+or by the gated tail of a Llama MLP, whose gate and up projections share one weight matrix (gate rows,
+then as many up rows):
+
+    sp  = R.split(y, 2, axis=-1)
+    out = R.multiply(R.nn.silu(sp[0]), sp[1])      # [M, N/2]
+
 `matmul(x, permute_dims(W))` is what `relax.op.linear` expands to
 (python/tvm/relax/op/linear_algebra.py:54-90).  The pattern name's prefix before the
 first "." becomes the `Codegen` attribute, i.e. the backend name
@@ -36,13 +42,16 @@ DECODE_FUNCS = {
 
 def patterns():
     """[(name, DFPattern)] for FuseOpsByPattern(patterns, annotate_codegen=True)."""
-    from tvm.relax.dpl import is_call_tir, is_op, wildcard  # python/tvm/relax/dpl/pattern.py:678-837
+    from tvm.relax.dpl import is_call_tir, is_op, is_tuple_get_item, wildcard  # python/tvm/relax/dpl/pattern.py:678-837
 
     def core(fn_name):
+        # Only the float32-accumulating form is taken: with out_dtype "" or "float16" the CPU path
+        # accumulates in float16 (python/tvm/relax/transform/legalize_ops.py:250-258), which the kernels
+        # do not reproduce.  A string matches a DataType attribute (src/relax/ir/dataflow_matcher.cc:128-133).
         decoded = is_call_tir(fn_name, [wildcard(), wildcard()])
         weight_t = is_op("relax.permute_dims")(decoded)
-        mm = is_op("relax.matmul")(wildcard(), weight_t)
-        return is_op("relax.astype")(mm)
+        mm = is_op("relax.matmul")(wildcard().has_dtype("float16"), weight_t).has_attr({"out_dtype": "float32"})
+        return is_op("relax.astype")(mm).has_attr({"dtype": "float16"})
 
     # Longest tail first: earlier entries have priority (transform.py:337-339).  A pattern cannot
     # tell a [N] bias from a [M, N] residual (no shape predicate without concrete extents); the
@@ -52,6 +61,10 @@ def patterns():
         base = f"{BACKEND}.q{q['bits']}f16_matmul"
         add1 = lambda: is_op("relax.add")(core(fn_name), wildcard())  # noqa: E731
         relu = lambda: is_op("relax.nn.relu")(add1())                 # noqa: E731
+        halves = lambda: is_op("relax.split")(core(fn_name)).has_attr({"indices_or_sections": 2})  # noqa: E731
+        gated = is_op("relax.multiply")(is_op("relax.nn.silu")(is_tuple_get_item(halves(), 0)),
+                                        is_tuple_get_item(halves(), 1))
+        table.append((base + "_silu_mul", gated))
         table.append((base + "_add_relu_add", is_op("relax.add")(relu(), wildcard())))
         table.append((base + "_add_add", is_op("relax.add")(add1(), wildcard())))
         table.append((base + "_add_relu", relu()))

@@ -113,7 +113,9 @@ def call_packed(symbol, args, *, type_code: int = K_TVM_NDARRAY_HANDLE, spec: Ca
             values[i].v_int64 = int(a)
             codes[i] = 0
     if spec is not None:
-        rc = L.mi355x_wq_packed_call(C.addressof(spec), C.addressof(values), codes, n)
+        # the body generated entries forward to: mi355x_wq_packed_call, or its _scratch twin by name
+        forward = L.mi355x_wq_packed_call_scratch if symbol == "mi355x_wq_packed_call_scratch" else L.mi355x_wq_packed_call
+        rc = forward(C.addressof(spec), C.addressof(values), codes, n)
     else:
         fn = getattr(L, symbol)
         ret_value = TVMValue()

@@ -5,7 +5,7 @@
 
 typedef int (*packed_cfunc)(void* args, int* type_codes, int num_args, void* ret, void* resource);
 
-#define MAX_FUNCS 16
+#define MAX_FUNCS 32
 static struct { char name[64]; packed_cfunc fn; void* resource; } g_funcs[MAX_FUNCS];
 static int g_count = 0;
 static char g_last_error[512] = "";

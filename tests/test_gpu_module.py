@@ -213,3 +213,61 @@ def test_empty_batch_and_empty_projection():
                                   torch.empty((0, 8), dtype=torch.float16, device="cuda"))
     none.get_function("e")(_dev(x), torch.empty((2, 0), dtype=torch.float16, device="cuda"))
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("bits, n, k, group", [(4, 200, 352, None), (4, 96, 96, None), (8, 136, 320, 64)])
+def test_tile_weights_flag_where_the_layout_is_not_defined(bits, n, k, group):
+    """The flag is a request: for a (bits, group, K) without a tile-major layout (int4 with K % 256 != 0,
+    group sizes other than 32 / 128) init keeps the canonical constants and calls run on them."""
+    vm_harness.set_stream()
+    for m in (1, 8, 70):
+        x, wq, s, g = O.make_case(41, m, n, k, bits, group)
+        assert lib.load().mi355x_wq_tiled_sizes(lib.make_desc(bits, g, n, k), None, None) == -1
+        mod = M.SubgraphModule.create("f", spec_for(bits, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1], M.TILE_WEIGHTS)
+        mod.get_function("__init_f")(wq, s)  # host constants, as after load_module
+        assert mod.initialized
+        y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+        mod.get_function("f")(_dev(x), y)
+        torch.cuda.synchronize()
+        assert torch.equal(y, plain(bits, _dev(x), _dev(wq), _dev(s)))
+        assert_close(y.cpu().numpy(), c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=8), (bits, m, n, k))
+        mod.close()
+
+
+def test_library_scratch_flag_and_packed_call_scratch():
+    """MI355X_WQ_MODULE_LIBRARY_SCRATCH / mi355x_wq_packed_call_scratch: decode calls may split K on the
+    library's scratch array; results equal the caller-workspace entry bit for bit, also on tile-major weights,
+    and the module survives export -> load with the flag."""
+    import relax_amd
+
+    vm_harness.set_stream()
+    bits, m, n, k = 8, 16, 5120, 13824
+    x, wq, s, g = O.make_case(42, m, n, k, bits)
+    dx, dw, ds = _dev(x), _dev(wq), _dev(s)
+    need = relax_amd.wq_workspace_bytes(bits, g, n, k, m)
+    assert need > 0
+    want = relax_amd.wq_matmul(dx, dw, ds, bits, g, workspace=relax_amd.wq_workspace(need))
+    for flags in (M.LIBRARY_SCRATCH, M.LIBRARY_SCRATCH | M.TILE_WEIGHTS):
+        mod = M.SubgraphModule.create("f", spec_for(bits, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1], flags)
+        mod, _ = M.SubgraphModule.load_from_binary(mod.save_to_binary())
+        mod.get_function("__init_f")(dw, ds)
+        y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+        mod.get_function("f")(dx, y)
+        torch.cuda.synchronize()
+        if flags & M.TILE_WEIGHTS:
+            wt, st = relax_amd.wq_tile_weights(dw, ds, bits, g)
+            need_t = relax_amd.wq_workspace_bytes(bits, g, n, k, m, tiled=True)
+            ref = relax_amd.wq_matmul(dx, wt, st, bits, g, tiled_n=n, workspace=relax_amd.wq_workspace(max(need_t, 16)))
+            torch.cuda.synchronize()
+            assert torch.equal(y.view(torch.int16), ref.view(torch.int16))
+        else:
+            assert torch.equal(y.view(torch.int16), want.view(torch.int16))
+        assert_close(y.cpu().numpy(), c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16), ("scratch", flags))
+        mod.close()
+    # the generated entries' forwarding function, called directly
+    spec = spec_for(bits, ("x", "wq", "scales", "out"))
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    targs = [vm_harness.TensorArg(t, as_uint32=(t.dtype == torch.int32)) for t in (dx, dw, ds, y)]
+    vm_harness.call_packed("mi355x_wq_packed_call_scratch", targs, spec=spec)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), want.view(torch.int16))

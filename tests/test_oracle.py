@@ -384,3 +384,91 @@ def test_tile_major_layout_definition_and_round_trip(bits, n, k):
     assert np.array_equal(w2, wq) and np.array_equal(s2.view(np.uint16), s.view(np.uint16))
     wpad, spad = O.untile_weights(wt, st, bits, rows)
     assert not wpad[n:].any() and not spad[n:].any()
+
+
+# ---------------------------------------------------------------- gated tail: multiply(nn.silu(gate), up)
+def _silu_both(g, u):
+    y = np.concatenate([np.asarray(g, dtype=np.float16).reshape(1, -1), np.asarray(u, dtype=np.float16).reshape(1, -1)], axis=1)
+    return O.epilogue(y, activation="silu_mul")[0], c_oracle.epilogue(y, activation="silu_mul")[0]
+
+
+def test_silu_mul_known_answers_and_special_values():
+    """Values the float16 operation sequence fixes by hand: silu(0) = 0; a large gate passes through
+    (exp(-g) rounds to 0, 1 / 1 = 1); a gate of -20 gives exp(20) = inf in float16, 1 / inf = 0, -20 * 0 = -0;
+    gate 1: e = f16(exp(-1)) = 0.36792, d = f16(1.36792) = 1.3682, s = f16(1 / 1.3682) = 0.73096, t = 0.73096."""
+    g = np.array([0.0, 12.0, -20.0, 1.0, 1.0, -np.inf, np.inf, np.nan], dtype=np.float16)
+    u = np.array([3.0, 0.5, 2.0, 1.0, -2.0, 1.0, 2.0, 1.0], dtype=np.float16)
+    for got in _silu_both(g, u):
+        assert got[0] == 0 and not np.signbit(got[0])
+        assert got[1] == np.float16(6.0)
+        assert got[2] == 0 and np.signbit(got[2])                     # -20 * (+0) = -0, times 2
+        assert got[3].view(np.uint16) == np.float16(0.73096).view(np.uint16)
+        assert got[4].view(np.uint16) == np.float16(-1.4619).view(np.uint16)
+        assert np.isnan(got[5])                                       # -inf * 0
+        assert got[6] == np.inf and np.isnan(got[7])
+
+
+def test_silu_mul_both_restatements_agree_on_every_gate_value():
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16)
+    for u in (1.0, -0.37, 23.5, 6.1e-5):
+        a, b = _silu_both(halves, np.full(65536, u, dtype=np.float16))
+        assert _bits_equal_nan_aware(a, b), u
+
+
+def test_silu_mul_tracks_the_float64_closed_form():
+    """g / (1 + exp(-g)) * u in float64 against the five-rounding float16 sequence: every result within
+    6 float16 ulp (five roundings of half an ulp each, and an ulp is between 2^-11 and 2^-10 of its value, so
+    errors carried across a power of two count double) -- a dropped term, a wrong sign or sigmoid in place of
+    silu is off by orders of magnitude more."""
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16)
+    # beyond |g| = 8 the sequence leaves the normal float16 range (1 / (1 + exp(9.7)) is subnormal, exp(11.1) overflows)
+    # and below |g| = 2^-12 the product g * s is subnormal
+    mag = np.abs(halves.astype(np.float64))
+    g = halves[np.isfinite(halves) & (mag <= 8.0) & (mag >= 2.0 ** -12)]
+    worst = 0.0
+    for u in (1.0, -0.37, 23.5):
+        got, _ = _silu_both(g, np.full(g.size, u, dtype=np.float16))
+        g64 = g.astype(np.float64)
+        exact = g64 / (1.0 + np.exp(-g64)) * np.float64(np.float16(u))
+        ulp = np.maximum(np.spacing(np.abs(exact).astype(np.float16)).astype(np.float64), 2.0 ** -24)
+        err = np.abs(got.astype(np.float64) - exact) / ulp
+        worst = max(worst, float(err.max()))
+    assert worst <= 6.0, worst
+
+
+def test_silu_mul_every_step_against_exact_rationals():
+    """Each of the four arithmetic steps (1 + e, 1 / d, g * s, t * u) rounded independently: exact fractions
+    and a nearest-even search in the table of all float16 values; exp(-g) in float16 comes from `math.exp`
+    (double precision) rounded by the same search."""
+    import bisect
+    import math
+    from fractions import Fraction
+
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16)
+    finite = halves[np.isfinite(halves) & ~((halves == 0) & np.signbit(halves))]
+    table = finite[np.argsort(finite.astype(np.float64), kind="stable")]
+    fracs = [Fraction(float(h)) for h in table]
+
+    def nearest(fr):
+        assert abs(fr) < 65520
+        i = bisect.bisect_left(fracs, fr)
+        cands = [j for j in (i - 1, i) if 0 <= j < len(fracs)]
+        dist = [abs(fracs[j] - fr) for j in cands]
+        if len(cands) == 2 and dist[0] == dist[1]:
+            j = cands[0] if (int(table[cands[0]].view(np.uint16)) & 1) == 0 else cands[1]
+        else:
+            j = cands[int(np.argmin(dist))]
+        return Fraction(float(table[j]))
+
+    rng = np.random.default_rng(7)
+    g = (rng.standard_normal(1500) * 3).astype(np.float16)
+    u = (rng.standard_normal(1500) * 2).astype(np.float16)
+    got_np, got_c = _silu_both(g, u)
+    for i in range(g.size):
+        gf, uf = Fraction(float(g[i])), Fraction(float(u[i]))
+        e = nearest(Fraction(math.exp(-float(g[i]))))
+        d = nearest(1 + e)
+        s = nearest(1 / d)
+        t = nearest(gf * s)
+        want = nearest(t * uf)
+        assert Fraction(float(got_np[i])) == want and Fraction(float(got_c[i])) == want, (g[i], u[i])

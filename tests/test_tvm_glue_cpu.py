@@ -215,7 +215,7 @@ def test_bound_weights_give_a_module_plan(fake_tvm):
     from relax_amd.vm_harness import CallSpec as CSpec
 
     n = 48
-    f = fake_tvm.quantized_linear(bound=("wq", "scales"))
+    f = fake_tvm.quantized_linear(bound=("wq", "scales"), k=256)
     assert [p.name_hint for p in f.params] == ["x_outer"]
     with pytest.raises(ValueError, match="use module_plan"):
         spec_from_function(f)
@@ -233,6 +233,15 @@ def test_bound_weights_give_a_module_plan(fake_tvm):
     assert plan.const_args == (0, 1, 2) and len(plan.const_names) == 3
     assert (s.bits, s.arg_wq, s.arg_scales, s.arg_bias, s.arg_x, s.arg_residual, s.arg_out, s.activation) == \
         (8, 0, 1, 2, 3, 4, 5, ACT_RELU)
+    # K for which the tile-major layout is not defined (int4 needs K % 256 == 0): the canonical constants
+    # stay, the module still loads (the flag is only set where the conversion exists)
+    for k in (128, 352):
+        f = fake_tvm.quantized_linear(bound=("wq", "scales"), k=k)
+        assert module_plan(f, constants_of(f)).flags == 0
+    f = fake_tvm.quantized_linear("decode_q8f16", bound=("wq", "scales"), k=384)  # int8: K % 128 == 0 suffices
+    assert module_plan(f, constants_of(f)).flags == MODULE_TILE_WEIGHTS
+    f = fake_tvm.quantized_linear(bound=("wq", "scales"), k=256)
+    assert module_plan(f, constants_of(f), tile_weights=False).flags == 0
     # only the weights bound, scales a parameter: no tile-major conversion (it needs both)
     f = fake_tvm.quantized_linear(bound=("wq",))
     plan = module_plan(f, constants_of(f))
@@ -254,3 +263,149 @@ def test_bound_weights_give_a_module_plan(fake_tvm):
     f = fake_tvm.quantized_linear(tail=[("add", [4, n])], bound=("wq", "scales", "operand0"))
     with pytest.raises(ValueError, match="residual of the composite is a constant"):
         module_plan(f, constants_of(f))
+
+
+# ---------------------------------------------------------------- fixtures in the shape of the reference's goldens
+def test_annotated_function_in_the_shape_of_the_reference_golden(fake_tvm):
+    """tests/python/relax/test_transform_fuse_ops_by_pattern.py:41-81 (Conv2dReLU_composite_annotated) with the
+    operators swapped for decode / permute_dims / matmul / astype: outer function with Codegen and
+    global_symbol, a local Primitive + Composite function whose body is one dataflow block, parameters in
+    first-use order, the symbol built from the callee names."""
+    from relax_amd.tvm_glue.codegen import ACT_NONE, _derive_roles, spec_from_function
+
+    symbol = fake_tvm.fused_name("decode_q4f16") + "_mi355x"
+    assert symbol == SYM  # fused + callee names (fuse_ops.cc:370-395), dots -> underscores, + "_" + backend (:1009)
+    f = fake_tvm.quantized_linear(symbol=symbol, golden_names=True)
+    # the golden's structure
+    assert f.attrs == {"Codegen": "mi355x", "global_symbol": symbol}
+    local_binding, call_binding = f.body.blocks[0].bindings
+    composite = local_binding.value
+    assert composite.attrs == {"Primitive": 1, "Composite": "mi355x.q4f16_matmul"}
+    assert isinstance(composite.body.blocks[0], fake_tvm.DataflowBlock) and len(composite.body.blocks) == 1
+    assert call_binding.value.op is local_binding.var and f.body.body is call_binding.var
+    # first-use order of the grouped bindings: decode's tuple (wq, scales), then matmul's x
+    assert [p.name_hint for p in composite.params] == ["wq", "s", "x"]
+    assert [p.name_hint for p in f.params] == ["wq1", "s1", "x1"]
+    decode, act, roles, outer = _derive_roles(f)
+    assert decode == "decode_q4f16" and act == ACT_NONE and len(outer) == 3
+    assert roles == {"wq": ("param", 0), "scales": ("param", 1), "x": ("param", 2)}
+    s = spec_from_function(f)
+    assert (s.arg_wq, s.arg_scales, s.arg_x, s.arg_out, s.num_args) == (0, 1, 2, 3, 4)
+    # the q8 flavour and a fused tail get their own names
+    assert fake_tvm.fused_name("decode_q8f16", [("add", [48]), ("relu",)]) == \
+        "fused_decode_q8f16_relax_permute_dims_relax_matmul_relax_astype_relax_add_relax_nn_relu"
+
+
+def test_call_form_after_run_codegen_matches_the_call_description(fake_tvm):
+    """tests/python/relax/test_transform_codegen_pass.py:184-251: RunCodegen turns every call of the annotated
+    function into call_tir(ExternFunc(symbol), (the call's own arguments), out_sinfo), one extern for repeated
+    calls; the lowered call appends the output (call_tir_rewrite.cc:94-110).  The call description must
+    address exactly that argument list."""
+    from relax_amd.tvm_glue.codegen import spec_from_function, trampoline_source
+
+    symbol = fake_tvm.fused_name("decode_q4f16") + "_mi355x"
+    f = fake_tvm.quantized_linear(symbol=symbol, golden_names=True, m=16, n=32, k=64)
+    spec = spec_from_function(f)
+    wq1, s1, data = fake_tvm.Var("weight1"), fake_tvm.Var("scale1"), fake_tvm.Var("data")
+    wq2, s2 = fake_tvm.Var("weight2"), fake_tvm.Var("scale2")
+    lv = fake_tvm.partitioned_main(symbol, (wq1, s1, data), [16, 32])
+    gv = fake_tvm.partitioned_main(symbol, (wq2, s2, fake_tvm.Var("lv")), [16, 32])
+    for call in (lv, gv):
+        assert call.args[0].global_symbol == symbol                 # the same extern for both calls
+        args = call.args[1].fields
+        assert len(args) + 1 == spec.num_args and spec.arg_out == len(args)
+        assert args[spec.arg_wq].name_hint.startswith("weight") and args[spec.arg_scales].name_hint.startswith("scale")
+        assert args[spec.arg_x].name_hint in ("data", "lv")
+        assert call.sinfo_args[0].shape == [16, 32] and call.sinfo_args[0].dtype == "float16"
+    # one generated entry serves both calls
+    assert trampoline_source([(symbol, spec)]).count("int " + symbol + "(") == 1
+
+
+def test_bound_constants_stay_inside_the_composite(fake_tvm):
+    """tests/python/relax/test_transform_fuse_ops_by_pattern.py:432-446: after BindParams the weight is a
+    relax.Constant argument of the operator inside the fused function, not a parameter."""
+    f = fake_tvm.quantized_linear(bound=("wq", "scales"), golden_names=True, k=256)
+    composite = f.body.blocks[0].bindings[0].value
+    decode_call = composite.body.blocks[0].bindings[0].value
+    wq, scales = decode_call.args[1].fields
+    assert isinstance(wq, fake_tvm.Constant) and isinstance(scales, fake_tvm.Constant)
+    assert [p.name_hint for p in composite.params] == ["x"] and [p.name_hint for p in f.params] == ["x1"]
+
+
+@pytest.mark.parametrize("kwargs,message", [
+    (dict(out_dtype=""), "out_dtype float32"),             # float16 accumulation on the CPU path
+    (dict(out_dtype="float16"), "out_dtype float32"),
+    (dict(astype_dtype="float32"), "must produce float16"),
+    (dict(axes=[0, 1]), "2-d transpose"),
+    (dict(x_shape=[2, 4, 128]), "x must be a 2-d tensor"),
+    (dict(x_dtype="float32"), "x must be float16"),
+])
+def test_role_derivation_rejects_composites_the_kernels_do_not_compute(fake_tvm, kwargs, message):
+    from relax_amd.tvm_glue.codegen import spec_from_function
+
+    with pytest.raises(ValueError, match=message):
+        spec_from_function(fake_tvm.quantized_linear(**kwargs))
+
+
+def test_role_derivation_accepts_the_explicit_transpose_and_checks_operand_types(fake_tvm):
+    from relax_amd.tvm_glue.codegen import spec_from_function
+
+    assert spec_from_function(fake_tvm.quantized_linear(axes=[1, 0])).arg_x == 2
+    f = fake_tvm.quantized_linear()
+    decode_call = f.body.blocks[0].bindings[0].value.body.blocks[0].bindings[0].value
+    decode_call.args[1].fields[0].struct_info.dtype = "int32"
+    with pytest.raises(ValueError, match="packed weights must be uint32"):
+        spec_from_function(f)
+
+
+def test_hook_honours_its_options(fake_tvm, monkeypatch):
+    """RunCodegen hands the hook a per-backend options map (src/relax/transform/run_codegen.cc:155-162)."""
+    import sys
+
+    from relax_amd.tvm_glue import codegen
+
+    created = []
+    registry = {
+        "relax.ext.mi355x.create_module": lambda *a: created.append(("module",) + a) or ("module", a[0]),
+        "runtime.CSourceModuleCreate": lambda *a: created.append(("csource",) + a) or ("csource", a[2]),
+    }
+    monkeypatch.setattr(sys.modules["tvm"], "get_global_func", lambda name: registry[name], raising=False)
+    bound = fake_tvm.quantized_linear(bound=("wq", "scales"), k=256, symbol="bound_mi355x")
+    free = fake_tvm.quantized_linear(symbol="free_mi355x")
+    names = constants_of(bound)
+    # defaults: tile-major conversion on, no scratch
+    mods = codegen.relax_ext_mi355x([bound, free], None, names)
+    assert [m[0] for m in mods] == ["module", "csource"]
+    assert created[0][-1] == codegen.MODULE_TILE_WEIGHTS and "mi355x_wq_packed_call(&spec" in created[1][1]
+    created.clear()
+    codegen.relax_ext_mi355x([bound, free], {"tile_weights": False, "workspace": True}, names)
+    assert created[0][-1] == codegen.MODULE_LIBRARY_SCRATCH
+    assert "mi355x_wq_packed_call_scratch(&spec" in created[1][1] and created[1][3] == ["free_mi355x"]
+    created.clear()
+    codegen.relax_ext_mi355x([bound], {"workspace": 1}, names)  # integers as TVM passes them
+    assert created[0][-1] == codegen.MODULE_TILE_WEIGHTS | codegen.MODULE_LIBRARY_SCRATCH
+    with pytest.raises(ValueError, match="unknown option 'tile_weight'"):
+        codegen.relax_ext_mi355x([free], {"tile_weight": True}, {})
+
+
+def test_gated_tail_of_a_gate_up_projection(fake_tvm):
+    """multiply(nn.silu(split(y, 2)[0]), split(y, 2)[1]) behind the cast: the call description carries
+    ACT_SILU_MUL and no fused operands; anything else around the split is refused."""
+    from relax_amd.tvm_glue.codegen import ACT_SILU_MUL, CallSpec as Spec, spec_from_function, trampoline_source
+
+    s = spec_from_function(fake_tvm.quantized_linear(n=64, tail=[("silu_mul",)]))
+    assert (s.activation, s.arg_bias, s.arg_residual, s.arg_wq, s.arg_scales, s.arg_x, s.arg_out, s.num_args) == \
+        (ACT_SILU_MUL, -1, -1, 0, 1, 2, 3, 4)
+    import re
+    assert re.search(r"-1,\s*-1, 2\};", trampoline_source([("gated_mi355x", s)]))  # ... arg_bias, arg_residual, activation
+    assert spec_from_function(fake_tvm.quantized_linear(n=64, tail=[("silu_mul", 2, 1)])).activation == ACT_SILU_MUL
+    for tail, message in [([("silu_mul", 4)], "splits the output in two"),
+                          ([("silu_mul", 2, 0)], "along its last axis"),
+                          ([("silu_mul", 2, -1, True)], "first half"),
+                          ([("add", [64]), ("silu_mul",)], "must halve the matmul result itself"),
+                          ([("silu_mul",), ("relu",)], "no further operations"),
+                          ([("silu_mul",), ("add", [4, 32])], "no bias and no residual")]:
+        with pytest.raises(ValueError, match=message):
+            spec_from_function(fake_tvm.quantized_linear(n=64, tail=tail))
+    with pytest.raises(ValueError, match="no bias and no residual"):
+        Spec(0, 4, 0, 7, 2, 0, 1, 4, 3, -1, ACT_SILU_MUL).validate()
