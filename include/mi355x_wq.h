@@ -156,7 +156,7 @@ MI355X_WQ_API int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const vo
                                            const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y,
                                            int64_t m, void* stream, int kernel);
 
-/* Decode with a caller workspace: for M <= 16 and projections whose 16-row tiles leave CUs idle for
+/* K split with a caller workspace.  Decode: for M <= 16 and projections whose 16-row tiles leave CUs idle for
  * whole rounds (5120 rows: 320 tiles on 256 CUs) or whose activations are large against one tile per CU,
  * the decode kernel splits K over two to four workgroups per tile; each writes a float32 partial tile
  * to the workspace, and the last to arrive adds them in the order of their K windows (the result does
@@ -169,6 +169,13 @@ MI355X_WQ_API int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const vo
  * arrival counters at the head, then 1 KB per 16-row tile and K window, so one workspace sized for the
  * largest projection serves projections of every shape; 0 if it
  * would not split (then the call equals mi355x_wq_matmul_fused / _tiled), -1 on an invalid descriptor.
+ *
+ * Above 64 rows the same call splits K for the direct-weight GEMM where 128 x 256 output tiles would leave
+ * at least half of the CUs without one (e.g. 256 rows x 5120 columns: 40 tiles): two to eight workgroups
+ * per tile, each on a window of at least 1024 (int8) or 2048 (int4) of K, 128 KB of float32 partials per
+ * tile and window behind the same 16 KB of counters, summed in window order as above.  Measured, int8 at
+ * 256 rows: 5120 x 13824 91 -> 63 us, 15360 x 5120 71 -> 60 us, 5120 x 5120 39 -> 37 us; int4 at 128-256
+ * rows x 4096 x 11008: 50 -> 40-45 us; shapes the split would slow (short K, int4 with more tiles) report 0.
  * Workspace rules: device memory, 16-byte aligned, all zero before its first use (the kernel leaves it
  * ready for the next call); calls that share a workspace must not overlap in time (one stream, or
  * ordered by events); a workspace that is NULL or smaller than required disables the split for that call. */

@@ -222,7 +222,7 @@ int64_t mi355x_wq_workspace_bytes(const mi355x_wq_desc* desc, int64_t m, int til
   if (m == 0 || desc->n == 0 || desc->k == 0) return 0;
   Problem p{nullptr, nullptr, nullptr, nullptr, m, desc->n, desc->k, desc->bits, desc->group, desc->zero_point, nullptr};
   p.tiled = tiled != 0;
-  return gemv_split_workspace_bytes(p);
+  return m <= 16 ? gemv_split_workspace_bytes(p) : gemm_split_workspace_bytes(p);
 }
 
 int mi355x_wq_matmul_ws(const mi355x_wq_desc* desc, const void* x, const void* wq_, const void* scales,
@@ -365,7 +365,7 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
   if (workspace != nullptr && family == MI355X_WQ_KERNEL_AUTO) {
     // a caller workspace allows the decode kernel's K split where it pays; everything else is as without
     if (!check_ptr(workspace, "workspace", 16)) return -1;
-    const int rc = launch_gemv_split(p, workspace, workspace_bytes);
+    const int rc = m <= 16 ? launch_gemv_split(p, workspace, workspace_bytes) : launch_gemm_split(p, workspace, workspace_bytes);
     if (rc != 0) return rc < 0 ? -1 : 0;
   }
   if (library_scratch) {

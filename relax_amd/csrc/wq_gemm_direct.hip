@@ -51,6 +51,7 @@
 // groups), group 32 (int4) or 128 (int8), operands < 1 GiB; other shapes use the other GEMM
 // kernels.
 #include <atomic>
+#include <algorithm>
 #include <type_traits>
 
 #include "wq_device.h"
@@ -59,6 +60,8 @@
 namespace wq {
 
 namespace {
+constexpr int64_t kGemmSplitMaxTiles = 4096;                      // arrival counters at the head of a workspace
+constexpr int64_t kGemmSplitCounterBytes = kGemmSplitMaxTiles * 4;  // (the decode kernel's split uses the same head)
 constexpr uint32_t kRowOobD = 0x80000000u;   // offset of a row that must read zeros
 constexpr uint32_t kStepOobD = 0x40000000u;  // added for a K step past K: beyond any buffer < 1 GiB
 
@@ -77,11 +80,11 @@ struct RawB {
   u32x4 w[2][NV];                               // [column tile][load]
 };
 
-template <int BITS, int GROUPS, int TM, int WAVES, bool TILED>
+template <int BITS, int GROUPS, int TM, int WAVES, bool TILED, bool KSPLIT = false>
 __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
     int M, int N, int K, int shift_and_zero, int tiles_m, int tiles_n, int tile_n0, half_t* y,
-    const Epilogue ep) {
+    const Epilogue ep, int ksplit, float* partials, unsigned int* counters) {
   // (argument order: the first 14 dwords are preloaded into SGPRs at wavefront launch, later ones are
   // a scalar load at the start of the kernel; what the K loop needs comes first, y and the epilogue last)
   const int group_shift = shift_and_zero & 0xFF, zero_point = (shift_and_zero >> 8) & 0xFF;
@@ -110,9 +113,15 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   // panels of eight tiles, row-major inside a panel: the 32 workgroups an XCD runs at a time
   // then cover 4 activation row blocks x 8 weight column tiles and walk K together, so its L2
   // serves every activation block eight times and every weight tile four times per fetch.
+  // K split across workgroups (caller workspace): S consecutive workgroup ids share a tile, each on its
+  // own window of K; S = 1 otherwise.
+  const int S = KSPLIT ? ksplit : 1;  // (a build of its own: the plain kernel keeps its registers)
   const int nblocks = tiles_m * tiles_n;
   int bid = blockIdx.x;
-  if ((nblocks & 7) == 0) bid = (bid & 7) * (nblocks >> 3) + (bid >> 3);
+  const int ks = S > 1 ? bid % S : 0;
+  if (S > 1) bid /= S;
+  const int tile_lin = bid;  // the tile's slot in the workspace
+  if (S == 1 && (nblocks & 7) == 0) bid = (bid & 7) * (nblocks >> 3) + (bid >> 3);
   constexpr int PANEL = 8;
   const int full = tiles_n / PANEL;                 // panels of full width
   const int in_full = bid / (tiles_m * PANEL);      // panel index if inside the full ones
@@ -133,10 +142,14 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
 
   // K range of this group, in 64-wide steps; both groups run the same number of steps and
   // the shorter one reads zeros (out-of-range offsets) past its end.
+  // (with a K split the same inside this workgroup's window of whole 256-wide macro steps)
   const int ksteps = K / BK;
-  const int nloop = GROUPS == 1 ? ksteps : 4 * ((ksteps / 4 + GROUPS - 1) / GROUPS);
-  const int kbase = grp * nloop;
-  const int kend = min(kbase + nloop, ksteps);
+  const int macro_per = (ksteps / 4 + S - 1) / S;
+  const int win_begin = min(ks * macro_per * 4, ksteps), win_end = min((ks + 1) * macro_per * 4, ksteps);
+  const int wsteps = win_end - win_begin;
+  const int nloop = GROUPS == 1 ? wsteps : 4 * ((wsteps / 4 + GROUPS - 1) / GROUPS);
+  const int kbase = win_begin + grp * nloop;
+  const int kend = min(kbase + nloop, win_end);
 
   const uint32_t row_bytes = (uint32_t)K * BITS / 8;
   const uint32_t groups_per_row = ((uint32_t)K / CH) >> group_shift;
@@ -436,6 +449,7 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
       for (int q = 0; q < SW; ++q) sc_cur[j][q] = sc_nxt[j][q];
   }
 
+  int mrow0 = m0, nrb = TM;  // first row and row blocks this wavefront finishes (a K split's sum shares them out)
   // ---- K groups: the other groups hand their partial sums to the first through LDS ---------
   // Rounds of 16 KB per wavefront (two row blocks each); a wavefront and its partners hold the
   // same elements in the same lanes, so the exchange is lane-contiguous 16-byte vectors.
@@ -472,7 +486,78 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
         __syncthreads();
       }
     }
-    if (grp != 0) return;
+    if (!KSPLIT && grp != 0) return;
+  }
+  if constexpr (KSPLIT) {
+    // K split: every workgroup writes the float32 partial tile of its window to the workspace (lane-contiguous
+    // 16-byte vectors) and counts itself in; the one that finds S - 1 others counted adds the S partials in the
+    // order of their windows -- whoever arrives last, the sum is the same -- and goes on to the epilogue; it
+    // returns the counter to zero for the next launch.  Partials and counters are only touched by accesses that
+    // are performed at the memory side of the chip's L2s (sc1), and a workgroup's stores have completed before
+    // the barrier after which its count goes out.
+    const bool owner = GROUPS == 1 || grp == 0;
+    constexpr uint32_t kWaveFloats = TM * 2 * 16 * 64;  // accumulators of one wavefront
+    const rsrc_t rp = make_rsrc(partials + (size_t)tile_lin * S * WAVES * kWaveFloats, (uint32_t)S * WAVES * kWaveFloats * 4u);
+    if (owner) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v4 = 0; v4 < 4; ++v4) {
+            const float16_t& a = acc[i][j];
+            const u32x4 bits = __builtin_bit_cast(u32x4, float4_t{a[v4 * 4], a[v4 * 4 + 1], a[v4 * 4 + 2], a[v4 * 4 + 3]});
+            __builtin_amdgcn_raw_buffer_store_b128(bits, rp, ((uint32_t)(ks * WAVES + wave) * (TM * 8) + (i * 2 + j) * 4 + v4) * 1024u + lane * 16u, 0, 0x10);
+          }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    int* const last = reinterpret_cast<int*>(wq_gemm_direct_smem);
+    if (threadIdx.x == 0)
+      *last = __hip_atomic_fetch_add(&counters[tile_lin], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(S - 1);
+    __syncthreads();
+    if (!*last) return;
+    if (threadIdx.x == 0) __hip_atomic_store(&counters[tile_lin], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // The K groups share the sum: each takes TM / GROUPS of the tile's row blocks (every wavefront of the
+    // workgroup reads; holding two windows in flight measured no faster) and finishes those rows itself.
+    constexpr int RG = (TM % GROUPS == 0) ? GROUPS : 1;
+    if (RG == 1 && !owner) return;
+    nrb = TM / RG;
+    const int i0 = RG == 1 ? 0 : grp * (TM / RG);
+    mrow0 = m0 + i0 * 32;
+#pragma unroll
+    for (int i = 0; i < TM / RG; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    auto load_window = [&](int q, u32x4 (&buf)[TM / RG][2][4]) {
+#pragma unroll
+      for (int i = 0; i < TM / RG; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v4 = 0; v4 < 4; ++v4)
+            buf[i][j][v4] = __builtin_amdgcn_raw_buffer_load_b128(
+                rp, ((uint32_t)(q * WAVES + wave) * (TM * 8) + ((i0 + i) * 2 + j) * 4 + v4) * 1024u + lane * 16u, 0, 0x10);
+    };
+    auto add_window = [&](const u32x4 (&buf)[TM / RG][2][4]) {
+#pragma unroll
+      for (int i = 0; i < TM / RG; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v4 = 0; v4 < 4; ++v4) {
+            const float4_t o = __builtin_bit_cast(float4_t, buf[i][j][v4]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][v4 * 4 + e] += o[e];
+          }
+    };
+    u32x4 win[TM / RG][2][4];
+    for (int q = 0; q < S; ++q) {  // windows are added in their order, whoever arrived last
+      load_window(q, win);
+      add_window(win);
+    }
   }
 
   // ---- epilogue: lane holds columns 2 (lane % 32), + 1 and rows 8*(v/4) + 4*(lane/32) + v%4 ------
@@ -483,8 +568,8 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int m = m0 + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
-        if (m < M && n + 1 < N) store_gated(y, m, n >> 1, N >> 1, acc[i][0][v], acc[i][1][v]);
+        const int m = mrow0 + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
+        if (i < nrb && m < M && n + 1 < N) store_gated(y, m, n >> 1, N >> 1, acc[i][0][v], acc[i][1][v]);
       }
     return;
   }
@@ -492,15 +577,16 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   if (paired && m0 + BM <= M && n0 + WAVES * 64 <= N) {
     // Tile inside the matrix, 4-byte accesses allowed: the tail's shape is decided once, outside the
     // unrolled stores (per-element tests of the three epilogue fields cost more than the stores).
-    half_t* const y0 = y + (size_t)(m0 + fh * 4) * N + n;
+    half_t* const y0 = y + (size_t)(mrow0 + fh * 4) * N + n;
     auto store_tile = [&](auto has_bias, auto relu, auto has_res) {
       half2_t b2 = half2_t{(half_t)0, (half_t)0};
       if constexpr (decltype(has_bias)::value) b2 = *reinterpret_cast<const half2_t*>(ep.bias + n);
-      const half_t* const r0 = decltype(has_res)::value ? ep.residual + (size_t)(m0 + fh * 4) * N + n : nullptr;
+      const half_t* const r0 = decltype(has_res)::value ? ep.residual + (size_t)(mrow0 + fh * 4) * N + n : nullptr;
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
+          if (i >= nrb) continue;
           half2_t res[4];
           if constexpr (decltype(has_res)::value) {
 #pragma unroll
@@ -537,32 +623,37 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const int m = m0 + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
-      if (m < M) store_out2(ep, y, m, n, N, acc[i][0][v], acc[i][1][v], paired);
+      const int m = mrow0 + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
+      if (i < nrb && m < M) store_out2(ep, y, m, n, N, acc[i][0][v], acc[i][1][v], paired);
     }
 }
 
 namespace {
 
 // Column tiles [tile_n0, tile_n0 + tile_count) of the matrix (tile_count < 0: all of them).
-template <int BITS, int GROUPS, int TM, int WAVES, bool TILED>
-bool launch_direct(const Problem& p, int group_shift, int tile_n0 = 0, int tile_count = -1) {
+template <int BITS, int GROUPS, int TM, int WAVES, bool TILED, bool KSPLIT = false>
+bool launch_direct(const Problem& p, int group_shift, int tile_n0 = 0, int tile_count = -1, int ksplit = 1,
+                   void* workspace = nullptr) {
   constexpr int BM = TM * 32, BN = WAVES * 64;
   const int tiles_m = (int)((p.m + BM - 1) / BM);
   const int tiles_n = tile_count >= 0 ? tile_count : (int)((p.n + BN - 1) / BN);
   if (tiles_n == 0) return true;
-  dim3 grid(tiles_m * tiles_n), block(GROUPS * WAVES * 64);
+  dim3 grid(tiles_m * tiles_n * ksplit), block(GROUPS * WAVES * 64);
+  // workspace of the K split: arrival counters at its head (shared with the decode kernel's split), then
+  // [tiles][ksplit] float32 partial tiles
+  unsigned int* const counters = static_cast<unsigned int*>(workspace);
+  float* const partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kGemmSplitCounterBytes);
   // four activation stages per K group; the K-group exchange needs 16 KB per wavefront of a group
   constexpr size_t stages = (size_t)GROUPS * 4 * BM * 128, exchange = GROUPS > 1 ? (size_t)WAVES * 16384 : 0;
   constexpr size_t lds_bytes = stages > exchange ? stages : exchange;
   static_assert(lds_bytes <= 160 * 1024, "LDS per workgroup");
   static std::atomic<bool> lds_ok[kMaxDevices];
-  if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED>, (int)lds_bytes, lds_ok))
+  if (!ensure_dynamic_lds((const void*)wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED, KSPLIT>, (int)lds_bytes, lds_ok))
     return false;
-  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED>), grid, block, lds_bytes, p.stream,
+  hipLaunchKernelGGL((wq_gemm_direct_kernel<BITS, GROUPS, TM, WAVES, TILED, KSPLIT>), grid, block, lds_bytes, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales, (int)p.m, (int)p.n,
                      (int)p.k, group_shift | (p.zero_point << 8) | (p.activation == kActGated ? 1 << 16 : 0), tiles_m, tiles_n, tile_n0, (half_t*)p.y,
-                     Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
+                     Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation}, ksplit, partials, counters);
   return true;
 }
 
@@ -573,6 +664,32 @@ bool launch_bits(const Problem& p, int group_shift, int tile_n0 = 0, int tile_co
                        : launch_direct<8, GROUPS, TM, WAVES, true>(p, group_shift, tile_n0, tile_count);
   return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES, false>(p, group_shift, tile_n0, tile_count)
                      : launch_direct<8, GROUPS, TM, WAVES, false>(p, group_shift, tile_n0, tile_count);
+}
+
+bool launch_split_bits(const Problem& p, int group_shift, int ksplit, void* workspace) {
+  if (p.tiled)
+    return p.bits == 4 ? launch_direct<4, 2, 4, 4, true, true>(p, group_shift, 0, -1, ksplit, workspace)
+                       : launch_direct<8, 2, 4, 4, true, true>(p, group_shift, 0, -1, ksplit, workspace);
+  return p.bits == 4 ? launch_direct<4, 2, 4, 4, false, true>(p, group_shift, 0, -1, ksplit, workspace)
+                     : launch_direct<8, 2, 4, 4, false, true>(p, group_shift, 0, -1, ksplit, workspace);
+}
+
+// Whether, and how many ways, to split K across workgroups for `p` (128 x 256 tiles, two K groups inside
+// the workgroup): where those tiles would leave at least half of the CUs without one -- the cases the
+// default selection answers with smaller tiles, whose workgroups then move two to four times the bytes
+// per output.  Every window costs a round trip through the workspace (partial tile out, count, the last
+// one reads them all), so the windows must stay long: measured on the Llama-2 projections, int8 weights
+// gain from windows of four macro steps (K 1024) on, int4 weights -- whose small-tile kernels are better --
+// only from eight macro steps on, with at least four windows and tiles on at most an eighth of the CUs.
+int gemm_split_ways(const Problem& p) {
+  if (p.m <= 64 || p.k % 256 != 0 || p.group != (p.bits == 4 ? 32 : 128) || !gemm_pipe_applicable(p)) return 1;
+  if (p.activation == kActGated) return 1;
+  const int64_t cu = cu_count(), tiles = ((p.m + 127) / 128) * ((p.n + 255) / 256), macro = p.k / 256;
+  if (tiles * (p.bits == 4 ? 8 : 2) > cu || tiles > kGemmSplitMaxTiles) return 1;
+  const int64_t ways = std::min<int64_t>({cu / tiles, macro / (p.bits == 4 ? 8 : 4), 8});
+  if (ways < (p.bits == 4 ? 4 : 2)) return 1;
+  const int64_t per = (macro + ways - 1) / ways;  // macro steps per window; drop windows that would be empty
+  return (int)((macro + per - 1) / per);
 }
 
 }  // namespace
@@ -612,6 +729,31 @@ bool launch_gemm_direct(const Problem& p, int group_shift, int variant) {
     }
     default: return false;
   }
+}
+
+
+// Bytes of caller workspace the K split of the direct-weight GEMM needs for `p`, 0 where it does not apply.
+int64_t gemm_split_workspace_bytes(const Problem& p) {
+  const int ways = gemm_split_ways(p);
+  if (ways < 2) return 0;
+  const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 255) / 256);
+  return kGemmSplitCounterBytes + tiles * ways * (128 * 256 * 4);
+}
+
+// 1 = launched with the K split, 0 = the split does not apply or the workspace is too small, -1 = failure
+int launch_gemm_split(const Problem& p, void* workspace, int64_t workspace_bytes) {
+  const int64_t need = gemm_split_workspace_bytes(p);
+  if (need == 0 || workspace == nullptr || workspace_bytes < need) return 0;
+  const int ch = 128 / p.bits;
+  int ratio = p.group / ch, group_shift = 0;
+  while ((1 << group_shift) < ratio) ++group_shift;
+  if (!launch_split_bits(p, group_shift, gemm_split_ways(p), workspace)) return -1;
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("gemm kernel (K split) launch failed: %s", hipGetErrorString(e));
+    return -1;
+  }
+  return 1;
 }
 
 }  // namespace wq

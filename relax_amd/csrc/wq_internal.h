@@ -36,6 +36,10 @@ int launch_gemv_split(const Problem& p, void* workspace, int64_t workspace_bytes
 // 1 launched, 0 the split does not apply, -1 failure (also when the problem needs more than the array holds).
 int launch_gemv_split_static(const Problem& p);
 int64_t gemv_static_scratch_bytes();
+// The same for the direct-weight GEMM (M > 64): 128 x 256 tiles whose K range is split over workgroups where
+// those tiles alone would leave half of the CUs idle.
+int64_t gemm_split_workspace_bytes(const Problem& p);
+int launch_gemm_split(const Problem& p, void* workspace, int64_t workspace_bytes);
 int launch_skinny(const Problem& p, int variant);
 int launch_gemm(const Problem& p, int variant);
 bool gemm_pipe_applicable(const Problem& p);  // K % 64 == 0, operands below 1 GiB

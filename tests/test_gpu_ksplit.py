@@ -207,3 +207,77 @@ def test_k_split_is_stable_while_another_stream_keeps_the_gpu_busy():
     bad = [i for i, y in enumerate(outs) if not torch.equal(y.view(torch.int16), ref.view(torch.int16))]
     assert not bad, bad[:10]
     assert int(ws[:16384].view(torch.int32).abs().sum()) == 0
+
+
+# (bits, M, N, K): prefill-side shapes whose 128 x 256 tiles fill at most half of the CUs
+GEMM_CASES = [(8, 256, 5120, 5120), (8, 256, 5120, 13824), (8, 256, 15360, 5120), (4, 256, 4096, 11008),
+              (4, 128, 4096, 11008), (4, 200, 4090, 8192), (8, 65, 5120, 5120), (8, 384, 1000, 2048)]
+
+
+@pytest.mark.parametrize("bits,m,n,k", GEMM_CASES)
+def test_gemm_k_split_matches_the_oracle_and_is_deterministic(bits, m, n, k):
+    import relax_amd
+
+    x, wq, s, g = O.make_case(71, m, n, k, bits)
+    need = relax_amd.wq_workspace_bytes(bits, g, n, k, m)
+    assert need > 16384, "the case is meant to split"
+    ws = relax_amd.wq_workspace(need)
+    dx, dwq, ds = _dev(x), _dev(wq), _dev(s)
+    y1 = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws)
+    torch.cuda.synchronize()
+    assert int(ws[:16384].view(torch.int32).abs().sum()) == 0, "arrival counters are back at zero"
+    rows = sorted({0, 1, m // 2, m - 2, m - 1} | set(np.random.default_rng(5).integers(0, m, 11).tolist()))
+    want = c_oracle.wq_matmul(x[rows], wq, s, bits, g, nthreads=16)
+    assert_close(y1.cpu().numpy()[rows], want, ("gemm k split", bits, m, n, k), ulp_fraction=0.005)
+    # every tile, against float32 torch on the dequantized weights (the oracle's rows pin the arithmetic)
+    ref = dx.float() @ relax_amd.wq_dequantize(dwq, ds, bits, g).float().T
+    err = (y1.float() - ref).abs()
+    assert bool((err <= 1e-2 + 1e-2 * ref.abs()).all()), float(err.max())
+    for _ in range(3):
+        y2 = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y1.view(torch.int16), y2.view(torch.int16))
+    # without a workspace: the plain kernels, same tolerance against the oracle
+    y0 = relax_amd.wq_matmul(dx, dwq, ds, bits, g)
+    torch.cuda.synchronize()
+    assert_close(y0.cpu().numpy()[rows], want, ("plain", bits, m, n, k), ulp_fraction=0.005)
+
+
+def test_gemm_k_split_applies_the_fused_tail_once():
+    import relax_amd
+
+    bits, m, n, k = 8, 256, 4096, 11008
+    x, wq, s, g = O.make_case(73, m, n, k, bits)
+    bias, res = _fused_operands(73, m, n)
+    ws = relax_amd.wq_workspace(relax_amd.wq_workspace_bytes(bits, g, n, k, m))
+    dx, dwq, ds = _dev(x), _dev(wq), _dev(s)
+    plain = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws)
+    fused = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws, bias=_dev(bias), activation="relu",
+                                residual=_dev(res))
+    torch.cuda.synchronize()
+    rows = [0, 7, 128, 255]
+    want_plain = c_oracle.wq_matmul(x[rows], wq, s, bits, g, nthreads=16)
+    assert_fused(fused.cpu().numpy()[rows], plain.cpu().numpy()[rows], want_plain, bias, "relu", res[rows],
+                 (bits, m, n, k))
+
+
+def test_one_workspace_serves_decode_and_prefill_shapes():
+    """The decode kernel's split and the GEMM's share the counters at the head of the workspace."""
+    import relax_amd
+
+    shapes = [(8, 256, 4096, 4096), (4, 8, 4096, 11008), (4, 256, 4096, 11008), (8, 16, 5120, 13824)]
+    cases = [(bits, O.make_case(81 + i, m, n, k, bits)) for i, (bits, m, n, k) in enumerate(shapes)]
+    need = max(relax_amd.wq_workspace_bytes(bits, g, wq.shape[0], x.shape[1], x.shape[0]) for bits, (x, wq, s, g) in cases)
+    ws = relax_amd.wq_workspace(need)
+    first = {}
+    for rnd in range(3):
+        for i, (bits, (x, wq, s, g)) in enumerate(cases):
+            y = relax_amd.wq_matmul(_dev(x), _dev(wq), _dev(s), bits, g, workspace=ws)
+            torch.cuda.synchronize()
+            if rnd == 0:
+                first[i] = y
+                rows = [0, x.shape[0] - 1]
+                assert_close(y.cpu().numpy()[rows], c_oracle.wq_matmul(x[rows], wq, s, bits, g, nthreads=16),
+                             shapes[i], ulp_fraction=0.005)
+            else:
+                assert torch.equal(y.view(torch.int16), first[i].view(torch.int16)), (rnd, shapes[i])
