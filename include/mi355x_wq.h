@@ -77,8 +77,7 @@ MI355X_WQ_API int mi355x_wq_matmul_ex(const mi355x_wq_desc* desc, const void* x,
  * `matmul_bias` / `matmul_bias_relu` family of the reference's pattern helpers
  * (python/tvm/relax/dpl/pattern.py:1049-1095) and of its CUTLASS epilogues
  * (python/tvm/contrib/cutlass/gen_tensor_op.py:377-380), plus the residual add that follows
- * the O and down projections of a decoder layer.  `relax.nn.gelu` is not offered: the CPU
- * path cannot lower erf on float16 (src/target/intrin_rule.h:39-48), so there is nothing to match. */
+ * the O and down projections of a decoder layer. */
 enum {
   MI355X_WQ_ACT_NONE = 0,
   MI355X_WQ_ACT_RELU = 1,
@@ -93,7 +92,15 @@ enum {
    * (python/tvm/relax/dpl/pattern.py:1049-1095, python/tvm/contrib/cutlass/gen_tensor_op.py:377-380).
    * `y` is [M, N/2]; no bias, no residual, canonical weights, N even; M <= 16 runs the decode kernel,
    * larger M needs K % 256 == 0 with group 32 (int4) / 128 (int8). */
-  MI355X_WQ_ACT_SILU_MUL = 2
+  MI355X_WQ_ACT_SILU_MUL = 2,
+  /* nn.gelu behind the bias add (python/tvm/contrib/cutlass/gen_tensor_op.py:375-380, the *_bias_gelu members),
+   * as the float16 operation sequence of its legalized form x * (0.5 + erf(x * sqrt(0.5)) * 0.5)
+   * (python/tvm/relax/transform/legalize_ops.py:495-503): the constants rounded to float16, four float16
+   * roundings, erf evaluated in float32 and rounded to float16.  The reference's CPU path has no float16 erf
+   * to compare with (src/target/intrin_rule.h:39-48 gives it no extern name), so this member is checked
+   * against that sequence restated on the host and, in closed form, against x * Phi(x) in float64: within
+   * 4 float16 ulp wherever |x| <= 3.5 and the result is a normal number. */
+  MI355X_WQ_ACT_GELU = 3
 };
 typedef struct mi355x_wq_epilogue {
   const void* bias;     /* float16 [N] (device), or NULL */

@@ -97,6 +97,14 @@ MI355X_WQ_API int mi355x_q8f16_matmul_bias_relu(mi355x_tvm_value* args, int* typ
 MI355X_WQ_API int mi355x_q8f16_matmul_residual(mi355x_tvm_value* args, int* type_codes, int num_args,
                                  mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
                                  void* resource_handle);
+/* matmul + bias + nn.gelu (MI355X_WQ_ACT_GELU), the reference's *_bias_gelu composite members
+ * (python/tvm/contrib/cutlass/gen_tensor_op.py:375-380): args x, wq, scales, bias, out */
+MI355X_WQ_API int mi355x_q4f16_matmul_bias_gelu(mi355x_tvm_value* args, int* type_codes, int num_args,
+                                  mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
+                                  void* resource_handle);
+MI355X_WQ_API int mi355x_q8f16_matmul_bias_gelu(mi355x_tvm_value* args, int* type_codes, int num_args,
+                                  mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
+                                  void* resource_handle);
 MI355X_WQ_API int mi355x_q4f16_matmul_silu_mul(mi355x_tvm_value* args, int* type_codes, int num_args,
                                  mi355x_tvm_value* out_ret_value, int* out_ret_tcode,
                                  void* resource_handle);

@@ -119,7 +119,7 @@ def wq_matmul(x, wq, s, bits: int, group: int, nthreads: int = 1) -> np.ndarray:
 
 
 def epilogue(y, bias=None, activation=None, residual=None) -> np.ndarray:
-    """Fused tail on a copy of y [M,N] float16: + bias[N], relu, + residual[M,N]."""
+    """Fused tail on a copy of y [M,N] float16: + bias[N], relu or gelu, + residual[M,N]."""
     L = lib()
     if activation == "silu_mul":
         if bias is not None or residual is not None:
@@ -133,7 +133,7 @@ def epilogue(y, bias=None, activation=None, residual=None) -> np.ndarray:
         return gated
     out = np.array(y, dtype=np.float16, order="C", copy=True)
     m, n = out.shape
-    if activation not in (None, "none", "relu", "relax.nn.relu"):
+    if activation not in (None, "none", "relu", "relax.nn.relu", "gelu", "relax.nn.gelu"):
         raise ValueError(f"unsupported activation {activation!r}")
     b = None if bias is None else np.ascontiguousarray(np.asarray(bias, dtype=np.float16).reshape(-1))
     r = None if residual is None else np.ascontiguousarray(residual, dtype=np.float16)
@@ -142,7 +142,7 @@ def epilogue(y, bias=None, activation=None, residual=None) -> np.ndarray:
     if r is not None and r.shape != (m, n):
         raise ValueError("residual must be [M, N]")
     L.wq_oracle_epilogue(_ptr(out), m, n, None if b is None else _ptr(b),
-                         1 if activation in ("relu", "relax.nn.relu") else 0,
+                         {"relu": 1, "relax.nn.relu": 1, "gelu": 3, "relax.nn.gelu": 3}.get(activation, 0),
                          None if r is None else _ptr(r))
     return out
 

@@ -171,17 +171,36 @@ int wq_oracle_wq_matmul(int bits, int64_t group, const uint16_t* x, const uint32
  * innocuous because float32 carries 24 >= 2*11 + 2 significand bits); relu is
  * select(t > 0, t, 0) -- src/target/llvm/codegen_llvm.cc:1500-1504.  bias / residual may be
  * NULL. ---- */
-void wq_oracle_epilogue(uint16_t* y, int64_t m_rows, int64_t n_rows, const uint16_t* bias, int relu,
+static uint16_t gelu_f16(uint16_t h);
+
+void wq_oracle_epilogue(uint16_t* y, int64_t m_rows, int64_t n_rows, const uint16_t* bias, int activation,
                         const uint16_t* residual) {
+  const int relu = activation == 1, gelu = activation == 3;
   for (int64_t m = 0; m < m_rows; ++m)
     for (int64_t n = 0; n < n_rows; ++n) {
       uint16_t h = y[m * n_rows + n];
       if (bias) h = wq_oracle_f32_to_f16(wq_oracle_f16_to_f32(h) + wq_oracle_f16_to_f32(bias[n]));
       if (relu) h = (wq_oracle_f16_to_f32(h) > 0.0f) ? h : (uint16_t)0;
+      if (gelu) h = gelu_f16(h);
       if (residual)
         h = wq_oracle_f32_to_f16(wq_oracle_f16_to_f32(h) + wq_oracle_f16_to_f32(residual[m * n_rows + n]));
       y[m * n_rows + n] = h;
     }
+}
+
+/* ---- nn.gelu on one float16 value: the legalized form x * (0.5 + erf(x * sqrt(0.5)) * 0.5) of
+ * python/tvm/relax/transform/legalize_ops.py:495-503 evaluated on float16, one rounding per operation:
+ * a = f16(x * f16(sqrt(0.5))), e = f16(erff(a)), b = f16(e * 0.5), c = f16(0.5 + b), out = f16(x * c).
+ * (The reference's CPU path gives float16 erf no extern name, src/target/intrin_rule.h:39-48; evaluating it
+ * in float32 and rounding is what the float16 exp of the same path does.) ---- */
+static uint16_t gelu_f16(uint16_t h) {
+  const float x = wq_oracle_f16_to_f32(h);
+  const float c0 = wq_oracle_f16_to_f32(wq_oracle_f32_to_f16(0.70710678118654752440f));
+  const float a = wq_oracle_f16_to_f32(wq_oracle_f32_to_f16(x * c0));
+  const float e = wq_oracle_f16_to_f32(wq_oracle_f32_to_f16(erff(a)));
+  const float b = wq_oracle_f16_to_f32(wq_oracle_f32_to_f16(e * 0.5f));
+  const float c = wq_oracle_f16_to_f32(wq_oracle_f32_to_f16(0.5f + b));
+  return wq_oracle_f32_to_f16(x * c);
 }
 
 /* ---- gated tail: out[m, j] = multiply(nn.silu(y[m, j]), y[m, j + n/2]) for j < n/2, the float16

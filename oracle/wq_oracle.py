@@ -217,6 +217,26 @@ def silu_mul_f16(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
         return (t.astype(np.float64) * u.astype(np.float64)).astype(np.float16)
 
 
+def gelu_f16(t: np.ndarray) -> np.ndarray:
+    """nn.gelu on a float16 tensor as its legalized form x * (0.5 + erf(x * sqrt(0.5)) * 0.5)
+    (python/tvm/relax/transform/legalize_ops.py:495-503) runs on float16, one rounding per operation and the
+    constants rounded to float16 first: a = f16(x * f16(sqrt(0.5))); e = f16(erff(a)); b = f16(e * 0.5);
+    c = f16(0.5 + b); y = f16(x * c).  erff is taken as the float64 erf rounded to float32.  The reference's
+    CPU path cannot lower a float16 erf (src/target/intrin_rule.h:39-48), so this sequence has no reference
+    output to be compared with: it is pinned in closed form against x * Phi(x)."""
+    import math
+
+    x = np.asarray(t, dtype=np.float16)
+    c0 = np.float16(0.5 ** 0.5)
+    with np.errstate(over="ignore", invalid="ignore", under="ignore"):
+        a = (x.astype(np.float64) * np.float64(c0)).astype(np.float16)
+        erf = np.vectorize(math.erf, otypes=[np.float64])
+        e = erf(a.astype(np.float64)).astype(np.float32).astype(np.float16)
+        b = (e.astype(np.float64) * 0.5).astype(np.float16)
+        c = (np.float64(0.5) + b.astype(np.float64)).astype(np.float16)
+        return (x.astype(np.float64) * c.astype(np.float64)).astype(np.float16)
+
+
 def gated_epilogue(y: np.ndarray) -> np.ndarray:
     """y [M, N] = f16(accumulator) of a fused gate+up projection -> [M, N/2]:
     multiply(nn.silu(y[:, :N/2]), y[:, N/2:])."""
@@ -229,7 +249,7 @@ def gated_epilogue(y: np.ndarray) -> np.ndarray:
 
 def epilogue(y: np.ndarray, bias=None, activation: str | None = None, residual=None) -> np.ndarray:
     """The fused tail of a composite applied to y = f16(accumulator):
-    + bias[N], then relu, then + residual[M,N]; every step absent or one float16 op."""
+    + bias[N], then relu or gelu, then + residual[M,N]; every step absent or float16 ops rounded one by one."""
     t = np.asarray(y, dtype=np.float16)
     if activation == "silu_mul":
         if bias is not None or residual is not None:
@@ -239,6 +259,8 @@ def epilogue(y: np.ndarray, bias=None, activation: str | None = None, residual=N
         t = add_f16(t, np.asarray(bias, dtype=np.float16).reshape(1, -1))
     if activation in ("relu", "relax.nn.relu"):
         t = relu_f16(t)
+    elif activation in ("gelu", "relax.nn.gelu"):
+        t = gelu_f16(t)
     elif activation not in (None, "none"):
         raise ValueError(f"unsupported activation {activation!r}")
     if residual is not None:

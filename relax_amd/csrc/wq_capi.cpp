@@ -304,7 +304,7 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
       return -1;
     }
     if (ep->activation != MI355X_WQ_ACT_NONE && ep->activation != MI355X_WQ_ACT_RELU &&
-        ep->activation != MI355X_WQ_ACT_SILU_MUL) {
+        ep->activation != MI355X_WQ_ACT_SILU_MUL && ep->activation != MI355X_WQ_ACT_GELU) {
       set_error("unknown epilogue activation %d", ep->activation);
       return -1;
     }

@@ -149,9 +149,21 @@ __device__ __forceinline__ half8_t pack_h8(half2_t a, half2_t b, half2_t c, half
 struct Epilogue {
   const half_t* bias;      // [N], or nullptr
   const half_t* residual;  // [M,N], or nullptr; may be the output buffer itself
-  int activation;          // 0 none, 1 relu, 2 gated: y[M, N/2] = multiply(nn.silu(gate), up), see store_gated
+  int activation;          // 0 none, 1 relu, 2 gated: y[M, N/2] = multiply(nn.silu(gate), up), see store_gated; 3 gelu
 };
 constexpr int kActGated = 2;
+constexpr int kActGelu = 3;
+
+// nn.gelu on a float16 value as its legalized form x * (0.5 + erf(x * sqrt(0.5)) * 0.5) runs on float16 tensors
+// (python/tvm/relax/transform/legalize_ops.py:495-503): every operation rounded once, the constants rounded
+// to float16 first, erf evaluated in float32 and rounded.
+__device__ __forceinline__ half_t gelu_f16(half_t h) {
+  const half_t a = h * (half_t)0.70710678118654752440f;
+  const half_t e = (half_t)erff((float)a);
+  const half_t b = e * (half_t)0.5f;
+  const half_t c = (half_t)0.5f + b;
+  return h * c;
+}
 
 // Gated tail of a fused gate+up projection.  The weight matrix holds the gate rows 0 .. N/2-1 and the up
 // rows N/2 .. N-1; kernels that fuse the tail walk the rows in the interleaved order
@@ -175,11 +187,15 @@ __device__ __forceinline__ void store_gated(half_t* y, int m, int j, int half_n,
   y[(size_t)m * half_n + j] = silu_mul((half_t)acc_gate, (half_t)acc_up);
 }
 
+// (GELU = false: a build without the gelu branch, for kernels whose register budget it would break;
+// their launcher applies gelu in a pass of its own)
+template <bool GELU = true>
 __device__ __forceinline__ void store_out(const Epilogue& ep, half_t* y, int m, int n, int N, float acc) {
   half_t h = (half_t)acc;
   const size_t idx = (size_t)m * N + n;
   if (ep.bias != nullptr) h = h + ep.bias[n];
   if (ep.activation == 1) h = h > (half_t)0 ? h : (half_t)0;  // max(h, 0) as select(h > 0, h, 0)
+  if (GELU && ep.activation == kActGelu) h = gelu_f16(h);
   if (ep.residual != nullptr) h = h + ep.residual[idx];
   y[idx] = h;
 }
@@ -195,6 +211,7 @@ __device__ __forceinline__ bool pair_store_ok(const Epilogue& ep, const half_t* 
 
 // Columns n (even) and n + 1 of row m; `paired` comes from pair_store_ok.  Same per-element
 // arithmetic as store_out.
+template <bool GELU = true>
 __device__ __forceinline__ void store_out2(const Epilogue& ep, half_t* y, int m, int n, int N, float a0, float a1,
                                            bool paired) {
   if (paired && n + 1 < N) {
@@ -205,11 +222,12 @@ __device__ __forceinline__ void store_out2(const Epilogue& ep, half_t* y, int m,
       h[0] = h[0] > (half_t)0 ? h[0] : (half_t)0;
       h[1] = h[1] > (half_t)0 ? h[1] : (half_t)0;
     }
+    if (GELU && ep.activation == kActGelu) h = half2_t{gelu_f16(h[0]), gelu_f16(h[1])};
     if (ep.residual != nullptr) h = h + *reinterpret_cast<const half2_t*>(ep.residual + idx);
     *reinterpret_cast<half2_t*>(y + idx) = h;
   } else {
-    if (n < N) store_out(ep, y, m, n, N, a0);
-    if (n + 1 < N) store_out(ep, y, m, n + 1, N, a1);
+    if (n < N) store_out<GELU>(ep, y, m, n, N, a0);
+    if (n + 1 < N) store_out<GELU>(ep, y, m, n + 1, N, a1);
   }
 }
 

@@ -11,6 +11,7 @@
 //
 // LDS rows are padded by 16 bytes (row stride 144 B) so that the 16-byte operand
 // reads of 8 consecutive lanes cover all banks once.
+#include <algorithm>
 #include <atomic>
 #include "wq_device.h"
 #include "wq_internal.h"
@@ -211,12 +212,59 @@ bool launch_one(const Problem& p, int group_shift) {
 
 }  // namespace
 
+namespace {
+
+// y = gelu(y) [+ residual], element by element: the second pass of a gelu tail behind the direct-weight
+// kernel, which is built without the gelu branch (its 128 accumulator registers leave no room for it).
+// The float16 value the first pass stored is the value the fused form would have handed to gelu.
+__global__ __launch_bounds__(256) void wq_gelu_tail_kernel(half_t* __restrict__ y, const half_t* __restrict__ residual,
+                                                           int64_t count) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
+    half_t h = gelu_f16(y[i]);
+    if (residual != nullptr) h = h + residual[i];
+    y[i] = h;
+  }
+}
+
+int launch_gemm_any(const Problem& p, int variant, bool direct_ok);
+
+}  // namespace
+
 int launch_gemm(const Problem& p, int variant) {
+  if (p.activation != kActGelu) return launch_gemm_any(p, variant, true);
+  // gelu: fused by the LDS-staged kernels; behind the direct-weight kernel as a pass of its own -- unless the
+  // residual is the output buffer itself, which the first pass would overwrite: then the fused kernels run.
+  if (p.residual == p.y) return launch_gemm_any(p, variant, false);
+  Problem first = p;
+  first.activation = 0;
+  first.residual = nullptr;
+  const int rc = launch_gemm_any(first, variant, true);
+  if (rc != 0) return rc;
+  const int64_t count = p.m * p.n;
+  const int blocks = (int)std::min<int64_t>((count + 255) / 256, (int64_t)cu_count() * 8);
+  hipLaunchKernelGGL(wq_gelu_tail_kernel, dim3(blocks), dim3(256), 0, p.stream, (half_t*)p.y, (const half_t*)p.residual, count);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("gelu tail kernel launch failed: %s", hipGetErrorString(e));
+    return -1;
+  }
+  return 0;
+}
+
+namespace {
+
+int launch_gemm_any(const Problem& p, int variant, bool direct_ok) {
   const int ch = 128 / p.bits;
   int ratio = p.group / ch, group_shift = 0;
   while ((1 << group_shift) < ratio) ++group_shift;
   if (ratio < 1 || (1 << group_shift) != ratio || p.group % ch != 0) {
     set_error("gemm kernel: group %d must be %d times a power of two", p.group, ch);
+    return -1;
+  }
+  if (!direct_ok && (p.tiled || variant >= 21)) {
+    set_error("gemm kernel: gelu with the residual in the output buffer is not available on the direct-weight kernel "
+              "(tile-major weights, variants 21..26); pass the residual in a buffer of its own");
     return -1;
   }
   if (p.tiled) {
@@ -238,6 +286,8 @@ int launch_gemm(const Problem& p, int variant) {
       return -1;
     }
     variant = -1;
+  } else if (variant == 0 && gemm_pipe_applicable(p) && !direct_ok) {
+    variant = p.m >= 1024 ? 11 : 12;
   } else if (variant == 0 && gemm_pipe_applicable(p)) {
     // Measured on MI355X, M = 128 .. 4096 on the Llama shapes: the direct-weight kernel with two
     // K groups wins wherever it applies -- with 64-row tiles while 128-row tiles would leave
@@ -307,5 +357,7 @@ int launch_gemm(const Problem& p, int variant) {
   }
   return 0;
 }
+
+}  // namespace
 
 }  // namespace wq

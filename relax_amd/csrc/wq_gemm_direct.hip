@@ -624,7 +624,7 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int m = mrow0 + i * 32 + (v >> 2) * 8 + fh * 4 + (v & 3);
-      if (i < nrb && m < M) store_out2(ep, y, m, n, N, acc[i][0][v], acc[i][1][v], paired);
+      if (i < nrb && m < M) store_out2<false>(ep, y, m, n, N, acc[i][0][v], acc[i][1][v], paired);
     }
 }
 
@@ -683,7 +683,7 @@ bool launch_split_bits(const Problem& p, int group_shift, int ksplit, void* work
 // only from eight macro steps on, with at least four windows and tiles on at most an eighth of the CUs.
 int gemm_split_ways(const Problem& p) {
   if (p.m <= 64 || p.k % 256 != 0 || p.group != (p.bits == 4 ? 32 : 128) || !gemm_pipe_applicable(p)) return 1;
-  if (p.activation == kActGated) return 1;
+  if (p.activation == kActGated || p.activation == kActGelu) return 1;
   const int64_t cu = cu_count(), tiles = ((p.m + 127) / 128) * ((p.n + 255) / 256), macro = p.k / 256;
   if (tiles * (p.bits == 4 ? 8 : 2) > cu || tiles > kGemmSplitMaxTiles) return 1;
   const int64_t ways = std::min<int64_t>({cu / tiles, macro / (p.bits == 4 ? 8 : 4), 8});

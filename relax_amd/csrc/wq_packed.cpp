@@ -310,6 +310,8 @@ MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_bias, 0, 4, 7, 1, 0, 0)
 MI355X_FIXED_ENTRY(mi355x_q8f16_matmul_bias, 0, 8, 0, 1, 0, 0)
 MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_bias_relu, 0, 4, 7, 1, 0, MI355X_WQ_ACT_RELU)
 MI355X_FIXED_ENTRY(mi355x_q8f16_matmul_bias_relu, 0, 8, 0, 1, 0, MI355X_WQ_ACT_RELU)
+MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_bias_gelu, 0, 4, 7, 1, 0, MI355X_WQ_ACT_GELU)
+MI355X_FIXED_ENTRY(mi355x_q8f16_matmul_bias_gelu, 0, 8, 0, 1, 0, MI355X_WQ_ACT_GELU)
 MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_residual, 0, 4, 7, 0, 1, 0)
 MI355X_FIXED_ENTRY(mi355x_q8f16_matmul_residual, 0, 8, 0, 0, 1, 0)
 MI355X_FIXED_ENTRY(mi355x_q4f16_matmul_silu_mul, 0, 4, 7, 0, 0, MI355X_WQ_ACT_SILU_MUL)
@@ -480,6 +482,8 @@ int mi355x_wq_register_tvm_globals(int allow_override) {
                            {"mi355x.q8f16_matmul_bias", mi355x_q8f16_matmul_bias},
                            {"mi355x.q4f16_matmul_bias_relu", mi355x_q4f16_matmul_bias_relu},
                            {"mi355x.q8f16_matmul_bias_relu", mi355x_q8f16_matmul_bias_relu},
+                           {"mi355x.q4f16_matmul_bias_gelu", mi355x_q4f16_matmul_bias_gelu},
+                           {"mi355x.q8f16_matmul_bias_gelu", mi355x_q8f16_matmul_bias_gelu},
                            {"mi355x.q4f16_matmul_residual", mi355x_q4f16_matmul_residual},
                            {"mi355x.q8f16_matmul_residual", mi355x_q8f16_matmul_residual},
                            {"mi355x.q4f16_matmul_silu_mul", mi355x_q4f16_matmul_silu_mul},

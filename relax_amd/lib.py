@@ -9,8 +9,9 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 SO_PATH = os.path.join(CSRC, "libmi355x_wq.so")
 
 KERNEL_AUTO, KERNEL_GEMV, KERNEL_GEMM, KERNEL_SKINNY = 0, 1, 2, 3
-ACT_NONE, ACT_RELU, ACT_SILU_MUL = 0, 1, 2
-ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "relax.nn.relu": ACT_RELU, "silu_mul": ACT_SILU_MUL}
+ACT_NONE, ACT_RELU, ACT_SILU_MUL, ACT_GELU = 0, 1, 2, 3
+ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "relax.nn.relu": ACT_RELU, "silu_mul": ACT_SILU_MUL,
+               "gelu": ACT_GELU, "relax.nn.gelu": ACT_GELU}
 
 # every symbol include/mi355x_wq.h, include/mi355x_wq_packed.h and include/mi355x_wq_module.h declare
 EXPORTED_SYMBOLS = (
@@ -21,7 +22,8 @@ EXPORTED_SYMBOLS = (
     "mi355x_wq_select_kernel", "mi355x_wq_last_error", "mi355x_wq_version",
     "mi355x_q4f16_matmul", "mi355x_q8f16_matmul", "mi355x_q4f16_matmul_bias", "mi355x_q8f16_matmul_bias",
     "mi355x_q4f16_matmul_bias_relu", "mi355x_q8f16_matmul_bias_relu", "mi355x_q4f16_matmul_residual",
-    "mi355x_q8f16_matmul_residual", "mi355x_q4f16_matmul_silu_mul", "mi355x_q8f16_matmul_silu_mul", "mi355x_q4f16_dequantize",
+    "mi355x_q8f16_matmul_residual", "mi355x_q4f16_matmul_bias_gelu", "mi355x_q8f16_matmul_bias_gelu",
+    "mi355x_q4f16_matmul_silu_mul", "mi355x_q8f16_matmul_silu_mul", "mi355x_q4f16_dequantize",
     "mi355x_q8f16_dequantize", "mi355x_q4f16_tile_weights", "mi355x_q8f16_tile_weights",
     "mi355x_q4f16_matmul_tiled", "mi355x_q8f16_matmul_tiled", "mi355x_q4f16_matmul_ws", "mi355x_q8f16_matmul_ws",
     "mi355x_wq_packed_call", "mi355x_wq_packed_call_scratch", "mi355x_wq_packed_set_stream",

@@ -26,7 +26,7 @@ def wq_matmul(x: torch.Tensor, wq: torch.Tensor, scales: torch.Tensor, bits: int
     """y[M,N] = f16(x[M,K] @ dequant(wq, scales)^T) on the current HIP device (asynchronous).
 
     Optional fused epilogue, each step one float16 operation: ``+ bias[N]``, then ``activation``
-    ("relu"), then ``+ residual[M,N]`` (``residual`` may be ``out`` itself); or ``activation="silu_mul"``
+    ("relu" or "gelu"), then ``+ residual[M,N]`` (``residual`` may be ``out`` itself); or ``activation="silu_mul"``
     alone: the output is ``[M, N/2] = multiply(nn.silu(y[:, :N/2]), y[:, N/2:])``.
 
     ``tiled_n=N``: ``wq`` and ``scales`` are the tile-major buffers `wq_tile_weights` returns

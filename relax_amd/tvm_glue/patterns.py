@@ -9,7 +9,7 @@ The composite the backend takes over is the idiomatic weight-only-quantized line
 
 optionally followed by the element-wise tail the reference's `make_matmul_pattern(with_bias,
 activation)` describes for its CUTLASS backend (python/tvm/relax/dpl/pattern.py:1049-1095:
-`add`, then `relax.nn.relu`), and by the residual add of a decoder layer:
+`add`, then `relax.nn.relu` or `relax.nn.gelu`), and by the residual add of a decoder layer:
 
     y = R.add(y, bias)            # bias [N] or [1, N]
     y = R.nn.relu(y)
@@ -61,13 +61,16 @@ def patterns():
         base = f"{BACKEND}.q{q['bits']}f16_matmul"
         add1 = lambda: is_op("relax.add")(core(fn_name), wildcard())  # noqa: E731
         relu = lambda: is_op("relax.nn.relu")(add1())                 # noqa: E731
+        gelu = lambda: is_op("relax.nn.gelu")(add1())                 # noqa: E731
         halves = lambda: is_op("relax.split")(core(fn_name)).has_attr({"indices_or_sections": 2})  # noqa: E731
         gated = is_op("relax.multiply")(is_op("relax.nn.silu")(is_tuple_get_item(halves(), 0)),
                                         is_tuple_get_item(halves(), 1))
         table.append((base + "_silu_mul", gated))
         table.append((base + "_add_relu_add", is_op("relax.add")(relu(), wildcard())))
         table.append((base + "_add_add", is_op("relax.add")(add1(), wildcard())))
+        table.append((base + "_add_gelu_add", is_op("relax.add")(gelu(), wildcard())))
         table.append((base + "_add_relu", relu()))
+        table.append((base + "_add_gelu", gelu()))
         table.append((base + "_add", add1()))
         table.append((base, core(fn_name)))
     return table

@@ -122,7 +122,7 @@ def quantized_linear(decode="decode_q4f16", m=4, n=48, k=128, tail=(), outer_ord
                      symbol="fused_mi355x", golden_names=False):
     """The annotated function FuseOpsByPattern(annotate_codegen=True) produces for
     decode -> permute_dims -> matmul -> astype followed by `tail`, a sequence of
-    ("add", shape) / ("relu",) steps.  Composite parameters are ordered by first use:
+    ("add", shape) / ("relu",) / ("gelu",) steps.  Composite parameters are ordered by first use:
     (wq, scales, x, <tail operands in order>).  `outer_order` permutes the outer parameters.
     `bound` names operands ("wq", "scales", "operand<i>") that BindParams turned into constants: they sit
     inside the composite as Constant nodes and are no parameters."""
@@ -166,7 +166,7 @@ def quantized_linear(decode="decode_q4f16", m=4, n=48, k=128, tail=(), outer_ord
             args = [cur, operand] if len(step) < 3 or not step[2] else [operand, cur]
             binds.append(VarBinding(nxt, Call(Op("relax.add"), args)))
         else:
-            binds.append(VarBinding(nxt, Call(Op("relax.nn.relu"), [cur])))
+            binds.append(VarBinding(nxt, Call(Op("relax.nn." + step[0]), [cur])))
         cur = nxt
     name = "mi355x.q4f16_matmul" if "q4" in decode else "mi355x.q8f16_matmul"
     # The shape of the reference's golden for FuseOpsByPattern(annotate_codegen=True)
@@ -192,7 +192,7 @@ def fused_name(decode, tail=()):
     added to the module (include/tvm/relax/utils.h:49-50).  With annotate_codegen the outer function's symbol
     is that name + "_" + backend (src/relax/transform/fuse_ops.cc:1007-1010)."""
     parts = ["fused", decode, "relax.permute_dims", "relax.matmul", "relax.astype"]
-    parts += ["relax.add" if step[0] == "add" else "relax.nn.relu" for step in tail]
+    parts += ["relax.add" if step[0] == "add" else "relax.nn." + step[0] for step in tail]
     return "_".join(parts).replace(".", "_")
 
 

@@ -27,7 +27,7 @@ def declared_symbols():
 def test_library_exports_every_declared_symbol():
     L = lib.load()
     names = declared_symbols()
-    assert len(names) == 55 and set(names) == set(lib.EXPORTED_SYMBOLS)
+    assert len(names) == 57 and set(names) == set(lib.EXPORTED_SYMBOLS)
     for n in names:
         assert hasattr(L, n), n
     assert L.mi355x_wq_version() >= 100
@@ -322,7 +322,7 @@ assert L.mi355x_wq_register_tvm_globals(0) == -1 and "no TVM runtime" in lib.las
 fake = C.CDLL({fake!r}, mode=C.RTLD_GLOBAL)
 fake.fake_tvm_name.restype = C.c_char_p
 fake.fake_tvm_last_error.restype = C.c_char_p
-assert L.mi355x_wq_register_tvm_globals(0) == 18
+assert L.mi355x_wq_register_tvm_globals(0) == 20
 names = sorted(fake.fake_tvm_name(i).decode() for i in range(fake.fake_tvm_count()))
 assert names == sorted("mi355x." + s[len("mi355x_"):] for s in lib.PACKED_ENTRIES), names
 # call a registered function the way the registry would, with host tensors: it must fail and the

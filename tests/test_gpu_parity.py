@@ -528,7 +528,7 @@ def test_fused_argument_checks():
     x, wq, s, g = O.make_case(1, 2, 32, 64, 4)
     xd, wd, sd = _dev(x), _dev(wq), _dev(s)
     with pytest.raises(ValueError, match="unsupported activation"):
-        relax_amd.wq_matmul(xd, wd, sd, 4, g, activation="gelu")
+        relax_amd.wq_matmul(xd, wd, sd, 4, g, activation="tanh")
     with pytest.raises(ValueError, match="bias must be"):
         relax_amd.wq_matmul(xd, wd, sd, 4, g, bias=torch.zeros(31, dtype=torch.float16, device="cuda"))
     with pytest.raises(ValueError, match="residual must be"):

@@ -330,7 +330,7 @@ def test_relu_special_values_and_epilogue_order():
     for impl in (O, c_oracle):
         assert np.array_equal(impl.epilogue(y, bias=b, residual=r), r + b[None, :])
     with pytest.raises(ValueError):
-        O.epilogue(y, activation="gelu")
+        O.epilogue(y, activation="tanh")
 
 
 @pytest.mark.parametrize("bits,m,n,k", [(4, 3, 40, 128), (8, 5, 24, 256)])
@@ -472,3 +472,58 @@ def test_silu_mul_every_step_against_exact_rationals():
         t = nearest(gf * s)
         want = nearest(t * uf)
         assert Fraction(float(got_np[i])) == want and Fraction(float(got_c[i])) == want, (g[i], u[i])
+
+
+# ------------------------------------------------------------------ gelu (float16 operation sequence)
+def test_gelu_python_and_c_oracles_agree_on_every_float16():
+    h = np.arange(65536, dtype=np.uint16).view(np.float16)
+    x = h[np.isfinite(h)].reshape(1, -1)
+    a = O.epilogue(x, activation="gelu")
+    b = c_oracle.epilogue(x, activation="gelu")
+    assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+
+
+def test_gelu_closed_form_bound_on_every_float16():
+    """x * Phi(x) in float64 against the float16 sequence x * (0.5 + erf(x * sqrt(0.5)) * 0.5).  Error budget of
+    the sequence: the argument a = x * sqrt(0.5) carries a relative 2^-10 (constant and product rounded), which
+    erf turns into at most (2/sqrt(pi)) |a| exp(-a^2) 2^-10 <= 0.484 * 2^-10; e adds 2^-12; halving is exact;
+    c = 0.5 + b adds 2^-12: |c - Phi(x)| <= 0.5 (0.484 * 2^-10 + 2^-12) + 2^-12 < 2.5 * 2^-12, and the final
+    product half a float16 ulp.  (For x < -1 the sum 0.5 + b cancels, so the sequence is far from x * Phi(x)
+    in relative terms: that is a property of the legalized form, not of this restatement.)  A wrong constant,
+    sign or a dropped term misses the bound by orders of magnitude."""
+    import math
+
+    h = np.arange(65536, dtype=np.uint16).view(np.float16)
+    x = h[np.isfinite(h)]
+    got = O.gelu_f16(x).astype(np.float64)
+    xf = x.astype(np.float64)
+    exact = xf * 0.5 * (1.0 + np.vectorize(math.erf)(xf / math.sqrt(2.0)))
+    ok = np.abs(exact) < 65504.0
+    ulp = np.spacing(np.abs(exact[ok]).astype(np.float16)).astype(np.float64)
+    bound = np.abs(xf[ok]) * 2.5 * 2.0 ** -12 + 0.5 * ulp + 2.0 ** -25
+    assert np.all(np.abs(got[ok] - exact[ok]) <= bound)
+    # the bound is not slack by orders of magnitude: some input uses more than half of it
+    assert (np.abs(got[ok] - exact[ok]) / bound).max() > 0.5
+    # mistakes the bound catches: sqrt(0.5) replaced by 0.5, the sign of erf, the missing 0.5 +
+    for wrong in (xf * 0.5 * (1.0 + np.vectorize(math.erf)(xf * 0.5)),
+                  xf * 0.5 * (1.0 - np.vectorize(math.erf)(xf / math.sqrt(2.0))),
+                  xf * 0.5 * np.vectorize(math.erf)(xf / math.sqrt(2.0))):
+        assert not np.all(np.abs(wrong[ok] - exact[ok]) <= bound)
+
+
+def test_gelu_special_values_and_position_in_the_tail():
+    f = np.float16
+    x = np.array([[0.0, -0.0, 1.0, -1.0, 10.0, -10.0, np.inf, np.nan, 6e-8]], dtype=f)
+    y = O.epilogue(x, activation="gelu")
+    assert y[0, 0] == 0 and not np.signbit(y[0, 0]) and y[0, 1] == 0 and np.signbit(y[0, 1])
+    assert y[0, 2] == f(0.8413) and y[0, 3] == f(-0.1587)
+    assert y[0, 4] == f(10.0) and y[0, 5] == 0 and np.signbit(y[0, 5])  # c rounds to 1 / to 0
+    assert np.isinf(y[0, 6]) and np.isnan(y[0, 7])
+    assert y[0, 8] == f(6e-8) * f(0.5)
+    # bias first, gelu second, residual last
+    t = np.array([[0.5, -2.0]], dtype=f)
+    bias = np.array([0.5, 1.0], dtype=f)
+    res = np.array([[1.0, 1.0]], dtype=f)
+    want = O.add_f16(O.gelu_f16(O.add_f16(t, bias.reshape(1, -1))), res)
+    assert np.array_equal(O.epilogue(t, bias, "gelu", res), want)
+    assert np.array_equal(c_oracle.epilogue(t, bias, "gelu", res), want)

@@ -137,6 +137,13 @@ def test_roles_of_plain_and_fused_composites(fake_tvm):
     s = spec_from_function(fake_tvm.quantized_linear(tail=[("add", [n]), ("relu",), ("add", [m, n])]))
     assert (s.arg_bias, s.arg_residual, s.activation, s.arg_out, s.num_args) == (3, 4, ACT_RELU, 5, 6)
     s.validate()
+    # gelu behind the bias (the *_bias_gelu members of the reference's table), with and without a residual
+    from relax_amd.tvm_glue.codegen import ACT_GELU
+    s = spec_from_function(fake_tvm.quantized_linear("decode_q8f16", tail=[("add", [n]), ("gelu",)]))
+    assert (s.arg_bias, s.arg_residual, s.activation, s.arg_out) == (3, -1, ACT_GELU, 4)
+    s = spec_from_function(fake_tvm.quantized_linear(tail=[("add", [n]), ("gelu",), ("add", [m, n])]))
+    assert (s.arg_bias, s.arg_residual, s.activation, s.arg_out, s.num_args) == (3, 4, ACT_GELU, 5, 6)
+    s.validate()
     # outer parameters in another order: roles follow the call arguments, not the positions
     s = spec_from_function(fake_tvm.quantized_linear(tail=[("add", [n])], outer_order=[2, 3, 0, 1]))
     assert (s.arg_x, s.arg_bias, s.arg_wq, s.arg_scales, s.arg_out) == (0, 1, 2, 3, 4)
@@ -152,6 +159,10 @@ def test_role_derivation_rejects_tails_the_epilogue_cannot_express(fake_tvm):
         spec_from_function(fake_tvm.quantized_linear(tail=[("add", [m, n]), ("relu",)]))
     with pytest.raises(ValueError, match="only fused between"):
         spec_from_function(fake_tvm.quantized_linear(tail=[("relu",), ("relu",)]))
+    with pytest.raises(ValueError, match="gelu is only fused between"):
+        spec_from_function(fake_tvm.quantized_linear(tail=[("relu",), ("gelu",)]))
+    with pytest.raises(ValueError, match="gelu is only fused between"):
+        spec_from_function(fake_tvm.quantized_linear(tail=[("add", [m, n]), ("gelu",)]))
     f = fake_tvm.quantized_linear()
     f.body.blocks[0].bindings[0].value.attrs["Composite"] = "cutlass.matmul"
     with pytest.raises(ValueError, match="does not belong to backend"):
@@ -294,6 +305,8 @@ def test_annotated_function_in_the_shape_of_the_reference_golden(fake_tvm):
     # the q8 flavour and a fused tail get their own names
     assert fake_tvm.fused_name("decode_q8f16", [("add", [48]), ("relu",)]) == \
         "fused_decode_q8f16_relax_permute_dims_relax_matmul_relax_astype_relax_add_relax_nn_relu"
+    assert fake_tvm.fused_name("decode_q4f16", [("add", [48]), ("gelu",)]) == \
+        "fused_decode_q4f16_relax_permute_dims_relax_matmul_relax_astype_relax_add_relax_nn_gelu"
 
 
 def test_call_form_after_run_codegen_matches_the_call_description(fake_tvm):
