@@ -63,6 +63,71 @@ def measured_traffic():
     return int(traffic.group(1))
 
 
+class ClockSampler:
+    """Reads the GPU's current shader clock and board power from sysfs (read only) every 50 ms on a host
+    thread while a workload runs.  The datasheet MFMA rate is quoted at the peak engine clock; what a
+    kernel can reach is set by the clock the power management sustains under that kernel."""
+
+    def __init__(self):
+        import glob
+        self.sclk = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))[:1]
+        self.power = (sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average")) +
+                      sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")))[:1]
+        self.samples, self._stop, self._thread = [], False, None
+
+    def _read(self):
+        mhz = watts = None
+        try:
+            for line in open(self.sclk[0]):
+                if "*" in line:
+                    mhz = float(line.split(":")[1].strip().lower().split("mhz")[0])
+            watts = int(open(self.power[0]).read()) / 1e6 if self.power else None
+        except (OSError, ValueError, IndexError):
+            pass
+        return mhz, watts
+
+    def __enter__(self):
+        import threading
+
+        def loop():
+            while not self._stop:
+                self.samples.append((time.time(),) + self._read())
+                time.sleep(0.05)
+        if self.sclk:
+            self._thread = threading.Thread(target=loop, daemon=True)
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        if self._thread is not None:
+            self._thread.join()
+
+    def steady(self, since):
+        """Median clock (MHz) and power (W) of the samples taken after `since` (time.time()); None if unreadable."""
+        mhz = sorted(c for t, c, _ in self.samples if t >= since and c is not None)
+        watts = sorted(w for t, _, w in self.samples if t >= since and w is not None)
+        return (mhz[len(mhz) // 2] if mhz else None, watts[len(watts) // 2] if watts else None)
+
+
+def sustained(torch, fn, work_per_call, seconds=1.5):
+    """Runs fn back to back for `seconds`, sampling clock and power; returns work per second, clock and power
+    over the second half of the run."""
+    with ClockSampler() as sampler:
+        t_begin = time.time()
+        while time.time() - t_begin < seconds / 2:
+            fn()
+            torch.cuda.synchronize()
+        t_mid, calls = time.time(), 0
+        while time.time() - t_mid < seconds / 2:
+            fn()
+            calls += 1
+            torch.cuda.synchronize()
+        elapsed = time.time() - t_mid
+    mhz, watts = sampler.steady(t_mid)
+    return work_per_call * calls / elapsed, mhz, watts
+
+
 def algorithmic_bytes(bits: int, group: int, m: int, n: int, k: int) -> int:
     return n * k * bits // 8 + n * (k // group) * 2 + 2 * m * k + 2 * m * n
 
@@ -157,6 +222,29 @@ def config_table(torch, dev, args) -> int:
                 torch.cuda.synchronize()
             times[tiled] = e0.elapsed_time(e1) * 1e3 / (reps * sets)
             del g
+        # with a caller workspace, where the library would split K across workgroups for this problem
+        need = relax_amd.wq_workspace_bytes(bits, group, n, k, m)
+        us_ws = None
+        if need > 0:
+            wsp = relax_amd.wq_workspace(need)
+            with torch.cuda.stream(stream):
+                for wq, s in ws:
+                    relax_amd.wq_matmul(x, wq, s, bits, group, out=y, workspace=wsp)
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    for wq, s in ws:
+                        relax_amd.wq_matmul(x, wq, s, bits, group, out=y, workspace=wsp)
+                g.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(reps):
+                    g.replay()
+                e1.record(stream)
+                torch.cuda.synchronize()
+            us_ws = e0.elapsed_time(e1) * 1e3 / (reps * sets)
+            del g, wsp
         us = times[False]
         ab = algorithmic_bytes(bits, group, m, n, k)
         fl = 2.0 * m * n * k
@@ -165,7 +253,9 @@ def config_table(torch, dev, args) -> int:
                     lib.load().mi355x_wq_select_kernel(lib.make_desc(bits, group, n, k), m)],
                 "GB/s": round(ab / us / 1e3, 0), "frac_hbm": round(ab / us / 1e3 / HBM_PEAK_GBS, 3),
                 "TFLOP/s": round(fl / us / 1e6, 1), "frac_mfma": round(fl / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 3),
-                "us_tile_major": round(times[True], 2), "tile_major_speedup": round(us / times[True], 3)}
+                "us_tile_major": round(times[True], 2), "tile_major_speedup": round(us / times[True], 3),
+                "us_with_workspace": None if us_ws is None else round(us_ws, 2),
+                "workspace_speedup": None if us_ws is None else round(us / us_ws, 3)}
         print(json.dumps(line), flush=True)
         del ws, wt
     return 0
@@ -183,6 +273,8 @@ def main() -> int:
     ap.add_argument("--no-ksplit", action="store_true", help="skip the caller-workspace (K split) leg")
     ap.add_argument("--no-tiled", action="store_true", help="skip the tile-major-weights decode leg")
     ap.add_argument("--no-streams", action="store_true", help="skip the two-stream (two independent chains) leg")
+    ap.add_argument("--no-sustained", action="store_true",
+                    help="skip the sustained-load segments that sample clock and power (use under a profiler)")
     ap.add_argument("--configs", action="store_true",
                     help="instead of the benchmark: time every shape of the decode, prefill and q8f16 "
                          "configurations on its own (weights rotated through more than 512 MB, one HIP "
@@ -287,6 +379,11 @@ def main() -> int:
                      "avg_launch_us": round(avg_launch_us, 3)},
     }
     result["roofline"]["traffic"] = measured_traffic()
+    # the clock and board power the decode step sustains (memory bound: the clock stays at its peak)
+    if not args.no_sustained:
+        with torch.cuda.stream(stream):
+            rate, mhz, watts = sustained(torch, graph.replay, bytes_per_step, seconds=1.0)
+        result["roofline"]["sustained"] = {"gbs": round(rate / 1e9, 1), "sclk_mhz": mhz, "power_w": watts}
 
     # ---- the same decode step on tile-major weights (the one-off layout transform applied at load) ----
     if not args.no_tiled:
@@ -387,6 +484,23 @@ def main() -> int:
                           "library_f16_gemm_tflops": round(flops / (lms * 1e-3) / 1e12, 1),
                           "library_f16_gemm_note": "torch.matmul (hipBLASLt) on float16 weights dequantized "
                                                    "beforehand, same shapes and data, timed alternately"}
+        # Sustained load, with the clock the power management holds under each kernel: the datasheet rate
+        # assumes the peak engine clock (2400 MHz); `frac_of_peak_at_clock` prices the kernel against the
+        # rate the matrix pipes have at the clock it actually ran at.
+        PEAK_MHZ = 2400.0
+        rate = lrate = 0.0
+        mhz = watts = lmhz = lwatts = None
+        if not args.no_sustained:
+            with torch.cuda.stream(stream):
+                rate, mhz, watts = sustained(torch, prefill_pass, flops)
+                lrate, lmhz, lwatts = sustained(torch, library_pass, flops)
+        result["gemm"]["sustained"] = None if args.no_sustained else {
+            "tflops": round(rate / 1e12, 1), "sclk_mhz": mhz, "power_w": watts,
+            "frac_of_peak_at_clock": round(rate / 1e12 / (MFMA_F16_PEAK_TFLOPS * mhz / PEAK_MHZ), 4) if mhz else None,
+            "library_tflops": round(lrate / 1e12, 1), "library_sclk_mhz": lmhz, "library_power_w": lwatts,
+            "library_frac_of_peak_at_clock": round(lrate / 1e12 / (MFMA_F16_PEAK_TFLOPS * lmhz / PEAK_MHZ), 4) if lmhz else None,
+            "note": "1.5 s of back-to-back passes each; clock and power are sysfs readings (pp_dpm_sclk, "
+                    "hwmon power1_*), median over the second half"}
         if ours_tiled:
             result["gemm"]["tile_major_tflops"] = round(flops / (sum(ours_tiled) / len(ours_tiled) * 1e-3) / 1e12, 1)
         result["roofline_gemm"] = {"bound": "mfma", "achieved": round(tflops, 1),
