@@ -518,32 +518,37 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     __syncthreads();
     if (!*last) return;
     if (threadIdx.x == 0) __hip_atomic_store(&counters[tile_lin], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    // The K groups share the sum: each takes TM / GROUPS of the tile's row blocks (every wavefront of the
-    // workgroup reads; holding two windows in flight measured no faster) and finishes those rows itself.
-    constexpr int RG = (TM % GROUPS == 0) ? GROUPS : 1;
-    if (RG == 1 && !owner) return;
-    nrb = TM / RG;
-    const int i0 = RG == 1 ? 0 : grp * (TM / RG);
+    // The K groups share the sum: the first RG of them take TM / RG of the tile's row blocks each and finish
+    // those rows themselves.  With one row block per group four windows' vectors are in flight together
+    // (one trip to the memory side instead of S); with two, one window at a time (two measured no faster).
+    constexpr int RG = (TM % GROUPS == 0) ? GROUPS : ((GROUPS % TM == 0) ? TM : 1);
+    constexpr int RPG = TM / RG;           // row blocks per reducing group
+    constexpr int WIN = RPG == 1 ? 4 : 1;  // windows in flight
+    if (grp >= RG) return;
+    nrb = RPG;
+    const int i0 = grp * RPG;
     mrow0 = m0 + i0 * 32;
 #pragma unroll
-    for (int i = 0; i < TM / RG; ++i)
+    for (int i = 0; i < RPG; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-    auto load_window = [&](int q, u32x4 (&buf)[TM / RG][2][4]) {
+    auto load_window = [&](int q, u32x4 (&buf)[RPG][2][4]) {
+      // (windows past the last read zeros: the offset is out of the buffer's range)
+      const uint32_t base = q < S ? (uint32_t)(q * WAVES + wave) * (TM * 8) * 1024u : kRowOobD;
 #pragma unroll
-      for (int i = 0; i < TM / RG; ++i)
+      for (int i = 0; i < RPG; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
           for (int v4 = 0; v4 < 4; ++v4)
             buf[i][j][v4] = __builtin_amdgcn_raw_buffer_load_b128(
-                rp, ((uint32_t)(q * WAVES + wave) * (TM * 8) + ((i0 + i) * 2 + j) * 4 + v4) * 1024u + lane * 16u, 0, 0x10);
+                rp, base + (((i0 + i) * 2 + j) * 4 + v4) * 1024u + lane * 16u, 0, 0x10);
     };
-    auto add_window = [&](const u32x4 (&buf)[TM / RG][2][4]) {
+    auto add_window = [&](const u32x4 (&buf)[RPG][2][4]) {
 #pragma unroll
-      for (int i = 0; i < TM / RG; ++i)
+      for (int i = 0; i < RPG; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -553,10 +558,12 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
             for (int e = 0; e < 4; ++e) acc[i][j][v4 * 4 + e] += o[e];
           }
     };
-    u32x4 win[TM / RG][2][4];
-    for (int q = 0; q < S; ++q) {  // windows are added in their order, whoever arrived last
-      load_window(q, win);
-      add_window(win);
+    u32x4 win[WIN][RPG][2][4];
+    for (int q = 0; q < S; q += WIN) {  // windows are added in their order, whoever arrived last
+#pragma unroll
+      for (int w = 0; w < WIN; ++w) load_window(q + w, win[w]);
+#pragma unroll
+      for (int w = 0; w < WIN; ++w) add_window(win[w]);  // (+ 0.0 for a window past the last: no change)
     }
   }
 
@@ -666,12 +673,19 @@ bool launch_bits(const Problem& p, int group_shift, int tile_n0 = 0, int tile_co
                      : launch_direct<8, GROUPS, TM, WAVES, false>(p, group_shift, tile_n0, tile_count);
 }
 
-bool launch_split_bits(const Problem& p, int group_shift, int ksplit, void* workspace) {
+// The K-split builds: 128 x 256 tiles with two K groups above 64 rows, 64 x 128 tiles with four K groups up to 64.
+template <int GROUPS, int TM, int WAVES>
+bool launch_split_shape(const Problem& p, int group_shift, int ksplit, void* workspace) {
   if (p.tiled)
-    return p.bits == 4 ? launch_direct<4, 2, 4, 4, true, true>(p, group_shift, 0, -1, ksplit, workspace)
-                       : launch_direct<8, 2, 4, 4, true, true>(p, group_shift, 0, -1, ksplit, workspace);
-  return p.bits == 4 ? launch_direct<4, 2, 4, 4, false, true>(p, group_shift, 0, -1, ksplit, workspace)
-                     : launch_direct<8, 2, 4, 4, false, true>(p, group_shift, 0, -1, ksplit, workspace);
+    return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES, true, true>(p, group_shift, 0, -1, ksplit, workspace)
+                       : launch_direct<8, GROUPS, TM, WAVES, true, true>(p, group_shift, 0, -1, ksplit, workspace);
+  return p.bits == 4 ? launch_direct<4, GROUPS, TM, WAVES, false, true>(p, group_shift, 0, -1, ksplit, workspace)
+                     : launch_direct<8, GROUPS, TM, WAVES, false, true>(p, group_shift, 0, -1, ksplit, workspace);
+}
+
+bool launch_split_bits(const Problem& p, int group_shift, int ksplit, void* workspace) {
+  return p.m > 64 ? launch_split_shape<2, 4, 4>(p, group_shift, ksplit, workspace)
+                  : launch_split_shape<4, 2, 2>(p, group_shift, ksplit, workspace);
 }
 
 // Whether, and how many ways, to split K across workgroups for `p` (128 x 256 tiles, two K groups inside
@@ -682,9 +696,28 @@ bool launch_split_bits(const Problem& p, int group_shift, int ksplit, void* work
 // gain from windows of four macro steps (K 1024) on, int4 weights -- whose small-tile kernels are better --
 // only from eight macro steps on, with at least four windows and tiles on at most an eighth of the CUs.
 int gemm_split_ways(const Problem& p) {
-  if (p.m <= 64 || p.k % 256 != 0 || p.group != (p.bits == 4 ? 32 : 128) || !gemm_pipe_applicable(p)) return 1;
+  if (p.m <= 16 || p.k % 256 != 0 || p.group != (p.bits == 4 ? 32 : 128) || !gemm_pipe_applicable(p)) return 1;
   if (p.activation == kActGated || p.activation == kActGelu) return 1;
-  const int64_t cu = cu_count(), tiles = ((p.m + 127) / 128) * ((p.n + 255) / 256), macro = p.k / 256;
+  const int64_t cu = cu_count(), macro = p.k / 256;
+  if (p.m <= 64) {
+    // 17 .. 64 rows: one row of 64 x 128 tiles (four K groups, so a window is at least four macro steps); without
+    // the split these shapes run on a fraction of the CUs or through the register-activation kernel, whose time
+    // grows with the rows (it re-reads the activations once per 16-row weight tile).  The split costs the same from
+    // 17 to 64 rows -- about 16 us on a 4096 x 4096 projection, most of it start-up and the exchange -- so it
+    // takes over where the other kernels have grown past it (measured on the Llama-2 7B / 13B projections):
+    // from 48 rows on, from 24 rows on when K is at least 8192 (int8: from 17), and on tile-major weights, where
+    // the register-activation kernel is faster, at 64 rows or from 32 rows on with K of at least 8192.
+    const bool long_k = p.k >= 8192;
+    const int64_t from = p.tiled ? (long_k ? 32 : 64) : (long_k ? (p.bits == 8 ? 17 : 24) : 48);
+    if (p.m < from) return 1;
+    const int64_t tiles = (p.n + 127) / 128;
+    if (tiles * 2 > cu || tiles > kGemmSplitMaxTiles) return 1;
+    const int64_t ways = std::min<int64_t>({cu / tiles, macro / 4, 8});
+    if (ways < 2) return 1;
+    const int64_t per = (macro + ways - 1) / ways;
+    return (int)((macro + per - 1) / per);
+  }
+  const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 255) / 256);
   if (tiles * (p.bits == 4 ? 8 : 2) > cu || tiles > kGemmSplitMaxTiles) return 1;
   const int64_t ways = std::min<int64_t>({cu / tiles, macro / (p.bits == 4 ? 8 : 4), 8});
   if (ways < (p.bits == 4 ? 4 : 2)) return 1;
@@ -736,6 +769,7 @@ bool launch_gemm_direct(const Problem& p, int group_shift, int variant) {
 int64_t gemm_split_workspace_bytes(const Problem& p) {
   const int ways = gemm_split_ways(p);
   if (ways < 2) return 0;
+  if (p.m <= 64) return kGemmSplitCounterBytes + ((p.n + 127) / 128) * ways * (64 * 128 * 4);
   const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 255) / 256);
   return kGemmSplitCounterBytes + tiles * ways * (128 * 256 * 4);
 }

@@ -86,8 +86,9 @@ def test_missing_or_small_workspace_is_the_plain_call():
     torch.cuda.synchronize()
     assert torch.equal(plain.view(torch.int16), y.view(torch.int16))
     assert int(small.sum()) == 0, "a workspace that is too small is not touched"
-    # problems the library does not split ignore the workspace: 33 rows, and a wide projection
-    for m2, n2, k2 in ((33, 5120, 13824), (8, 12288, 4096)):
+    # problems the library does not split ignore the workspace: 33 rows on a wide projection (172 tiles of
+    # 64 x 128 already fill the CUs), and a wide projection at 8 rows
+    for m2, n2, k2 in ((33, 22016, 4096), (8, 12288, 4096)):
         x2, wq2, s2, _ = O.make_case(48, m2, n2, k2, 4)
         assert relax_amd.wq_workspace_bytes(4, 32, n2, k2, m2) == 0
         a = relax_amd.wq_matmul(_dev(x2), _dev(wq2), _dev(s2), 4, 32)
@@ -211,7 +212,10 @@ def test_k_split_is_stable_while_another_stream_keeps_the_gpu_busy():
 
 # (bits, M, N, K): prefill-side shapes whose 128 x 256 tiles fill at most half of the CUs
 GEMM_CASES = [(8, 256, 5120, 5120), (8, 256, 5120, 13824), (8, 256, 15360, 5120), (4, 256, 4096, 11008),
-              (4, 128, 4096, 11008), (4, 200, 4090, 8192), (8, 65, 5120, 5120), (8, 384, 1000, 2048)]
+              (4, 128, 4096, 11008), (4, 200, 4090, 8192), (8, 65, 5120, 5120), (8, 384, 1000, 2048),
+              # 17 .. 64 rows: 64 x 128 tiles, four K groups per workgroup
+              (4, 64, 4096, 4096), (4, 48, 12288, 4096), (8, 17, 5120, 13824), (4, 33, 4090, 11008),
+              (8, 50, 1000, 2048), (4, 64, 4096, 11008), (8, 64, 5120, 5120)]
 
 
 @pytest.mark.parametrize("bits,m,n,k", GEMM_CASES)
@@ -226,7 +230,7 @@ def test_gemm_k_split_matches_the_oracle_and_is_deterministic(bits, m, n, k):
     y1 = relax_amd.wq_matmul(dx, dwq, ds, bits, g, workspace=ws)
     torch.cuda.synchronize()
     assert int(ws[:16384].view(torch.int32).abs().sum()) == 0, "arrival counters are back at zero"
-    rows = sorted({0, 1, m // 2, m - 2, m - 1} | set(np.random.default_rng(5).integers(0, m, 11).tolist()))
+    rows = sorted({0, 1, m // 2, m - 2, m - 1} | set(np.random.default_rng(5).integers(0, m, 11).tolist()))  # (all rows when m is small)
     want = c_oracle.wq_matmul(x[rows], wq, s, bits, g, nthreads=16)
     assert_close(y1.cpu().numpy()[rows], want, ("gemm k split", bits, m, n, k), ulp_fraction=0.005)
     # every tile, against float32 torch on the dequantized weights (the oracle's rows pin the arithmetic)
@@ -241,6 +245,15 @@ def test_gemm_k_split_matches_the_oracle_and_is_deterministic(bits, m, n, k):
     y0 = relax_amd.wq_matmul(dx, dwq, ds, bits, g)
     torch.cuda.synchronize()
     assert_close(y0.cpu().numpy()[rows], want, ("plain", bits, m, n, k), ulp_fraction=0.005)
+    # tile-major weights: the same windows in the same order where the library splits there the same way
+    wq_t, s_t = relax_amd.wq_tile_weights(dwq, ds, bits, g)
+    y3 = relax_amd.wq_matmul(dx, wq_t, s_t, bits, g, tiled_n=n, workspace=ws)
+    torch.cuda.synchronize()
+    assert int(ws[:16384].view(torch.int32).abs().sum()) == 0
+    if relax_amd.wq_workspace_bytes(bits, g, n, k, m, tiled=True) == need:
+        assert torch.equal(y1.view(torch.int16), y3.view(torch.int16))
+    else:
+        assert_close(y3.cpu().numpy()[rows], want, ("tile-major", bits, m, n, k), ulp_fraction=0.005)
 
 
 def test_gemm_k_split_applies_the_fused_tail_once():
