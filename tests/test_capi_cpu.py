@@ -69,7 +69,14 @@ def test_workspace_size_query_without_a_gpu():
     assert q(lib.make_desc(4, 32, 12288, 4096), 8, 0) == 0 and q(lib.make_desc(4, 32, 4096, 4096), 16, 0) == 0
     assert q(lib.make_desc(8, 128, 5120, 13824), 4, 1) == 0                              # tile-major: from 12 rows on
     assert q(lib.make_desc(8, 128, 5120, 13824), 16, 1) == 16384 + 320 * 4 * 1024
-    assert q(lib.make_desc(4, 32, 4096, 11008), 32, 0) == 0                              # not a decode batch
+    # 17 .. 64 rows: the GEMM's split on 64 x 128 tiles (32 KB per tile and window) from the measured row counts on
+    assert q(lib.make_desc(4, 32, 4096, 11008), 32, 0) == 16384 + 32 * 8 * 32768
+    assert q(lib.make_desc(4, 32, 4096, 11008), 20, 0) == 0 and q(lib.make_desc(4, 32, 4096, 4096), 32, 0) == 0
+    assert q(lib.make_desc(4, 32, 4096, 4096), 64, 0) == 16384 + 32 * 4 * 32768
+    assert q(lib.make_desc(4, 32, 22016, 4096), 64, 0) == 0                              # 172 tiles fill the CUs
+    # above 64 rows: 128 x 256 tiles (128 KB per tile and window)
+    assert q(lib.make_desc(8, 128, 5120, 13824), 256, 0) == 16384 + 40 * 6 * 131072
+    assert q(lib.make_desc(4, 32, 4096, 4096), 512, 0) == 0
     assert q(lib.make_desc(4, 32, 4096, 320), 8, 1) == 0                                 # layout not defined: no split
     assert q(lib.make_desc(5, 32, 4096, 4096), 8, 0) == -1 and "bits" in lib.last_error()
     ok = 0x10000
