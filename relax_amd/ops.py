@@ -191,10 +191,11 @@ def _wq_matmul_ws(x, wq, scales, bits, group, tiled_n, zero_point, out, stream, 
             raise ValueError(f"tile-major buffers must hold {wb} and {sb} bytes for N={n}, K={k}")
     elif wq.shape[1] * (32 // bits) != k or tuple(scales.shape) != (n, k // group):
         raise ValueError("wq / scales do not match x's K")
+    out_cols = n // 2 if activation == "silu_mul" else n  # the gated tail halves the output
     if out is None:
-        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
-    elif tuple(out.shape) != (m, n) or out.dtype != torch.float16 or not out.is_contiguous():
-        raise ValueError("out must be a compact float16 [M, N] tensor")
+        out = torch.empty((m, out_cols), dtype=torch.float16, device=x.device)
+    elif tuple(out.shape) != (m, out_cols) or out.dtype != torch.float16 or not out.is_contiguous():
+        raise ValueError(f"out must be a compact float16 [{m}, {out_cols}] tensor")
     if activation not in _lib.ACTIVATIONS:
         raise ValueError(f"unsupported activation {activation!r}")
     ep = _lib.WqEpilogue(bias.data_ptr() if bias is not None else None,
