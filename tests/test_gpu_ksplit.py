@@ -164,7 +164,8 @@ def test_workspace_entry_called_vm_style():
     import relax_amd
 
     vm_harness.set_stream()
-    for bits, m, n, k in [(8, 2, 5120, 13824), (4, 16, 4096, 11008), (4, 8, 50, 512)]:
+    for bits, m, n, k in [(8, 2, 5120, 13824), (4, 16, 4096, 11008), (4, 8, 50, 512), (8, 256, 5120, 5120),
+                          (4, 64, 4096, 4096)]:  # decode split, no split, the GEMM's split above and below 64 rows
         x, wq, s, g = O.make_case(60 + m, m, n, k, bits)
         need = relax_amd.wq_workspace_bytes(bits, g, n, k, m)
         ws = torch.zeros(max(need, 64), dtype=torch.uint8, device="cuda")

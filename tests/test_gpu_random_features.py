@@ -83,3 +83,53 @@ def test_random_problems_with_workspace_layouts_and_tails(chunk):
                 mag = mag + np.abs(bias.astype(np.float64))[None, :]
             bound = 1.2 * (ATOL + RTOL * mag) + 2.0 ** -9 * (np.abs(ref) + (mag if tail != "silu_mul" else 0))
             assert np.all(np.isfinite(got)) and np.all(np.abs(got - ref) <= bound), (what, float(np.abs(got - ref).max()))
+
+
+@pytest.mark.parametrize("chunk", range(3))
+def test_random_call_descriptions_through_the_packed_boundary(chunk):
+    """The generic PackedFunc entry with random argument orders, every activation and both scratch modes,
+    against the C ABI's result for the same problem (bit for bit: it is the same kernel on the same stream)."""
+    import relax_amd
+    from relax_amd import vm_harness
+    from relax_amd.vm_harness import CallSpec, TensorArg
+
+    vm_harness.set_stream()
+    rng = np.random.default_rng(8100 + chunk)
+    for _ in range(10):
+        bits = int(rng.choice([4, 8]))
+        g = 32 if bits == 4 else 128
+        m = int(rng.choice([1, 8, 16, 40, 130]))
+        n = 2 * int(rng.integers(20, 300))
+        k = 256 * int(rng.integers(1, 9))
+        act = int(rng.choice([0, 1, 2, 3]))
+        with_bias = act != 2 and bool(rng.random() < 0.6)
+        with_res = act != 2 and bool(rng.random() < 0.5)
+        x, wq, s, _ = O.make_case(int(rng.integers(1 << 20)), m, n, k, bits)
+        bias, res = _fused_operands(m + n, m, n)
+        out_cols = n // 2 if act == 2 else n
+        out = torch.empty((m, out_cols), dtype=torch.float16, device="cuda")
+        tensors = {"x": _dev(x), "wq": _dev(wq), "scales": _dev(s), "out": out}
+        if with_bias:
+            tensors["bias"] = _dev(bias)
+        if with_res:
+            tensors["residual"] = _dev(res)
+        order = list(tensors)
+        rng.shuffle(order)
+        pos = {name: i for i, name in enumerate(order)}
+        spec = CallSpec(op=0, bits=bits, group=0, zero_point=7 if bits == 4 else 0, arg_x=pos["x"], arg_wq=pos["wq"],
+                        arg_scales=pos["scales"], arg_out=pos["out"], num_args=len(order),
+                        arg_bias=pos.get("bias", -1), arg_residual=pos.get("residual", -1), activation=act)
+        args = [TensorArg(tensors[name], as_uint32=(name == "wq")) for name in order]
+        scratch = bool(rng.random() < 0.5)
+        vm_harness.call_packed("mi355x_wq_packed_call_scratch" if scratch else "mi355x_wq_packed_call", args, spec=spec)
+        torch.cuda.synchronize()
+        name = {0: None, 1: "relu", 2: "silu_mul", 3: "gelu"}[act]
+        want = relax_amd.wq_matmul(tensors["x"], tensors["wq"], tensors["scales"], bits, g,
+                                   bias=tensors.get("bias"), activation=name, residual=tensors.get("residual"))
+        torch.cuda.synchronize()
+        what = (bits, m, n, k, name, with_bias, with_res, order, scratch)
+        if scratch and m <= 16 and relax_amd.wq_workspace_bytes(bits, g, n, k, m) > 0:
+            # the scratch entry splits K where the plain call does not: same tolerance, other summation order
+            assert_close(out.cpu().numpy(), want.cpu().numpy(), what, ulp_fraction=0.01)
+        else:
+            assert torch.equal(out.view(torch.int16), want.view(torch.int16)), what
