@@ -4,7 +4,7 @@ The reference holds no vectors for a quantized matmul (it has no such operator),
 fixtures are outputs of the pinned CPU oracle on seeded inputs; they freeze the layout
 (least-significant field first) and the rounding sequence.  Run from the repo root:
 
-    python tests/golden/make_golden.py            (--fused-only / --tiled-only: just those fixtures)
+    python tests/golden/make_golden.py            (--fused-only / --tiled-only / --tails-only: just those fixtures)
 """
 import os
 import sys
@@ -27,6 +27,12 @@ FUSED_CASES = [  # name, seed, M, N, K, bits, group, bias?, activation, residual
     ("fused_q4f16_m4_n48_k128_bias_relu_res", 21, 4, 48, 128, 4, 32, True, "relu", True),
     ("fused_q4f16_m1_n80_k256_res", 22, 1, 80, 256, 4, 32, False, None, True),
     ("fused_q8f16_m70_n24_k256_bias", 23, 70, 24, 256, 8, 128, True, None, False),
+]
+
+
+TAIL_CASES = [  # name, seed, M, N, K, bits, group, bias?, activation: the tails with a float32 transcendental inside
+    ("tail_q4f16_m6_n64_k256_bias_gelu", 41, 6, 64, 256, 4, 32, True, "gelu"),
+    ("tail_q8f16_m9_n48_k256_silu_mul", 42, 9, 48, 256, 8, 128, False, "silu_mul"),
 ]
 
 
@@ -53,6 +59,17 @@ if __name__ == "__main__":
                             bits=np.int32(bits), group=np.int32(g))
         print(name, wt.shape, st.shape)
     if "--tiled-only" in sys.argv:
+        sys.exit(0)
+    for name, seed, m, n, k, bits, group, wb, act in TAIL_CASES:
+        x, wq, s, g = O.make_case(seed, m, n, k, bits, group)
+        bias, _ = fused_operands(seed, m, n, wb, False)
+        y = O.wq_matmul_fused(x, wq, s, bits, g, bias, act, None)
+        extra = {} if bias is None else {"bias": bias}
+        np.savez_compressed(os.path.join(here, name + ".npz"), x=x, wq=wq, scales=s, y=y,
+                            y_plain=O.wq_matmul(x, wq, s, bits, g), bits=np.int32(bits), group=np.int32(g),
+                            activation=np.array(act), **extra)
+        print(name, y.shape, float(np.abs(y).max()))
+    if "--tails-only" in sys.argv:
         sys.exit(0)
     for name, seed, m, n, k, bits, group, wb, act, wr in FUSED_CASES:
         x, wq, s, g = O.make_case(seed, m, n, k, bits, group)

@@ -9,8 +9,9 @@ from oracle import c_oracle, wq_oracle as O
 FILES = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
 
 
-PLAIN = [f for f in FILES if not os.path.basename(f).startswith(("fused_", "tiled_"))]
+PLAIN = [f for f in FILES if not os.path.basename(f).startswith(("fused_", "tiled_", "tail_"))]
 FUSED = [f for f in FILES if os.path.basename(f).startswith("fused_")]
+TAILS = [f for f in FILES if os.path.basename(f).startswith("tail_")]
 TILED = [f for f in FILES if os.path.basename(f).startswith("tiled_")]
 
 
@@ -45,6 +46,23 @@ def test_fused_fixtures_match_both_oracles():
             assert np.array_equal(y.view(np.uint16), z["y"].view(np.uint16)), f
             assert np.array_equal(impl.epilogue(z["y_plain"], bias, act, res).view(np.uint16),
                                   z["y"].view(np.uint16)), f
+
+
+def test_gelu_and_gated_tail_fixtures_match_both_oracles():
+    """The two tails with a float32 transcendental inside (erf, exp): the NumPy restatement takes it as the
+    float64 value rounded to float32, the C one asks the host's libm; the fixtures hold the former and the
+    latter must agree wherever the libm's last float32 bit does (everywhere, on every libm seen so far)."""
+    assert len(TAILS) >= 2
+    for f in TAILS:
+        z = np.load(f)
+        bits, g = int(z["bits"]), int(z["group"])
+        bias, act, _ = fused_operands(z)
+        y = O.wq_matmul_fused(z["x"], z["wq"], z["scales"], bits, g, bias, act, None)
+        assert np.array_equal(y.view(np.uint16), z["y"].view(np.uint16)), f
+        yc = c_oracle.wq_matmul_fused(z["x"], z["wq"], z["scales"], bits, g, bias, act, None)
+        off = yc.view(np.uint16) != z["y"].view(np.uint16)
+        assert off.sum() <= max(1, y.size // 500), (f, int(off.sum()))
+        assert y.shape[1] == (z["wq"].shape[0] // 2 if act == "silu_mul" else z["wq"].shape[0])
 
 
 def test_fused_fixture_by_hand():

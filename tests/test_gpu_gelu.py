@@ -122,3 +122,35 @@ def test_gelu_with_the_residual_in_the_output_buffer(bits, m, n, k):
         with pytest.raises(lib.WqError, match="buffer of its own"):
             relax_amd.wq_matmul(_dev(x), _dev(wq), _dev(s), bits, g, bias=_dev(bias), activation="gelu", residual=h,
                                 out=h, kernel=lib.KERNEL_GEMM, variant=21)
+
+
+def test_tail_golden_fixtures():
+    """The committed fixtures of the gelu and gated tails: at least 99.9 % of the outputs equal the fixture's tail
+    applied to this kernel's own matmul output bit for bit, and everything within the matmul tolerance of the fixture."""
+    import glob
+    import os
+
+    import relax_amd
+    from relax_amd import lib
+    from tests.test_gpu_parity import _dev
+
+    files = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "tail_*.npz")))
+    assert len(files) >= 2
+    for f in files:
+        z = np.load(f)
+        bits, g, act = int(z["bits"]), int(z["group"]), str(z["activation"])
+        bias = z["bias"] if "bias" in z.files else None
+        m = z["x"].shape[0]
+        fam = lib.KERNEL_GEMV if m <= 16 else lib.KERNEL_GEMM
+        dx, dwq, ds = _dev(z["x"]), _dev(z["wq"]), _dev(z["scales"])
+        h = relax_amd.wq_matmul(dx, dwq, ds, bits, g, kernel=fam).cpu().numpy()
+        got = relax_amd.wq_matmul(dx, dwq, ds, bits, g, kernel=fam, bias=None if bias is None else _dev(bias),
+                                  activation=act).cpu().numpy()
+        own = O.epilogue(h, bias, act, None)
+        assert (got.view(np.uint16) != own.view(np.uint16)).sum() <= max(1, got.size // 1000), f
+        err = np.abs(got.astype(np.float64) - z["y"].astype(np.float64))
+        mag = np.abs(z["y_plain"].astype(np.float64))
+        if act == "silu_mul":
+            half = mag.shape[1] // 2
+            mag = 2.0 * (1.0 + mag[:, :half] + mag[:, half:]) * (1.0 + np.abs(z["y"].astype(np.float64)))
+        assert np.all(err <= 1.2 * (ATOL + RTOL * mag) + 2.0 ** -9 * np.abs(z["y"].astype(np.float64))), (f, float(err.max()))
