@@ -154,25 +154,23 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
   if (m > kSkinnyMaxM) return MI355X_WQ_KERNEL_GEMM;
   // 17..64 rows.  The skinny kernel re-reads the activations from L2 once per 16-row weight tile, so
   // its time grows with M and N; the direct-weight GEMM with its 64x128 tile and four K groups costs
-  // the same from 1 to 64 rows.  Measured crossovers on MI355X (q4f16 and q8f16, K = 4096 ... 13824):
-  // with 160 or more 128-column tiles the GEMM wins from 24 rows on (N = 22016: 29 us against
-  // 36 - 52 us), with 96 or more tiles of int4 weights from 33 rows on, with 64 or more from 49.
+  // the same from 1 to 64 rows.  Measured crossovers on MI355X (q4f16 and q8f16, K = 4096 ... 13824, with
+  // the skinny kernel's activations staged through LDS): with 160 or more 128-column tiles the GEMM wins
+  // from 17 rows on (N = 22016: 28 us against 30 - 42 us; int8 N = 27648: 53 against 55 - 69 us), with 96 or
+  // more tiles of int4 weights from 49 rows on (N = 12288 at 56 rows: 26.7 against 27.8 us); with fewer the
+  // skinny kernel stays ahead up to 64 rows (8192 x 4096 at 64 rows: 16.9 against 24.2 us).
   const int64_t tiles128 = (d->n + 127) / 128;
   const bool direct_small_tile = d->k % 256 == 0 && d->k >= 1024 && tiles128 <= cu_count() &&
                                  ((d->bits == 4 && d->group == 32) || (d->bits == 8 && d->group == 128));
   if (tiled) {
     // On tile-major weights the skinny kernel's loads are contiguous and it holds out longer
-    // (N = 12288, 32 rows: 14 us against the GEMM's 22 us): for int4 the GEMM takes over from 40 rows
-    // with 160 or more column tiles and from 57 rows with 64 or more; int8 stays with the skinny
-    // kernel up to 56 rows (27648 x 5120 at 48 rows: 44 against 50 us) and goes to the GEMM beyond
-    // with 160 or more column tiles (32000 x 4096 at 64 rows: 42 against 48 us).
-    if (direct_small_tile && d->bits == 4 && ((tiles128 >= 160 && m >= 40) || (m > 56 && tiles128 >= 64)))
-      return MI355X_WQ_KERNEL_GEMM;
-    if (direct_small_tile && d->bits == 8 && tiles128 >= 160 && m > 56) return MI355X_WQ_KERNEL_GEMM;
+    // (N = 12288: 12.9 - 23.9 us from 17 to 64 rows against the GEMM's 23 - 25 us): the GEMM takes over from
+    // 40 rows with 160 or more column tiles (22016 x 4096: 27.0 against 27.8 us; int8 27648 x 5120: 47.7
+    // against 48.6 us).
+    if (direct_small_tile && tiles128 >= 160 && m >= 40) return MI355X_WQ_KERNEL_GEMM;
     return MI355X_WQ_KERNEL_SKINNY;
   }
-  if (direct_small_tile && ((m >= 24 && tiles128 >= 160) || (d->bits == 4 && m > 32 && tiles128 >= 96) ||
-                            (d->bits == 4 && m > 48 && tiles128 >= 64)))
+  if (direct_small_tile && (tiles128 >= 160 || (d->bits == 4 && m > 48 && tiles128 >= 96)))
     return MI355X_WQ_KERNEL_GEMM;
   return MI355X_WQ_KERNEL_SKINNY;
 }

@@ -702,13 +702,13 @@ int gemm_split_ways(const Problem& p) {
   if (p.m <= 64) {
     // 17 .. 64 rows: one row of 64 x 128 tiles (four K groups, so a window is at least four macro steps); without
     // the split these shapes run on a fraction of the CUs or through the register-activation kernel, whose time
-    // grows with the rows (it re-reads the activations once per 16-row weight tile).  The split costs the same from
-    // 17 to 64 rows -- about 16 us on a 4096 x 4096 projection, most of it start-up and the exchange -- so it
+    // grows with the rows.  The split costs the same from 17 to 64 rows -- about 16 us on a 4096 x 4096
+    // projection, 22 us on 4096 x 11008, 34 us on 5120 x 13824 int8, most of it start-up and the exchange -- so it
     // takes over where the other kernels have grown past it (measured on the Llama-2 7B / 13B projections):
-    // from 48 rows on, from 24 rows on when K is at least 8192 (int8: from 17), and on tile-major weights, where
-    // the register-activation kernel is faster, at 64 rows or from 32 rows on with K of at least 8192.
+    // with K of at least 8192 from 40 rows on (int8 on canonical weights: from 17), else from 56 rows on
+    // canonical weights and not at all on tile-major ones.
     const bool long_k = p.k >= 8192;
-    const int64_t from = p.tiled ? (long_k ? 32 : 64) : (long_k ? (p.bits == 8 ? 17 : 24) : 48);
+    const int64_t from = p.tiled ? (long_k ? 40 : 65) : (long_k ? (p.bits == 8 ? 17 : 40) : 56);
     if (p.m < from) return 1;
     const int64_t tiles = (p.n + 127) / 128;
     if (tiles * 2 > cu || tiles > kGemmSplitMaxTiles) return 1;

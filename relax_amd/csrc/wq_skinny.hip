@@ -24,6 +24,8 @@
 
 namespace wq {
 
+__device__ __forceinline__ bool m_ok_row(int row, int M) { return row < M; }
+
 template <int BITS, int R, int MT, int U>
 struct SkinnyBatch {
   static constexpr int NJ = (128 / BITS) / 8;
@@ -32,7 +34,13 @@ struct SkinnyBatch {
   u32x4 xa[U][MT][NJ];
 };
 
-template <int BITS, int R, int MT, int WAVES, int U, bool TILED>
+// XST: the activations of a k-step reach the MFMA operand registers through a wavefront-private LDS area
+// instead of directly.  Directly, lane (row m, chunk kq) loads the 16-byte pieces of its own row: 64 pieces
+// from 16 rows per instruction, 64 tag lookups in the L1.  Staged, a load instruction covers 1 KB of four
+// rows (8 lines), the wavefront stores the pieces to LDS as loaded and every lane reads back the pieces of
+// its operand; which piece a lane loads is XOR-swizzled with the row on the global side so that the
+// reads of 16 rows at one position fall on 16 different bank groups.
+template <int BITS, int R, int MT, int WAVES, int U, bool TILED, bool XST = false>
 __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
     half_t* y, int M, int N, int K, int group_shift, int zero_point, const Epilogue ep) {
@@ -84,6 +92,33 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
     xbase[mt] = (uint32_t)m * (uint32_t)K * 2u;
   }
 
+  // staged activations: ROWB bytes of every row per k-step, MT * 4 KB (int4) per wavefront
+  constexpr int ROWB = 4 * CH * 2;            // 256 (int4) / 128 (int8)
+  constexpr int PIECES = ROWB / 16;           // 16-byte pieces per row and k-step
+  constexpr int RPI = 64 / PIECES;            // rows one load instruction covers: 4 / 8
+  constexpr int XI = MT * 16 / RPI;           // load instructions per k-step (= MT * NJ)
+  static_assert(XI == MT * NJ, "the staged form uses the registers of the direct one");
+  constexpr size_t kRedBytes = (size_t)WAVES * R * MT * 1024, kStageBytes = XST ? (size_t)WAVES * MT * 16 * ROWB : 0;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[kRedBytes > kStageBytes ? kRedBytes : kStageBytes];
+  unsigned char* const xst = smem + (size_t)wave * (MT * 16 * ROWB);
+  // (256-byte rows span all 64 banks: 16 rows need 16 positions; 128-byte rows alternate between the bank halves,
+  // so a pair of rows shares a position)
+  auto swz = [](int row) { return PIECES == 16 ? (row & 15) : ((row >> 1) & 7); };
+  uint32_t xs_rd[MT][NJ];  // where lane (col, kq) finds piece kq * NJ + j of row mt * 16 + col
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+      xs_rd[mt][j] = (uint32_t)((mt * 16 + col) * ROWB + (((kq * NJ + j) ^ swz(mt * 16 + col)) * 16));
+  // the row and the piece this lane loads in instruction t: row t * RPI + lane / PIECES, stored piece lane % PIECES
+  uint32_t xl_base[XI];
+#pragma unroll
+  for (int t = 0; t < XI; ++t) {
+    const int row = t * RPI + lane / PIECES;
+    const int piece = (lane % PIECES) ^ swz(row);
+    xl_base[t] = (m_ok_row(row, M)) ? (uint32_t)row * (uint32_t)K * 2u + (uint32_t)piece * 16u : kOobOffset;
+  }
+
   float4_t acc[R][MT];
 #pragma unroll
   for (int r = 0; r < R; ++r)
@@ -110,11 +145,19 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
         b.w[u][r] = load_b128(rw, wbase[r] + winc);  // valid base < 2^31: the sum cannot wrap
         b.sc[u][r] = load_b16(rs, sbase[r] + sinc);
       }
+      if constexpr (XST) {
+        // line by line: instruction t reads ROWB bytes of RPI rows; a k-step past the end reads zeros
+        const uint32_t kinc = (uint32_t)ks * ROWB;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const uint32_t xo = (ok && xrow_ok[mt]) ? xbase[mt] + xinc : kOobOffset;
+        for (int t = 0; t < XI; ++t)
+          b.xa[u][t / NJ][t % NJ] = load_b128(rx, (ks < ks_end && xl_base[t] != kOobOffset) ? xl_base[t] + kinc : kOobOffset);
+      } else {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) b.xa[u][mt][j] = load_b128(rx, xo + j * 16u);
+        for (int mt = 0; mt < MT; ++mt) {
+          const uint32_t xo = (ok && xrow_ok[mt]) ? xbase[mt] + xinc : kOobOffset;
+#pragma unroll
+          for (int j = 0; j < NJ; ++j) b.xa[u][mt][j] = load_b128(rx, xo + j * 16u);
+        }
       }
     }
   };
@@ -123,11 +166,18 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       half8_t a[MT][NJ];
+      if constexpr (XST) {
+#pragma unroll
+        for (int t = 0; t < XI; ++t)
+          *reinterpret_cast<u32x4*>(xst + t * 1024 + lane * 16) = b.xa[u][t / NJ][t % NJ];
+      }
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-          const u32x4 v = b.xa[u][mt][j];
+          u32x4 v;
+          if constexpr (XST) v = *reinterpret_cast<const u32x4*>(xst + xs_rd[mt][j]);
+          else v = b.xa[u][mt][j];
           if constexpr (BITS == 4) {
             // activations follow the weight pair order (k0,k4)(k1,k5)(k2,k6)(k3,k7)
             u32x4 p;
@@ -179,7 +229,8 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
   }
 
   // cross-wave reduction of the K split
-  __shared__ float red[WAVES][R * MT][4][64];
+  if constexpr (XST) __syncthreads();  // (the staging areas are about to become the reduction buffer)
+  float (*red)[R * MT][4][64] = reinterpret_cast<float (*)[R * MT][4][64]>(smem);
 #pragma unroll
   for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -201,11 +252,11 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
 
 namespace {
 
-template <int BITS, int R, int MT, int WAVES, int U, bool TILED = false>
+template <int BITS, int R, int MT, int WAVES, int U, bool TILED = false, bool XST = false>
 void launch_one(const Problem& p, int group_shift) {
   const int tiles = (int)((p.n + 15) / 16);
   dim3 grid((tiles + R - 1) / R), block(WAVES * 64);
-  hipLaunchKernelGGL((wq_skinny_kernel<BITS, R, MT, WAVES, U, TILED>), grid, block, 0, p.stream,
+  hipLaunchKernelGGL((wq_skinny_kernel<BITS, R, MT, WAVES, U, TILED, XST>), grid, block, 0, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point,
                      Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
@@ -213,6 +264,27 @@ void launch_one(const Problem& p, int group_shift) {
 
 template <int BITS, int MT>
 bool dispatch_variant(const Problem& p, int group_shift, int variant) {
+  if (variant > 20 && MT < 2) return false;  // (one row block: the direct loads)
+  if (variant > 20) {  // staged activations (two row blocks and more), both layouts
+    if (p.tiled) {
+      switch (variant - 20) {
+        case 1: launch_one<BITS, 1, MT, 4, 2, true, true>(p, group_shift); return true;
+        case 2: launch_one<BITS, 2, MT, 4, 2, true, true>(p, group_shift); return true;
+        case 5: launch_one<BITS, 2, MT, 8, 1, true, true>(p, group_shift); return true;
+        case 7: launch_one<BITS, 4, MT, 4, 1, true, true>(p, group_shift); return true;
+        case 11: launch_one<BITS, 8, MT, 4, 1, true, true>(p, group_shift); return true;
+        default: return false;
+      }
+    }
+    switch (variant - 20) {
+      case 1: launch_one<BITS, 1, MT, 4, 2, false, true>(p, group_shift); return true;
+      case 2: launch_one<BITS, 2, MT, 4, 2, false, true>(p, group_shift); return true;
+      case 5: launch_one<BITS, 2, MT, 8, 1, false, true>(p, group_shift); return true;
+      case 7: launch_one<BITS, 4, MT, 4, 1, false, true>(p, group_shift); return true;
+      case 11: launch_one<BITS, 8, MT, 4, 1, false, true>(p, group_shift); return true;
+      default: return false;
+    }
+  }
   if (p.tiled) {  // the variants the default choice uses, reading the tile-major layout
     switch (variant) {
       case 1: launch_one<BITS, 1, MT, 4, 2, true>(p, group_shift); return true;
@@ -263,11 +335,16 @@ int launch_skinny(const Problem& p, int variant) {
     // round of workgroups costs more: 5120 x 13824 at 64 rows 114 -> 67 us); more: four
     // tiles per workgroup; many: two tiles per 8-wave workgroup for one row block, else four.
     const int64_t tiles = (p.n + 15) / 16;
-    if (tiles <= 256) variant = 1;
+    // From 17 rows on the activations are staged through LDS (variants 21 ...: the same shapes with
+    // line-by-line activation loads): 10 - 30 % faster from 32 rows on (4096 x 11008 at 64 rows 46 -> 35 us,
+    // int8 5120 x 13824 at 64 rows 72 -> 53 us), level at 17; not on tile-major int4 weights with 513 - 1024
+    // tiles (12288 x 4096 at 32 rows: 15.0 direct, 15.2 staged) and not with more than 1024 tiles.
+    const bool staged = mt >= 2;
+    if (tiles <= 256) variant = staged ? 21 : 1;
     // (one tile per workgroup is 1.5 - 1.8x slower here; int8 at up to 4 rows on tile-major weights:
     // eight wavefronts, 3 - 5 % ahead)
-    else if (tiles <= 512) variant = (p.bits == 4 || (p.tiled && p.m <= 4)) ? 5 : 2;
-    else if (tiles <= 1024) variant = 7;
+    else if (tiles <= 512) variant = staged ? 25 : ((p.bits == 4 || (p.tiled && p.m <= 4)) ? 5 : 2);
+    else if (tiles <= 1024) variant = (staged && !(p.tiled && p.bits == 4)) ? 27 : 7;
     // several rounds of workgroups: eight tiles share one pass over the activations (four for int8 on
     // tile-major weights: 32000 x 4096 at 24 - 32 rows, 33.5 against 36.5 us)
     else variant = mt == 1 ? 5 : (p.tiled && p.bits == 8 ? 7 : 11);

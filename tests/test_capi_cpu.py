@@ -70,8 +70,10 @@ def test_workspace_size_query_without_a_gpu():
     assert q(lib.make_desc(8, 128, 5120, 13824), 4, 1) == 0                              # tile-major: from 12 rows on
     assert q(lib.make_desc(8, 128, 5120, 13824), 16, 1) == 16384 + 320 * 4 * 1024
     # 17 .. 64 rows: the GEMM's split on 64 x 128 tiles (32 KB per tile and window) from the measured row counts on
-    assert q(lib.make_desc(4, 32, 4096, 11008), 32, 0) == 16384 + 32 * 8 * 32768
-    assert q(lib.make_desc(4, 32, 4096, 11008), 20, 0) == 0 and q(lib.make_desc(4, 32, 4096, 4096), 32, 0) == 0
+    assert q(lib.make_desc(4, 32, 4096, 11008), 48, 0) == 16384 + 32 * 8 * 32768
+    assert q(lib.make_desc(4, 32, 4096, 11008), 32, 0) == 0 and q(lib.make_desc(4, 32, 4096, 4096), 48, 0) == 0
+    assert q(lib.make_desc(8, 128, 5120, 13824), 17, 0) == 16384 + 40 * 6 * 32768
+    assert q(lib.make_desc(4, 32, 4096, 4096), 64, 1) == 0                                # tile-major, short K: never
     assert q(lib.make_desc(4, 32, 4096, 4096), 64, 0) == 16384 + 32 * 4 * 32768
     assert q(lib.make_desc(4, 32, 22016, 4096), 64, 0) == 0                              # 172 tiles fill the CUs
     # above 64 rows: 128 x 256 tiles (128 KB per tile and window)
@@ -134,10 +136,11 @@ def test_kernel_selection_by_rows():
     # 17..64 rows on wide projections: the GEMM's 64x128 tile costs the same for any row count, the
     # skinny kernel grows with it
     wide, mid = lib.make_desc(4, 32, 22016, 4096), lib.make_desc(4, 32, 12288, 4096)
-    assert L.mi355x_wq_select_kernel(wide, 23) == lib.KERNEL_SKINNY
-    assert L.mi355x_wq_select_kernel(wide, 24) == lib.KERNEL_GEMM
-    assert L.mi355x_wq_select_kernel(mid, 32) == lib.KERNEL_SKINNY
-    assert L.mi355x_wq_select_kernel(mid, 33) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(wide, 16) == lib.KERNEL_GEMV
+    assert L.mi355x_wq_select_kernel(wide, 17) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(mid, 48) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(mid, 49) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 8192, 4096), 64) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 27648, 5120), 24) == lib.KERNEL_GEMM
     assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 15360, 5120), 48) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 22016, 4000), 48) == lib.KERNEL_SKINNY  # K % 256 != 0

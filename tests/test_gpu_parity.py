@@ -167,6 +167,32 @@ def test_skinny_kernel_matches_oracle(variant, bits, m, n, k):
     assert_close(got, want, (variant, bits, m, n, k))
 
 
+@pytest.mark.parametrize("variant", [21, 22, 25, 27, 31])
+@pytest.mark.parametrize("bits,m,n,k", [
+    (4, 17, 33, 352), (4, 33, 64, 512), (4, 64, 80, 1152), (4, 48, 4096, 4096), (4, 31, 1000, 11008),
+    (8, 20, 72, 640), (8, 64, 16, 1280), (8, 33, 5120, 5120), (8, 50, 300, 13824),
+])
+def test_skinny_kernel_with_staged_activations(variant, bits, m, n, k):
+    """Variants 21 ...: the activations of a k-step loaded line by line and handed to the operand lanes through
+    LDS.  The MFMAs see the same operands in the same order as in the direct variants: bit-equal to them, on both
+    weight layouts, and within tolerance of the oracle.  One row block (M <= 16) has no staged build."""
+    import relax_amd
+    from relax_amd import lib
+
+    x, wq, s, g = O.make_case(150 + m + n, m, n, k, bits)
+    got = run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_SKINNY, variant=variant)
+    direct = run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_SKINNY, variant=variant - 20)
+    assert np.array_equal(got.view(np.uint16), direct.view(np.uint16))
+    assert_close(got, c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16), (variant, bits, m, n, k), ulp_fraction=0.005)
+    if k % 256 == 0:
+        wt, st = relax_amd.wq_tile_weights(_dev(wq), _dev(s), bits, g)
+        tiled = relax_amd.wq_matmul(_dev(x), wt, st, bits, g, tiled_n=n, kernel=lib.KERNEL_SKINNY, variant=variant)
+        torch.cuda.synchronize()
+        assert np.array_equal(tiled.cpu().numpy().view(np.uint16), got.view(np.uint16))
+    with pytest.raises(lib.WqError, match="unknown variant"):
+        run_matmul(x[:8], wq, s, bits, g, kernel=lib.KERNEL_SKINNY, variant=variant)
+
+
 def test_config1_single_gemv_4096():
     """The reference's CPU-runnable case: x[1,4096] ~ N(0,1), W int4 4096x4096, group 32, zero point 7."""
     x, wq, s, g = O.make_case(0, 1, 4096, 4096, 4)
@@ -350,7 +376,7 @@ def test_golden_fixtures():
     import os
 
     files = sorted(f for f in glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz"))
-                   if not os.path.basename(f).startswith(("fused_", "tiled_")))
+                   if not os.path.basename(f).startswith(("fused_", "tiled_", "tail_")))
     assert files, "no golden fixtures found"
     import relax_amd
 
