@@ -98,9 +98,27 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
   constexpr int RPI = 64 / PIECES;            // rows one load instruction covers: 4 / 8
   constexpr int XI = MT * 16 / RPI;           // load instructions per k-step (= MT * NJ)
   static_assert(XI == MT * NJ, "the staged form uses the registers of the direct one");
-  constexpr size_t kRedBytes = (size_t)WAVES * R * MT * 1024, kStageBytes = XST ? (size_t)WAVES * MT * 16 * ROWB : 0;
+  // (canonical weights take the same way: a k-step's 64 bytes of 16 R rows, 16 rows per load instruction
+  // instead of 64 pieces from 16 rows each; R KB per wavefront)
+  constexpr bool WST = XST && !TILED;
+  constexpr int kWaveStage = MT * 16 * ROWB + (WST ? R * 1024 : 0);
+  constexpr size_t kRedBytes = (size_t)WAVES * R * MT * 1024, kStageBytes = XST ? (size_t)WAVES * kWaveStage : 0;
   __shared__ __attribute__((aligned(16))) unsigned char smem[kRedBytes > kStageBytes ? kRedBytes : kStageBytes];
-  unsigned char* const xst = smem + (size_t)wave * (MT * 16 * ROWB);
+  unsigned char* const xst = smem + (size_t)wave * kWaveStage;
+  unsigned char* const wst = xst + MT * 16 * ROWB;
+  // loader: instruction t reads rows 16 t + lane / 4 of the workgroup's R tiles, piece (lane % 4) ^ (row / 4 % 4);
+  // operand lane (col, kq) of tile r finds its piece at position kq ^ (col / 4 % 4) of row 16 r + col
+  uint32_t wl_base[R];
+  int wl_piece = 0;
+  if constexpr (WST) {
+    wl_piece = (lane & 3) ^ ((lane >> 4) & 3);
+#pragma unroll
+    for (int t = 0; t < R; ++t) {
+      const int n = min((int)(blockIdx.x * R + t) * 16 + (lane >> 2), (int)n_stored - 1);
+      wl_base[t] = (uint32_t)n * row_bytes + (uint32_t)wl_piece * 16u;
+    }
+  }
+  const uint32_t ws_rd = (uint32_t)(col * 64 + ((kq ^ ((col >> 2) & 3)) * 16));
   // (256-byte rows span all 64 banks: 16 rows need 16 positions; 128-byte rows alternate between the bank halves,
   // so a pair of rows shares a position)
   auto swz = [](int row) { return PIECES == 16 ? (row & 15) : ((row >> 1) & 7); };
@@ -140,10 +158,18 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
                             : !TILED ? (uc >> group_shift) * 2u
                             : BITS == 4 ? (uc >> 3) * 256u + (c8 >> 1) * 64u + (c8 & 1u) * 2u : (uc >> 3) * 32u;
       const uint32_t xinc = (uint32_t)chunk * (CH * 2u);
+      if constexpr (WST) {
+        const bool okw = (ks < ks_end) && (ks * 4 + wl_piece < nchunks);
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        b.w[u][r] = load_b128(rw, wbase[r] + winc);  // valid base < 2^31: the sum cannot wrap
-        b.sc[u][r] = load_b16(rs, sbase[r] + sinc);
+        for (int t = 0; t < R; ++t) b.w[u][t] = load_b128(rw, okw ? wl_base[t] + (uint32_t)ks * 64u : kOobOffset);
+#pragma unroll
+        for (int r = 0; r < R; ++r) b.sc[u][r] = load_b16(rs, sbase[r] + sinc);
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          b.w[u][r] = load_b128(rw, wbase[r] + winc);  // valid base < 2^31: the sum cannot wrap
+          b.sc[u][r] = load_b16(rs, sbase[r] + sinc);
+        }
       }
       if constexpr (XST) {
         // line by line: instruction t reads ROWB bytes of RPI rows; a k-step past the end reads zeros
@@ -190,20 +216,27 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
             a[mt][j] = __builtin_bit_cast(half8_t, v);
           }
         }
+      if constexpr (WST) {
+#pragma unroll
+        for (int t = 0; t < R; ++t) *reinterpret_cast<u32x4*>(wst + t * 1024 + lane * 16) = b.w[u][t];
+      }
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const half2_t s2 = bcast_h2(__builtin_bit_cast(half_t, (uint16_t)b.sc[u][r]));
+        u32x4 wv;
+        if constexpr (WST) wv = *reinterpret_cast<const u32x4*>(wst + r * 1024 + ws_rd);
+        else wv = b.w[u][r];
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
           half8_t bm;
           if constexpr (BITS == 4) {
             half2_t h[4];
-            q4_word_paired(b.w[u][r][j], s2, qc, h);
+            q4_word_paired(wv[j], s2, qc, h);
             bm = pack_h8(h[0], h[1], h[2], h[3]);
           } else {
             half2_t h0[2], h1[2];
-            q8_word_natural(b.w[u][r][2 * j], s2, h0);
-            q8_word_natural(b.w[u][r][2 * j + 1], s2, h1);
+            q8_word_natural(wv[2 * j], s2, h0);
+            q8_word_natural(wv[2 * j + 1], s2, h1);
             bm = pack_h8(h0[0], h0[1], h1[0], h1[1]);
           }
 #pragma unroll
