@@ -174,7 +174,8 @@ LLAMA13B = [("qkv", 15360, 5120), ("o", 5120, 5120), ("gate_up", 27648, 5120), (
 
 def config_table(torch, dev, args) -> int:
     """Every (M, N, K) of the parity configurations timed alone: q4f16 g32 at the 7B shapes for
-    M in {1, 8, 512, 2048}, q8f16 g128 at the 13B shapes for M in {1, 16, 256}.  Each case rotates
+    M in {1, 8, 512, 2048}, q8f16 g128 at the 13B shapes for M in {1, 16, 256}, and both families at
+    32 and 64 rows (no parity configuration sits there).  Each case rotates
     through enough distinct weight sets (> 512 MB in total) that no launch finds its weights in a
     cache, inside one HIP graph; the time is the graph's divided by its launches.  Every case is
     timed on canonical and on tile-major weights."""
@@ -183,6 +184,9 @@ def config_table(torch, dev, args) -> int:
 
     cases = [(4, 32, m, n, k) for m in (1, 8, 512, 2048) for _, n, k in LLAMA7B]
     cases += [(8, 128, m, n, k) for m in (1, 16, 256) for _, n, k in LLAMA13B]
+    # between the configurations: the 17 to 64 row region (register-activation kernel, small GEMM tile)
+    cases += [(4, 32, m, n, k) for m in (32, 64) for _, n, k in LLAMA7B]
+    cases += [(8, 128, m, n, k) for m in (32, 64) for _, n, k in LLAMA13B]
     stream = torch.cuda.Stream()
     for bits, group, m, n, k in cases:
         wbytes = n * k * bits // 8 + n * (k // group) * 2
