@@ -164,10 +164,10 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
                                  ((d->bits == 4 && d->group == 32) || (d->bits == 8 && d->group == 128));
   if (tiled) {
     // On tile-major weights the skinny kernel's loads are contiguous and it holds out longer
-    // (N = 12288: 12.9 - 23.9 us from 17 to 64 rows against the GEMM's 23 - 25 us): the GEMM takes over from
-    // 40 rows with 160 or more column tiles (22016 x 4096: 27.0 against 27.8 us; int8 27648 x 5120: 47.7
-    // against 48.6 us).
-    if (direct_small_tile && tiles128 >= 160 && m >= 40) return MI355X_WQ_KERNEL_GEMM;
+    // (N = 12288: 12.9 - 23.9 us from 17 to 64 rows against the GEMM's 23 - 25 us): with 160 or more column
+    // tiles the GEMM takes over from 40 rows at int4 (22016 x 4096: 27.4 against 27.1 us) and from 49 rows
+    // at int8 (27648 x 5120: 44.0 against 48.7 us at 48 rows, 48.2 against 47.7 at 64).
+    if (direct_small_tile && tiles128 >= 160 && m >= (d->bits == 8 ? 49 : 40)) return MI355X_WQ_KERNEL_GEMM;
     return MI355X_WQ_KERNEL_SKINNY;
   }
   if (direct_small_tile && (tiles128 >= 160 || (d->bits == 4 && m > 48 && tiles128 >= 96)))

@@ -305,6 +305,8 @@ bool dispatch_variant(const Problem& p, int group_shift, int variant) {
         case 2: launch_one<BITS, 2, MT, 4, 2, true, true>(p, group_shift); return true;
         case 5: launch_one<BITS, 2, MT, 8, 1, true, true>(p, group_shift); return true;
         case 7: launch_one<BITS, 4, MT, 4, 1, true, true>(p, group_shift); return true;
+        case 8: launch_one<BITS, 4, MT, 8, 1, true, true>(p, group_shift); return true;
+        case 6: launch_one<BITS, 1, MT, 8, 1, true, true>(p, group_shift); return true;
         case 11: launch_one<BITS, 8, MT, 4, 1, true, true>(p, group_shift); return true;
         default: return false;
       }
@@ -314,6 +316,8 @@ bool dispatch_variant(const Problem& p, int group_shift, int variant) {
       case 2: launch_one<BITS, 2, MT, 4, 2, false, true>(p, group_shift); return true;
       case 5: launch_one<BITS, 2, MT, 8, 1, false, true>(p, group_shift); return true;
       case 7: launch_one<BITS, 4, MT, 4, 1, false, true>(p, group_shift); return true;
+      case 8: launch_one<BITS, 4, MT, 8, 1, false, true>(p, group_shift); return true;
+      case 6: launch_one<BITS, 1, MT, 8, 1, false, true>(p, group_shift); return true;
       case 11: launch_one<BITS, 8, MT, 4, 1, false, true>(p, group_shift); return true;
       default: return false;
     }
@@ -370,17 +374,25 @@ int launch_skinny(const Problem& p, int variant) {
     const int64_t tiles = (p.n + 15) / 16;
     // From 17 rows on the activations are staged through LDS (variants 21 ...: the same shapes with
     // line-by-line activation loads): 10 - 30 % faster from 32 rows on (4096 x 11008 at 64 rows 46 -> 35 us,
-    // int8 5120 x 13824 at 64 rows 72 -> 53 us), level at 17; not on tile-major int4 weights with 513 - 1024
-    // tiles (12288 x 4096 at 32 rows: 15.0 direct, 15.2 staged) and not with more than 1024 tiles.
+    // int8 5120 x 13824 at 64 rows 72 -> 53 us), level at 17.  With staged loads more wavefronts per
+    // workgroup pay: eight on one int4 tile (4096 x 4096 at 32 rows 8.9 -> 8.0 us, 4096 x 11008 at 64 rows
+    // 36.7 -> 30.4), eight on four tiles with 513 - 1024 tiles (12288 x 4096 at 48 rows 21.8 -> 20.6; not at
+    // four row blocks of int4, whose staging areas fill the LDS; there tile-major weights keep the direct loads).
     const bool staged = mt >= 2;
-    if (tiles <= 256) variant = staged ? 21 : 1;
+    if (tiles <= 256) variant = staged ? (p.bits == 4 ? 26 : 21) : 1;
     // (one tile per workgroup is 1.5 - 1.8x slower here; int8 at up to 4 rows on tile-major weights:
     // eight wavefronts, 3 - 5 % ahead)
     else if (tiles <= 512) variant = staged ? 25 : ((p.bits == 4 || (p.tiled && p.m <= 4)) ? 5 : 2);
-    else if (tiles <= 1024) variant = (staged && !(p.tiled && p.bits == 4)) ? 27 : 7;
-    // several rounds of workgroups: eight tiles share one pass over the activations (four for int8 on
-    // tile-major weights: 32000 x 4096 at 24 - 32 rows, 33.5 against 36.5 us)
-    else variant = mt == 1 ? 5 : (p.tiled && p.bits == 8 ? 7 : 11);
+    else if (tiles <= 1024) {
+      if (!staged) variant = 7;
+      else if (p.bits == 8 || mt <= 3) variant = 28;
+      else variant = p.tiled ? 7 : 27;  // (the same wavefront split on both layouts: their results are bit-equal)
+    }
+    // several rounds of workgroups: eight tiles share one pass over the activations; staged from 17 rows
+    // on for int8 (27648 x 5120 tile-major at 32 rows 43.4 -> 38.5 us) and for canonical int4 up to 48 rows
+    else if (!staged) variant = 5;
+    else if (p.bits == 8) variant = 31;
+    else variant = (!p.tiled && mt <= 3) ? 27 : 11;
   }
   bool ok;
   if (p.bits == 4) {

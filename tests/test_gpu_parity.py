@@ -167,7 +167,7 @@ def test_skinny_kernel_matches_oracle(variant, bits, m, n, k):
     assert_close(got, want, (variant, bits, m, n, k))
 
 
-@pytest.mark.parametrize("variant", [21, 22, 25, 27, 31])
+@pytest.mark.parametrize("variant", [21, 22, 25, 26, 27, 28, 31])
 @pytest.mark.parametrize("bits,m,n,k", [
     (4, 17, 33, 352), (4, 33, 64, 512), (4, 64, 80, 1152), (4, 48, 4096, 4096), (4, 31, 1000, 11008),
     (8, 20, 72, 640), (8, 64, 16, 1280), (8, 33, 5120, 5120), (8, 50, 300, 13824),
