@@ -71,10 +71,16 @@ def test_workspace_size_query_without_a_gpu():
     assert q(lib.make_desc(8, 128, 5120, 13824), 16, 1) == 16384 + 320 * 4 * 1024
     # 17 .. 64 rows: the GEMM's split on 64 x 128 tiles (32 KB per tile and window) from the measured row counts on
     assert q(lib.make_desc(4, 32, 4096, 11008), 48, 0) == 16384 + 32 * 8 * 32768
+    assert q(lib.make_desc(4, 32, 4096, 11008), 33, 0) == 16384 + 32 * 8 * 32768          # three row blocks on
+    assert q(lib.make_desc(4, 32, 4096, 11008), 33, 1) == 16384 + 32 * 8 * 32768
     assert q(lib.make_desc(4, 32, 4096, 11008), 32, 0) == 0 and q(lib.make_desc(4, 32, 4096, 4096), 48, 0) == 0
     assert q(lib.make_desc(8, 128, 5120, 13824), 17, 0) == 16384 + 40 * 6 * 32768
+    assert q(lib.make_desc(8, 128, 5120, 13824), 32, 1) == 0                              # tile-major int8: from 33
     assert q(lib.make_desc(4, 32, 4096, 4096), 64, 1) == 0                                # tile-major, short K: never
-    assert q(lib.make_desc(4, 32, 4096, 4096), 64, 0) == 16384 + 32 * 4 * 32768
+    # short K: only where the plain call runs the 64 x 128 tile anyway (int4, canonical, 49 rows on, 96 tiles on)
+    assert q(lib.make_desc(4, 32, 4096, 4096), 64, 0) == 0 and q(lib.make_desc(8, 128, 5120, 5120), 64, 0) == 0
+    assert q(lib.make_desc(4, 32, 12288, 4096), 64, 0) == 16384 + 96 * 2 * 32768
+    assert q(lib.make_desc(4, 32, 12288, 4096), 48, 0) == 0
     assert q(lib.make_desc(4, 32, 22016, 4096), 64, 0) == 0                              # 172 tiles fill the CUs
     # above 64 rows: 128 x 256 tiles (128 KB per tile and window)
     assert q(lib.make_desc(8, 128, 5120, 13824), 256, 0) == 16384 + 40 * 6 * 131072

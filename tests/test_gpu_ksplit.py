@@ -165,7 +165,7 @@ def test_workspace_entry_called_vm_style():
 
     vm_harness.set_stream()
     for bits, m, n, k in [(8, 2, 5120, 13824), (4, 16, 4096, 11008), (4, 8, 50, 512), (8, 256, 5120, 5120),
-                          (4, 64, 4096, 4096)]:  # decode split, no split, the GEMM's split above and below 64 rows
+                          (4, 64, 4096, 11008)]:  # decode split, no split, the GEMM's split above and below 64 rows
         x, wq, s, g = O.make_case(60 + m, m, n, k, bits)
         need = relax_amd.wq_workspace_bytes(bits, g, n, k, m)
         ws = torch.zeros(max(need, 64), dtype=torch.uint8, device="cuda")
@@ -215,8 +215,8 @@ def test_k_split_is_stable_while_another_stream_keeps_the_gpu_busy():
 GEMM_CASES = [(8, 256, 5120, 5120), (8, 256, 5120, 13824), (8, 256, 15360, 5120), (4, 256, 4096, 11008),
               (4, 128, 4096, 11008), (4, 200, 4090, 8192), (8, 65, 5120, 5120), (8, 384, 1000, 2048),
               # 17 .. 64 rows: 64 x 128 tiles, four K groups per workgroup
-              (4, 64, 4096, 4096), (4, 56, 12288, 4096), (8, 17, 5120, 13824), (4, 41, 4090, 11008),
-              (8, 60, 1000, 2048), (4, 64, 4096, 11008), (8, 64, 5120, 5120)]
+              (4, 64, 12288, 4096), (4, 56, 12288, 4096), (8, 17, 5120, 13824), (4, 41, 4090, 11008),
+              (8, 60, 1000, 8192), (4, 64, 4096, 11008), (8, 64, 5120, 8192), (4, 33, 2000, 8448)]
 
 
 @pytest.mark.parametrize("bits,m,n,k", GEMM_CASES)
