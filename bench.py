@@ -272,6 +272,36 @@ def config_table(torch, dev, args) -> int:
                 "workspace_speedup": None if us_ws is None else round(us / us_ws, 3)}
         print(json.dumps(line), flush=True)
         del ws, wt
+
+    # the exported dequantize (packed weights + scales in, float16 matrix out), same rotation and timing
+    for bits, group, shapes in ((4, 32, LLAMA7B), (8, 128, LLAMA13B)):
+        for _, n, k in shapes:
+            ab = n * k * bits // 8 + n * (k // group) * 2 + n * k * 2
+            sets = max(2, -(-(2048 << 20) // ab) + 1)
+            ws = [(torch.randint(-2**31, 2**31 - 1, (n, k * bits // 32), dtype=torch.int32, device=dev),
+                   (torch.rand((n, k // group), device=dev) * 0.01 + 0.002).to(torch.float16)) for _ in range(sets)]
+            outs = [torch.empty((n, k), dtype=torch.float16, device=dev) for _ in range(sets)]
+            with torch.cuda.stream(stream):
+                for (wq, s), o in zip(ws, outs):
+                    relax_amd.wq_dequantize(wq, s, bits, group, out=o)
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    for (wq, s), o in zip(ws, outs):
+                        relax_amd.wq_dequantize(wq, s, bits, group, out=o)
+                warm_replays(g)
+                reps = max(3, min(args.steps, 2000 // sets))
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(reps):
+                    g.replay()
+                e1.record(stream)
+                torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / (reps * sets)
+            print(json.dumps({"case": "dequantize q%df16 g%d N=%d K=%d" % (bits, group, n, k), "us": round(us, 2),
+                              "kernel": "dequant", "bytes": ab, "GB/s": round(ab / us / 1e3, 0),
+                              "frac_hbm": round(ab / us / 1e3 / HBM_PEAK_GBS, 3)}), flush=True)
+            del ws, outs, g
     return 0
 
 
