@@ -59,6 +59,24 @@ def test_dequantize_bit_exact(bits, n, k):
     assert np.array_equal(wd.cpu().numpy().view(np.uint16), want.view(np.uint16))
 
 
+@pytest.mark.parametrize("bits,group,n,k", [
+    (4, 32, 1, 32), (4, 32, 3, 8224), (4, 32, 257, 2080),      # the quad kernel: one quad, ragged last wavefronts
+    (8, 128, 1, 128), (8, 128, 9, 8320), (8, 128, 130, 1152),
+    (4, 64, 33, 4096), (4, 128, 7, 256), (4, 256, 5, 2304),     # other groups: one lane per 8 weights, rows of
+    (8, 32, 5, 96), (8, 64, 19, 2112), (8, 16, 3, 48),          # more and of fewer than 256 units
+])
+def test_dequantize_groups_and_ragged_ends(bits, group, n, k):
+    """Both dequantize kernels: the quad-per-lane one of the two standard quantizations at sizes that end inside a
+    wavefront, and the general one at other group sizes, on rows longer and shorter than a workgroup's span."""
+    import relax_amd
+
+    _, wq, s, g = O.make_case(300 + n + k, 1, n, k, bits, group)
+    wd = relax_amd.wq_dequantize(_dev(wq), _dev(s), bits, g)
+    torch.cuda.synchronize()
+    want = c_oracle.dequant(wq, s, bits, g, nthreads=8)
+    assert np.array_equal(wd.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 def test_dequantize_every_field_value_and_special_scales(bits):
     """All field values against scales that give zeros, subnormals, the largest finite value and inf."""
