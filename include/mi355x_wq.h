@@ -185,7 +185,7 @@ MI355X_WQ_API int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const vo
  * rows x 4096 x 11008: 50 -> 40-45 us; shapes the split would slow (short K, int4 with more tiles) report 0.
  * From 17 to 64 rows the split runs 64 x 128 tiles (32 KB of partials per tile and window) where the column tiles
  * fill at most half of the CUs and the other kernels have grown past its fixed cost: with K >= 8192 from 33 rows on
- * (int8 on canonical weights: from 17), with shorter K only for int4 on canonical weights above 48 rows with 96 or
+ * (int8 on canonical weights: from 25), with shorter K only for int4 on canonical weights above 48 rows with 96 or
  * more column tiles; 4096 x 11008 int4 at 64 rows 31 -> 22 us, 5120 x 13824 int8 at 64 rows 50 -> 34 us.
  * Workspace rules: device memory, 16-byte aligned, all zero before its first use (the kernel leaves it
  * ready for the next call); calls that share a workspace must not overlap in time (one stream, or

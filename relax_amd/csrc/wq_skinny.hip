@@ -31,6 +31,7 @@ struct SkinnyBatch {
   static constexpr int NJ = (128 / BITS) / 8;
   u32x4 w[U][R];
   uint32_t sc[U][R];
+  u32x2 ss[U][(R + 3) / 4];  // staged scales: a k-step's scales of 64 rows per load (canonical staged builds)
   u32x4 xa[U][MT][NJ];
 };
 
@@ -101,11 +102,28 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
   // (canonical weights take the same way: a k-step's 64 bytes of 16 R rows, 16 rows per load instruction
   // instead of 64 pieces from 16 rows each; R KB per wavefront)
   constexpr bool WST = XST && !TILED;
-  constexpr int kWaveStage = MT * 16 * ROWB + (WST ? R * 1024 : 0);
+  // (and so do their scales: a lane loads the 8 bytes -- int4, four groups -- or 2 bytes -- int8, one group -- that a
+  // row contributes to a k-step, one row per lane, instead of every lane its own 2 bytes from 16 rows per tile:
+  // a quarter of the scale loads.  The launcher admits these builds for the standard quantizations only, int4 with
+  // whole k-steps.)
+  constexpr int NSI = (R + 3) / 4;  // scale load instructions per k-step
+  constexpr int kWaveStage = MT * 16 * ROWB + (WST ? R * 1024 + NSI * 512 : 0);
   constexpr size_t kRedBytes = (size_t)WAVES * R * MT * 1024, kStageBytes = XST ? (size_t)WAVES * kWaveStage : 0;
   __shared__ __attribute__((aligned(16))) unsigned char smem[kRedBytes > kStageBytes ? kRedBytes : kStageBytes];
   unsigned char* const xst = smem + (size_t)wave * kWaveStage;
   unsigned char* const wst = xst + MT * 16 * ROWB;
+  unsigned char* const sst = wst + R * 1024;
+  uint32_t sl_base[NSI];
+  bool sl_ok[NSI];
+  if constexpr (WST) {
+#pragma unroll
+    for (int i = 0; i < NSI; ++i) {
+      const int row = i * 64 + lane;  // among the workgroup's R * 16 rows
+      sl_ok[i] = row < R * 16;
+      sl_base[i] = (uint32_t)min((int)(blockIdx.x * R) * 16 + row, (int)n_stored - 1) * groups_per_row * 2u;
+    }
+  }
+  const uint32_t ss_rd = BITS == 4 ? (uint32_t)(col * 8 + kq * 2) : (uint32_t)(col * 2);
   // loader: instruction t reads rows 16 t + lane / 4 of the workgroup's R tiles, piece (lane % 4) ^ (row / 4 % 4);
   // operand lane (col, kq) of tile r finds its piece at position kq ^ (col / 4 % 4) of row 16 r + col
   uint32_t wl_base[R];
@@ -163,7 +181,14 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
 #pragma unroll
         for (int t = 0; t < R; ++t) b.w[u][t] = load_b128(rw, okw ? wl_base[t] + (uint32_t)ks * 64u : kOobOffset);
 #pragma unroll
-        for (int r = 0; r < R; ++r) b.sc[u][r] = load_b16(rs, sbase[r] + sinc);
+        for (int i = 0; i < NSI; ++i) {
+          const bool oks = sl_ok[i] && ks < ks_end;
+          if constexpr (BITS == 4) {
+            b.ss[u][i] = load_b64(rs, oks ? sl_base[i] + (uint32_t)ks * 8u : kOobOffset);
+          } else {
+            b.ss[u][i][0] = load_b16(rs, oks ? sl_base[i] + ((uint32_t)ks >> 1) * 2u : kOobOffset);
+          }
+        }
       } else {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -219,10 +244,21 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
       if constexpr (WST) {
 #pragma unroll
         for (int t = 0; t < R; ++t) *reinterpret_cast<u32x4*>(wst + t * 1024 + lane * 16) = b.w[u][t];
+#pragma unroll
+        for (int i = 0; i < NSI; ++i) {
+          // every lane stores, also those past the workgroup's rows (the area holds 64 entries per instruction):
+          // behind a store under a condition the compiler may reuse the previous k-step's read for the lanes
+          // that do not store -- it does not know that other lanes' stores feed them
+          if constexpr (BITS == 4) *reinterpret_cast<u32x2*>(sst + (i * 64 + lane) * 8) = b.ss[u][i];
+          else *reinterpret_cast<uint16_t*>(sst + (i * 64 + lane) * 2) = (uint16_t)b.ss[u][i][0];
+        }
       }
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const half2_t s2 = bcast_h2(__builtin_bit_cast(half_t, (uint16_t)b.sc[u][r]));
+        uint16_t sbits;
+        if constexpr (WST) sbits = *reinterpret_cast<const uint16_t*>(sst + r * (BITS == 4 ? 128 : 32) + ss_rd);
+        else sbits = (uint16_t)b.sc[u][r];
+        const half2_t s2 = bcast_h2(__builtin_bit_cast(half_t, sbits));
         u32x4 wv;
         if constexpr (WST) wv = *reinterpret_cast<const u32x4*>(wst + r * 1024 + ws_rd);
         else wv = b.w[u][r];
@@ -298,6 +334,11 @@ void launch_one(const Problem& p, int group_shift) {
 template <int BITS, int MT>
 bool dispatch_variant(const Problem& p, int group_shift, int variant) {
   if (variant > 20 && MT < 2) return false;  // (one row block: the direct loads)
+  // the staged builds on canonical weights load a k-step's scales by row: standard quantizations, whole k-steps;
+  // anything else runs the direct form of the same shape
+  if (variant > 20 && !p.tiled && (group_shift != (BITS == 4 ? 0 : 3) || (BITS == 4 && p.k % 128 != 0))) variant -= 20;
+  // (so does int4 at four row blocks with eight wavefronts on four tiles: its staging areas exceed the LDS)
+  if (variant == 28 && !p.tiled && BITS == 4 && MT == 4) variant = 8;
   if (variant > 20) {  // staged activations (two row blocks and more), both layouts
     if (p.tiled) {
       switch (variant - 20) {
@@ -316,7 +357,13 @@ bool dispatch_variant(const Problem& p, int group_shift, int variant) {
       case 2: launch_one<BITS, 2, MT, 4, 2, false, true>(p, group_shift); return true;
       case 5: launch_one<BITS, 2, MT, 8, 1, false, true>(p, group_shift); return true;
       case 7: launch_one<BITS, 4, MT, 4, 1, false, true>(p, group_shift); return true;
-      case 8: launch_one<BITS, 4, MT, 8, 1, false, true>(p, group_shift); return true;
+      case 8:
+        // (int4 at four row blocks: the staging areas of eight wavefronts would not fit the LDS)
+        if constexpr (BITS == 8 || MT <= 3) {
+          launch_one<BITS, 4, MT, 8, 1, false, true>(p, group_shift);
+          return true;
+        }
+        return false;
       case 6: launch_one<BITS, 1, MT, 8, 1, false, true>(p, group_shift); return true;
       case 11: launch_one<BITS, 8, MT, 4, 1, false, true>(p, group_shift); return true;
       default: return false;

@@ -74,7 +74,8 @@ def test_workspace_size_query_without_a_gpu():
     assert q(lib.make_desc(4, 32, 4096, 11008), 33, 0) == 16384 + 32 * 8 * 32768          # three row blocks on
     assert q(lib.make_desc(4, 32, 4096, 11008), 33, 1) == 16384 + 32 * 8 * 32768
     assert q(lib.make_desc(4, 32, 4096, 11008), 32, 0) == 0 and q(lib.make_desc(4, 32, 4096, 4096), 48, 0) == 0
-    assert q(lib.make_desc(8, 128, 5120, 13824), 17, 0) == 16384 + 40 * 6 * 32768
+    assert q(lib.make_desc(8, 128, 5120, 13824), 25, 0) == 16384 + 40 * 6 * 32768
+    assert q(lib.make_desc(8, 128, 5120, 13824), 24, 0) == 0
     assert q(lib.make_desc(8, 128, 5120, 13824), 32, 1) == 0                              # tile-major int8: from 33
     assert q(lib.make_desc(4, 32, 4096, 4096), 64, 1) == 0                                # tile-major, short K: never
     # short K: only where the plain call runs the 64 x 128 tile anyway (int4, canonical, 49 rows on, 96 tiles on)
