@@ -155,10 +155,10 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
   // 17..64 rows.  The skinny kernel re-reads the activations from L2 once per 16-row weight tile, so
   // its time grows with M and N; the direct-weight GEMM with its 64x128 tile and four K groups costs
   // the same from 1 to 64 rows.  Measured crossovers on MI355X (q4f16 and q8f16, K = 4096 ... 13824, with
-  // the skinny kernel's activations staged through LDS): with 160 or more 128-column tiles the GEMM wins
-  // from 17 rows on (N = 22016: 28 us against 30 - 42 us; int8 N = 27648: 53 against 55 - 69 us), with 96 or
-  // more tiles of int4 weights from 49 rows on (N = 12288 at 56 rows: 26.7 against 27.8 us); with fewer the
-  // skinny kernel stays ahead up to 64 rows (8192 x 4096 at 64 rows: 16.9 against 24.2 us).
+  // the skinny kernel's activations, canonical weights and scales staged through LDS): the GEMM takes over only
+  // with 160 or more 128-column tiles, and there from the skinny kernel's third row block on (below); with fewer
+  // tiles the skinny kernel stays ahead up to 64 rows (12288 x 4096 at 64 rows: 24.7 against 25.7 us,
+  // 8192 x 8192: 28 against 43 us).
   const int64_t tiles128 = (d->n + 127) / 128;
   const bool direct_small_tile = d->k % 256 == 0 && d->k >= 1024 && tiles128 <= cu_count() &&
                                  ((d->bits == 4 && d->group == 32) || (d->bits == 8 && d->group == 128));
@@ -170,8 +170,9 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
     if (direct_small_tile && tiles128 >= 160 && m >= (d->bits == 8 ? 49 : 40)) return MI355X_WQ_KERNEL_GEMM;
     return MI355X_WQ_KERNEL_SKINNY;
   }
-  if (direct_small_tile && (tiles128 >= 160 || (d->bits == 4 && m > 48 && tiles128 >= 96)))
-    return MI355X_WQ_KERNEL_GEMM;
+  // canonical weights: with 160 or more column tiles the GEMM from 33 rows on (22016 x 4096: 29 us from 1 to 64
+  // rows against 26 - 27 us up to 32 rows and 33 - 45 us above; int8 27648 x 5120: 53 against 48 - 49 and 56 - 59)
+  if (direct_small_tile && tiles128 >= 160 && m >= 33) return MI355X_WQ_KERNEL_GEMM;
   return MI355X_WQ_KERNEL_SKINNY;
 }
 

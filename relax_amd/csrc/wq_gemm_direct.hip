@@ -706,8 +706,8 @@ int gemm_split_ways(const Problem& p) {
     // projection, 22 us on 4096 x 11008, 34 us on 5120 x 13824 int8, most of it start-up and the exchange -- so it
     // takes over where the other kernels have grown past it (measured on the Llama-2 7B / 13B projections):
     // with K of at least 8192 from 33 rows on (three row blocks in the register-activation kernel; int8 on
-    // canonical weights: from 25); with shorter K only where the plain call runs this tile anyway (int4 on
-    // canonical weights, more than 48 rows, 96 or more column tiles: 12288 x 4096 at 64 rows 26.2 -> 23.2 us).
+    // canonical weights: from 25); with shorter K only for int4 on canonical weights at more than 48 rows and
+    // 96 or more column tiles (12288 x 4096 at 64 rows 24.7 -> 23.1 us).
     const int64_t tiles128 = (p.n + 127) / 128;
     if (p.k >= 8192) {
       if (p.m < ((!p.tiled && p.bits == 8) ? 25 : 33)) return 1;

@@ -78,7 +78,7 @@ def test_workspace_size_query_without_a_gpu():
     assert q(lib.make_desc(8, 128, 5120, 13824), 24, 0) == 0
     assert q(lib.make_desc(8, 128, 5120, 13824), 32, 1) == 0                              # tile-major int8: from 33
     assert q(lib.make_desc(4, 32, 4096, 4096), 64, 1) == 0                                # tile-major, short K: never
-    # short K: only where the plain call runs the 64 x 128 tile anyway (int4, canonical, 49 rows on, 96 tiles on)
+    # short K: int4 on canonical weights only, from 49 rows and 96 column tiles on
     assert q(lib.make_desc(4, 32, 4096, 4096), 64, 0) == 0 and q(lib.make_desc(8, 128, 5120, 5120), 64, 0) == 0
     assert q(lib.make_desc(4, 32, 12288, 4096), 64, 0) == 16384 + 96 * 2 * 32768
     assert q(lib.make_desc(4, 32, 12288, 4096), 48, 0) == 0
@@ -144,11 +144,12 @@ def test_kernel_selection_by_rows():
     # skinny kernel grows with it
     wide, mid = lib.make_desc(4, 32, 22016, 4096), lib.make_desc(4, 32, 12288, 4096)
     assert L.mi355x_wq_select_kernel(wide, 16) == lib.KERNEL_GEMV
-    assert L.mi355x_wq_select_kernel(wide, 17) == lib.KERNEL_GEMM
-    assert L.mi355x_wq_select_kernel(mid, 48) == lib.KERNEL_SKINNY
-    assert L.mi355x_wq_select_kernel(mid, 49) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(wide, 32) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(wide, 33) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(mid, 64) == lib.KERNEL_SKINNY  # 96 column tiles: never
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 8192, 4096), 64) == lib.KERNEL_SKINNY
-    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 27648, 5120), 24) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 27648, 5120), 24) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 27648, 5120), 40) == lib.KERNEL_GEMM
     assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 15360, 5120), 48) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 22016, 4000), 48) == lib.KERNEL_SKINNY  # K % 256 != 0
     assert L.mi355x_wq_select_kernel(d, -1) == -1
