@@ -151,7 +151,16 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
     if (tiled && d->k >= 16384 && tiles <= cu_count() && m >= 8 && m <= 12) few_tiles = true;
     if (!tiny && !few_tiles) return MI355X_WQ_KERNEL_GEMV;
   }
-  if (m > kSkinnyMaxM) return MI355X_WQ_KERNEL_GEMM;
+  if (m > 64) {
+    // 65..128 rows: the GEMM's tiles leave most CUs idle on narrow projections (5120 x 5120 at 65 rows: 40 column
+    // tiles of 128, 43 us), where the register-activation kernel runs the rows as two grid slices (25 us).
+    // Measured on both layouts: it is ahead with up to 48 column tiles at int8 (16 at int4) for all 128 rows, and
+    // with up to 80 (32) up to 96 rows -- three row blocks per slice; beyond, level or behind.
+    const int64_t t128 = (d->n + 127) / 128;
+    if (m <= kSkinnyMaxM && (t128 <= (d->bits == 8 ? 48 : 16) || (m <= 96 && t128 <= (d->bits == 8 ? 80 : 32))))
+      return MI355X_WQ_KERNEL_SKINNY;
+    return MI355X_WQ_KERNEL_GEMM;
+  }
   // 17..64 rows.  The skinny kernel re-reads the activations from L2 once per 16-row weight tile, so
   // its time grows with M and N; the direct-weight GEMM with its 64x128 tile and four K groups costs
   // the same from 1 to 64 rows.  Measured crossovers on MI355X (q4f16 and q8f16, K = 4096 ... 13824, with

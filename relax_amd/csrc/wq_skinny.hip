@@ -44,8 +44,10 @@ struct SkinnyBatch {
 template <int BITS, int R, int MT, int WAVES, int U, bool TILED, bool XST = false>
 __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ wq, const half_t* __restrict__ scales,
-    half_t* y, int M, int N, int K, int group_shift, int zero_point, const Epilogue ep) {
+    half_t* y, int M, int N, int K, int group_shift, int zero_point, const Epilogue ep, int slice_rows) {
   constexpr int CH = 128 / BITS;  // k covered by one 16-byte lane load: 32 / 16
+  // more than 64 rows: blockIdx.y picks a slice of slice_rows (<= 16 MT) rows; every slice walks all weights
+  const int m0 = (int)blockIdx.y * slice_rows;
   constexpr int NJ = CH / 8;      // MFMAs fed by one lane load: 4 / 2
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform loop control
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
   }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + col;
+    const int m = m0 + mt * 16 + col;
     xrow_ok[mt] = m < M;
     xbase[mt] = (uint32_t)m * (uint32_t)K * 2u;
   }
@@ -150,8 +152,8 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
   uint32_t xl_base[XI];
 #pragma unroll
   for (int t = 0; t < XI; ++t) {
-    const int row = t * RPI + lane / PIECES;
-    const int piece = (lane % PIECES) ^ swz(row);
+    const int local = t * RPI + lane / PIECES, row = m0 + local;
+    const int piece = (lane % PIECES) ^ swz(local);
     xl_base[t] = (m_ok_row(row, M)) ? (uint32_t)row * (uint32_t)K * 2u + (uint32_t)piece * 16u : kOobOffset;
   }
 
@@ -313,7 +315,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) sum += red[w][t][i][l];
     const int r = t / MT, mt = t % MT;
-    const int m = mt * 16 + 4 * (l >> 4) + i;
+    const int m = m0 + mt * 16 + 4 * (l >> 4) + i;
     const int n = (blockIdx.x * R + r) * 16 + (l & 15);
     if (m < M && n < N) store_out(ep, y, m, n, N, sum);
   }
@@ -321,14 +323,21 @@ __global__ __launch_bounds__(WAVES * 64) void wq_skinny_kernel(
 
 namespace {
 
+// Rows per grid slice: up to 64 rows one slice; above, equal slices of whole 16-row blocks (80 rows: 2 x 48).
+int skinny_slice_rows(int64_t m) {
+  const int64_t slices = (m + 63) / 64;
+  return (int)(((m + slices - 1) / slices + 15) / 16 * 16);
+}
+
 template <int BITS, int R, int MT, int WAVES, int U, bool TILED = false, bool XST = false>
 void launch_one(const Problem& p, int group_shift) {
   const int tiles = (int)((p.n + 15) / 16);
-  dim3 grid((tiles + R - 1) / R), block(WAVES * 64);
+  const int slice_rows = skinny_slice_rows(p.m);
+  dim3 grid((tiles + R - 1) / R, (unsigned)((p.m + slice_rows - 1) / slice_rows)), block(WAVES * 64);
   hipLaunchKernelGGL((wq_skinny_kernel<BITS, R, MT, WAVES, U, TILED, XST>), grid, block, 0, p.stream,
                      (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                      (half_t*)p.y, (int)p.m, (int)p.n, (int)p.k, group_shift, p.zero_point,
-                     Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation});
+                     Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation}, slice_rows);
 }
 
 template <int BITS, int MT>
@@ -410,7 +419,7 @@ int launch_skinny(const Problem& p, int variant) {
     set_error("skinny kernel: M = %lld exceeds %lld", (long long)p.m, (long long)kSkinnyMaxM);
     return -1;
   }
-  const int mt = (int)((p.m + 15) / 16);
+  const int mt = (int)((std::min<int64_t>(p.m, skinny_slice_rows(p.m)) + 15) / 16);
   if (variant == 0) {
     // Measured on MI355X (q4f16, Llama-2-7B shapes, M = 4 .. 64): the number of workgroups is what
     // matters: as few tiles per workgroup as still give every CU at most one workgroup.

@@ -139,7 +139,15 @@ def test_kernel_selection_by_rows():
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 32000, 4096), 1) == lib.KERNEL_GEMV
     assert L.mi355x_wq_select_kernel(d, 17) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(d, 64) == lib.KERNEL_SKINNY
-    assert L.mi355x_wq_select_kernel(d, 65) == lib.KERNEL_GEMM
+    # 65..128 rows on narrow projections: two grid slices of the register-activation kernel
+    assert L.mi355x_wq_select_kernel(d, 65) == lib.KERNEL_SKINNY and L.mi355x_wq_select_kernel(d, 96) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(d, 97) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 2048, 8192), 128) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 2048, 8192), 129) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 5120, 13824), 128) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 10240, 5120), 96) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 10240, 5120), 112) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 12288, 4096), 65) == lib.KERNEL_GEMM
     # 17..64 rows on wide projections: the GEMM's 64x128 tile costs the same for any row count, the
     # skinny kernel grows with it
     wide, mid = lib.make_desc(4, 32, 22016, 4096), lib.make_desc(4, 32, 12288, 4096)
@@ -169,8 +177,8 @@ def test_pointer_checks_happen_before_any_launch():
     d0 = lib.make_desc(4, 32, 0, 64)
     assert L.mi355x_wq_matmul(d0, None, None, None, None, 3, None) == 0
     assert L.mi355x_wq_dequantize(d0, None, None, None, None) == 0
-    assert L.mi355x_wq_matmul_ex(d, ok, ok, ok, ok, 100, None, lib.KERNEL_SKINNY) == -1 \
-        and "exceeds 64" in lib.last_error()
+    assert L.mi355x_wq_matmul_ex(d, ok, ok, ok, ok, 200, None, lib.KERNEL_SKINNY) == -1 \
+        and "exceeds 128" in lib.last_error()
     assert L.mi355x_wq_matmul_ex(d, ok, ok, ok, ok, 1, None, 77) == -1 and "unknown kernel family" in lib.last_error()
 
 

@@ -211,6 +211,38 @@ def test_skinny_kernel_with_staged_activations(variant, bits, m, n, k):
         run_matmul(x[:8], wq, s, bits, g, kernel=lib.KERNEL_SKINNY, variant=variant)
 
 
+@pytest.mark.parametrize("bits,m,n,k", [
+    (4, 65, 4096, 4096), (4, 96, 200, 1280), (4, 128, 2048, 8192), (4, 81, 33, 352), (4, 112, 1000, 11008),
+    (8, 80, 5120, 5120), (8, 128, 300, 2304), (8, 97, 72, 640), (8, 66, 5120, 13824),
+])
+def test_skinny_kernel_in_two_row_slices(bits, m, n, k):
+    """65 .. 128 rows: the register-activation kernel runs the rows as two grid slices of whole 16-row blocks
+    (81 rows: 48 + 33).  Forced and, where the selection picks it, by default; against the oracle, bit-equal on
+    tile-major weights, and with a fused tail whose residual and output rows belong to the second slice too."""
+    import relax_amd
+    from relax_amd import lib
+
+    x, wq, s, g = O.make_case(170 + m + n, m, n, k, bits)
+    want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
+    got = run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_SKINNY)
+    assert_close(got, want, ("sliced", bits, m, n, k), ulp_fraction=0.005)
+    if lib.load().mi355x_wq_select_kernel(lib.make_desc(bits, g, n, k), m) == lib.KERNEL_SKINNY:
+        assert np.array_equal(run_matmul(x, wq, s, bits, g).view(np.uint16), got.view(np.uint16))
+    if k % 256 == 0:
+        wt, st = relax_amd.wq_tile_weights(_dev(wq), _dev(s), bits, g)
+        tiled = relax_amd.wq_matmul(_dev(x), wt, st, bits, g, tiled_n=n, kernel=lib.KERNEL_SKINNY)
+        torch.cuda.synchronize()
+        assert np.array_equal(tiled.cpu().numpy().view(np.uint16), got.view(np.uint16))
+    rng = np.random.default_rng(m + n)
+    bias = rng.standard_normal(n).astype(np.float16)
+    res = rng.standard_normal((m, n)).astype(np.float16)
+    fused = relax_amd.wq_matmul(_dev(x), _dev(wq), _dev(s), bits, g, kernel=lib.KERNEL_SKINNY, bias=_dev(bias),
+                                activation="relu", residual=_dev(res))
+    torch.cuda.synchronize()
+    want_f = c_oracle.wq_matmul_fused(x, wq, s, bits, g, bias=bias, activation="relu", residual=res, nthreads=16)
+    assert_close(fused.cpu().numpy(), want_f, ("sliced fused", bits, m, n, k), ulp_fraction=0.005)
+
+
 def test_config1_single_gemv_4096():
     """The reference's CPU-runnable case: x[1,4096] ~ N(0,1), W int4 4096x4096, group 32, zero point 7."""
     x, wq, s, g = O.make_case(0, 1, 4096, 4096, 4)

@@ -143,10 +143,15 @@ def test_tile_major_layout_is_refused_where_it_is_not_defined():
     s = torch.zeros((32, 8), dtype=torch.float16, device="cuda")
     with pytest.raises(lib.WqError, match="group 32"):
         relax_amd.wq_tile_weights(wq, s, 4, 64)
-    # int8 with K % 128 == 0 but K % 256 != 0: decode runs, a GEMM-sized batch is refused
-    x, wq8, s8, g = O.make_case(80, 100, 64, 384, 8)
+    # int8 with K % 128 == 0 but K % 256 != 0: decode and the register-activation kernel (up to 128 rows on a
+    # narrow projection) run, a GEMM-sized batch is refused
+    x, wq8, s8, g = O.make_case(80, 200, 64, 384, 8)
     wt, st = relax_amd.wq_tile_weights(_dev(wq8), _dev(s8), 8, g)
     relax_amd.wq_matmul(_dev(x[:8]), wt, st, 8, g, tiled_n=64)
+    y100 = relax_amd.wq_matmul(_dev(x[:100]), wt, st, 8, g, tiled_n=64)
+    ref100 = relax_amd.wq_matmul(_dev(x[:100]), _dev(wq8), _dev(s8), 8, g)
+    torch.cuda.synchronize()
+    assert torch.equal(y100.view(torch.int16), ref100.view(torch.int16))
     with pytest.raises(lib.WqError, match="direct-weight kernel"):
         relax_amd.wq_matmul(_dev(x), wt, st, 8, g, tiled_n=64)
 
