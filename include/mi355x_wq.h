@@ -153,7 +153,8 @@ MI355X_WQ_API int mi355x_wq_untile_weights(const mi355x_wq_desc* desc, const voi
 
 /* mi355x_wq_matmul_fused on tile-major weights (`ep` may be NULL).  The same three kernel families
  * (the decode kernel reads the contiguous stream, the skinny kernel and the direct-weight GEMM
- * address the layout) with crossovers measured on this layout; M > 64 needs K % 256 == 0. */
+ * address the layout) with crossovers measured on this layout; where the GEMM runs (more than 128 rows, more
+ * than 64 on wider projections) K % 256 == 0 is required. */
 MI355X_WQ_API int mi355x_wq_matmul_tiled(const mi355x_wq_desc* desc, const void* x, const void* wq_tiled,
                                         const void* scales_tiled, const mi355x_wq_epilogue* ep, void* y,
                                         int64_t m, void* stream);
