@@ -153,12 +153,12 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
   }
   if (m > 64) {
     // 65..128 rows: the GEMM's tiles leave most CUs idle on narrow projections (5120 x 5120 at 65 rows: 40 column
-    // tiles of 128, 43 us), where the register-activation kernel runs the rows as two grid slices (25 us).
-    // Measured on both layouts: it is ahead with up to 48 column tiles at int8 (16 at int4) for all 128 rows, and
-    // with up to 80 (32) up to 96 rows -- three row blocks per slice; beyond, level or behind.
+    // tiles of 128, 43 us; 4096 x 11008 int4: 54 us), where the register-activation kernel runs the rows as two
+    // grid slices (23 and 30 us).  Measured on both layouts: ahead or level with up to 64 column tiles at int4
+    // (8192 x 8192: 31 - 40 against 43 us) and up to 80 at int8 (10240 x 5120: 34 - 41 against 45 us), behind
+    // from 96 (12288 x 4096: 29 - 42 against 26 - 28 us) and 120 (15360 x 5120) on.
     const int64_t t128 = (d->n + 127) / 128;
-    if (m <= kSkinnyMaxM && (t128 <= (d->bits == 8 ? 48 : 16) || (m <= 96 && t128 <= (d->bits == 8 ? 80 : 32))))
-      return MI355X_WQ_KERNEL_SKINNY;
+    if (m <= kSkinnyMaxM && t128 <= (d->bits == 8 ? 80 : 64)) return MI355X_WQ_KERNEL_SKINNY;
     return MI355X_WQ_KERNEL_GEMM;
   }
   // 17..64 rows.  The skinny kernel re-reads the activations from L2 once per 16-row weight tile, so

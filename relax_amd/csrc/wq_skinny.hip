@@ -427,7 +427,10 @@ int launch_skinny(const Problem& p, int variant) {
     // tiles per workgroup, eight wavefronts for int4 and four for int8 (a second, mostly empty
     // round of workgroups costs more: 5120 x 13824 at 64 rows 114 -> 67 us); more: four
     // tiles per workgroup; many: two tiles per 8-wave workgroup for one row block, else four.
-    const int64_t tiles = (p.n + 15) / 16;
+    // (above 64 rows the grid has two slices of rows: what counts is tiles x slices -- 4096 x 4096 at 96 rows:
+    // two tiles per eight-wavefront workgroup 12.5 us, one tile 19.4)
+    const int64_t slices = (p.m + skinny_slice_rows(p.m) - 1) / skinny_slice_rows(p.m);
+    const int64_t tiles = (p.n + 15) / 16 * slices;
     // From 17 rows on the activations are staged through LDS (variants 21 ...: the same shapes with
     // line-by-line activation loads): 10 - 30 % faster from 32 rows on (4096 x 11008 at 64 rows 46 -> 35 us,
     // int8 5120 x 13824 at 64 rows 72 -> 53 us), level at 17.  With staged loads more wavefronts per
@@ -447,7 +450,7 @@ int launch_skinny(const Problem& p, int variant) {
     // several rounds of workgroups: eight tiles share one pass over the activations; staged from 17 rows
     // on for int8 (27648 x 5120 tile-major at 32 rows 43.4 -> 38.5 us) and for canonical int4 up to 48 rows
     else if (!staged) variant = 5;
-    else if (p.bits == 8) variant = 31;
+    else if (p.bits == 8) variant = slices > 1 ? 27 : 31;  // (10240 x 5120 at 96 rows: 36 against 44 us)
     else variant = (!p.tiled && mt <= 3) ? 27 : 11;
   }
   bool ok;

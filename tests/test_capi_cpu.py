@@ -140,13 +140,12 @@ def test_kernel_selection_by_rows():
     assert L.mi355x_wq_select_kernel(d, 17) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(d, 64) == lib.KERNEL_SKINNY
     # 65..128 rows on narrow projections: two grid slices of the register-activation kernel
-    assert L.mi355x_wq_select_kernel(d, 65) == lib.KERNEL_SKINNY and L.mi355x_wq_select_kernel(d, 96) == lib.KERNEL_SKINNY
-    assert L.mi355x_wq_select_kernel(d, 97) == lib.KERNEL_GEMM
-    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 2048, 8192), 128) == lib.KERNEL_SKINNY
-    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 2048, 8192), 129) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(d, 65) == lib.KERNEL_SKINNY and L.mi355x_wq_select_kernel(d, 128) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(d, 129) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 8192, 8192), 128) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 5120, 13824), 128) == lib.KERNEL_SKINNY
-    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 10240, 5120), 96) == lib.KERNEL_SKINNY
-    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 10240, 5120), 112) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 10240, 5120), 112) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 15360, 5120), 65) == lib.KERNEL_GEMM
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 12288, 4096), 65) == lib.KERNEL_GEMM
     # 17..64 rows on wide projections: the GEMM's 64x128 tile costs the same for any row count, the
     # skinny kernel grows with it
