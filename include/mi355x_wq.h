@@ -188,6 +188,8 @@ MI355X_WQ_API int mi355x_wq_matmul_tiled_ex(const mi355x_wq_desc* desc, const vo
  * fill at most half of the CUs and the other kernels have grown past its fixed cost: with K >= 8192 from 33 rows on
  * (int8 on canonical weights: from 25), with shorter K only for int4 on canonical weights above 48 rows with 96 or
  * more column tiles; 4096 x 11008 int4 at 64 rows 31 -> 22 us, 5120 x 13824 int8 at 64 rows 50 -> 34 us.
+ * (Above 64 rows on narrow projections, where the plain call runs the register-activation kernel in row slices,
+ * 0 is reported: that path is the faster one there.)
  * Workspace rules: device memory, 16-byte aligned, all zero before its first use (the kernel leaves it
  * ready for the next call); calls that share a workspace must not overlap in time (one stream, or
  * ordered by events); a workspace that is NULL or smaller than required disables the split for that call. */

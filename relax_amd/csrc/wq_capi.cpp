@@ -158,7 +158,11 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
     // (8192 x 8192: 31 - 40 against 43 us) and up to 80 at int8 (10240 x 5120: 34 - 41 against 45 us), behind
     // from 96 (12288 x 4096: 29 - 42 against 26 - 28 us) and 120 (15360 x 5120) on.
     const int64_t t128 = (d->n + 127) / 128;
-    if (m <= kSkinnyMaxM && t128 <= (d->bits == 8 ? 80 : 64)) return MI355X_WQ_KERNEL_SKINNY;
+    if (m <= 128 && t128 <= (d->bits == 8 ? 80 : 64)) return MI355X_WQ_KERNEL_SKINNY;
+    // and with three or four slices on the narrowest ones: int8 up to 48 column tiles up to 192 rows (5120 x 5120:
+    // 26 against 43 us; at 256 rows 38 against 43, and a workspace call takes 34), int4 up to 16 tiles up to 256
+    // rows (2048 x 8192: 23 - 26 against 40 us)
+    if (m <= kSkinnyMaxM && (d->bits == 8 ? (t128 <= 48 && m <= 192) : t128 <= 16)) return MI355X_WQ_KERNEL_SKINNY;
     return MI355X_WQ_KERNEL_GEMM;
   }
   // 17..64 rows.  The skinny kernel re-reads the activations from L2 once per 16-row weight tile, so
@@ -230,6 +234,7 @@ int64_t mi355x_wq_workspace_bytes(const mi355x_wq_desc* desc, int64_t m, int til
   if (m == 0 || desc->n == 0 || desc->k == 0) return 0;
   Problem p{nullptr, nullptr, nullptr, nullptr, m, desc->n, desc->k, desc->bits, desc->group, desc->zero_point, nullptr};
   p.tiled = tiled != 0;
+  if (m > 64 && select_kernel(desc, m, tiled != 0) == MI355X_WQ_KERNEL_SKINNY) return 0;  // (see mi355x_wq_matmul_ws)
   return m <= 16 ? gemv_split_workspace_bytes(p) : gemm_split_workspace_bytes(p);
 }
 
@@ -373,7 +378,10 @@ int matmul_any_layout(const mi355x_wq_desc* desc, const void* x, const void* wq_
   if (workspace != nullptr && family == MI355X_WQ_KERNEL_AUTO) {
     // a caller workspace allows the decode kernel's K split where it pays; everything else is as without
     if (!check_ptr(workspace, "workspace", 16)) return -1;
-    const int rc = m <= 16 ? launch_gemv_split(p, workspace, workspace_bytes) : launch_gemm_split(p, workspace, workspace_bytes);
+    // (above 64 rows, where the plain call runs row slices of the register-activation kernel, that is the faster
+    // one -- 5120 x 5120 int8 at 192 rows: 26 us against 34 us split -- and the workspace stays unused)
+    const bool sliced = m > 64 && select_kernel(desc, m, tiled) == MI355X_WQ_KERNEL_SKINNY;
+    const int rc = sliced ? 0 : m <= 16 ? launch_gemv_split(p, workspace, workspace_bytes) : launch_gemm_split(p, workspace, workspace_bytes);
     if (rc != 0) return rc < 0 ? -1 : 0;
   }
   if (library_scratch) {

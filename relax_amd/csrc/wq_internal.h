@@ -53,7 +53,7 @@ int launch_tile_weights(const Problem& p, void* wq_out, void* scales_out, bool f
 bool tiled_layout_defined(int bits, int group, int64_t k);
 
 // Upper bound of rows the skinny family accepts.
-constexpr int64_t kSkinnyMaxM = 128;  // (above 64 rows as two grid slices)
+constexpr int64_t kSkinnyMaxM = 256;  // (above 64 rows as grid slices)
 
 void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 

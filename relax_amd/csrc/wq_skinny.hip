@@ -427,7 +427,7 @@ int launch_skinny(const Problem& p, int variant) {
     // tiles per workgroup, eight wavefronts for int4 and four for int8 (a second, mostly empty
     // round of workgroups costs more: 5120 x 13824 at 64 rows 114 -> 67 us); more: four
     // tiles per workgroup; many: two tiles per 8-wave workgroup for one row block, else four.
-    // (above 64 rows the grid has two slices of rows: what counts is tiles x slices -- 4096 x 4096 at 96 rows:
+    // (above 64 rows the grid has two to four slices of rows: what counts is tiles x slices -- 4096 x 4096 at 96 rows:
     // two tiles per eight-wavefront workgroup 12.5 us, one tile 19.4)
     const int64_t slices = (p.m + skinny_slice_rows(p.m) - 1) / skinny_slice_rows(p.m);
     const int64_t tiles = (p.n + 15) / 16 * slices;

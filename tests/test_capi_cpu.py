@@ -142,6 +142,10 @@ def test_kernel_selection_by_rows():
     # 65..128 rows on narrow projections: two grid slices of the register-activation kernel
     assert L.mi355x_wq_select_kernel(d, 65) == lib.KERNEL_SKINNY and L.mi355x_wq_select_kernel(d, 128) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(d, 129) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 5120, 5120), 192) == lib.KERNEL_SKINNY  # three slices
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 5120, 5120), 193) == lib.KERNEL_GEMM
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 2048, 8192), 256) == lib.KERNEL_SKINNY   # four
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 2048, 8192), 257) == lib.KERNEL_GEMM
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 8192, 8192), 128) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 5120, 13824), 128) == lib.KERNEL_SKINNY
     assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 10240, 5120), 112) == lib.KERNEL_SKINNY
@@ -176,8 +180,8 @@ def test_pointer_checks_happen_before_any_launch():
     d0 = lib.make_desc(4, 32, 0, 64)
     assert L.mi355x_wq_matmul(d0, None, None, None, None, 3, None) == 0
     assert L.mi355x_wq_dequantize(d0, None, None, None, None) == 0
-    assert L.mi355x_wq_matmul_ex(d, ok, ok, ok, ok, 200, None, lib.KERNEL_SKINNY) == -1 \
-        and "exceeds 128" in lib.last_error()
+    assert L.mi355x_wq_matmul_ex(d, ok, ok, ok, ok, 300, None, lib.KERNEL_SKINNY) == -1 \
+        and "exceeds 256" in lib.last_error()
     assert L.mi355x_wq_matmul_ex(d, ok, ok, ok, ok, 1, None, 77) == -1 and "unknown kernel family" in lib.last_error()
 
 

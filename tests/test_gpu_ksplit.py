@@ -213,7 +213,7 @@ def test_k_split_is_stable_while_another_stream_keeps_the_gpu_busy():
 
 # (bits, M, N, K): prefill-side shapes whose 128 x 256 tiles fill at most half of the CUs
 GEMM_CASES = [(8, 256, 5120, 5120), (8, 256, 5120, 13824), (8, 256, 15360, 5120), (4, 256, 4096, 11008),
-              (4, 128, 4096, 11008), (4, 200, 4090, 8192), (8, 65, 5120, 5120), (8, 384, 1000, 2048),
+              (4, 160, 4096, 11008), (4, 200, 4090, 8192), (8, 200, 5120, 5120), (8, 384, 1000, 2048),
               # 17 .. 64 rows: 64 x 128 tiles, four K groups per workgroup
               (4, 64, 12288, 4096), (4, 56, 12288, 4096), (8, 25, 5120, 13824), (4, 41, 4090, 11008),
               (8, 60, 1000, 8192), (4, 64, 4096, 11008), (8, 64, 5120, 8192), (4, 33, 2000, 8448)]

@@ -214,10 +214,11 @@ def test_skinny_kernel_with_staged_activations(variant, bits, m, n, k):
 @pytest.mark.parametrize("bits,m,n,k", [
     (4, 65, 4096, 4096), (4, 96, 200, 1280), (4, 128, 2048, 8192), (4, 81, 33, 352), (4, 112, 1000, 11008),
     (8, 80, 5120, 5120), (8, 128, 300, 2304), (8, 97, 72, 640), (8, 66, 5120, 13824),
+    (8, 192, 5120, 5120), (8, 161, 200, 1280), (4, 256, 2048, 8192), (4, 200, 136, 768), (8, 250, 40, 384),
 ])
-def test_skinny_kernel_in_two_row_slices(bits, m, n, k):
-    """65 .. 128 rows: the register-activation kernel runs the rows as two grid slices of whole 16-row blocks
-    (81 rows: 48 + 33).  Forced and, where the selection picks it, by default; against the oracle, bit-equal on
+def test_skinny_kernel_in_row_slices(bits, m, n, k):
+    """65 .. 256 rows: the register-activation kernel runs the rows as two to four grid slices of whole 16-row
+    blocks (81 rows: 48 + 33).  Forced and, where the selection picks it, by default; against the oracle, bit-equal on
     tile-major weights, and with a fused tail whose residual and output rows belong to the second slice too."""
     import relax_amd
     from relax_amd import lib
