@@ -175,7 +175,7 @@ LLAMA13B = [("qkv", 15360, 5120), ("o", 5120, 5120), ("gate_up", 27648, 5120), (
 def config_table(torch, dev, args) -> int:
     """Every (M, N, K) of the parity configurations timed alone: q4f16 g32 at the 7B shapes for
     M in {1, 8, 512, 2048}, q8f16 g128 at the 13B shapes for M in {1, 16, 256}, and both families at
-    32 and 64 rows (no parity configuration sits there).  Each case rotates through distinct weight
+    32, 64 and 128 rows (no parity configuration sits there).  Each case rotates through distinct weight
     sets of more than 2 GB in total inside one HIP graph: no launch finds its weights in a cache, and
     the graph holds enough launches that its own start does not show.  The time is the graph's divided
     by its launches, taken after 50 ms of untimed replays.  Every case is
@@ -185,9 +185,9 @@ def config_table(torch, dev, args) -> int:
 
     cases = [(4, 32, m, n, k) for m in (1, 8, 512, 2048) for _, n, k in LLAMA7B]
     cases += [(8, 128, m, n, k) for m in (1, 16, 256) for _, n, k in LLAMA13B]
-    # between the configurations: the 17 to 64 row region (register-activation kernel, small GEMM tile)
-    cases += [(4, 32, m, n, k) for m in (32, 64) for _, n, k in LLAMA7B]
-    cases += [(8, 128, m, n, k) for m in (32, 64) for _, n, k in LLAMA13B]
+    # between the configurations: 17 to 128 rows (register-activation kernel, in row slices above 64; small GEMM tile)
+    cases += [(4, 32, m, n, k) for m in (32, 64, 128) for _, n, k in LLAMA7B]
+    cases += [(8, 128, m, n, k) for m in (32, 64, 128) for _, n, k in LLAMA13B]
     stream = torch.cuda.Stream()
 
     def warm_replays(g):

@@ -723,6 +723,10 @@ int gemm_split_ways(const Problem& p) {
   }
   const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 255) / 256);
   if (tiles * (p.bits == 4 ? 8 : 2) > cu || tiles > kGemmSplitMaxTiles) return 1;
+  // (not where the plain call's 64 x 128 tiles fill three quarters of the CUs or more in one round:
+  // 15360 x 5120 int8 at 128 rows, 240 tiles, 46 us plain against 49 us split)
+  const int64_t plain = ((p.m + 63) / 64) * ((p.n + 127) / 128);
+  if (p.m <= 128 && plain <= cu && plain * 4 >= cu * 3) return 1;
   const int64_t ways = std::min<int64_t>({cu / tiles, macro / (p.bits == 4 ? 8 : 4), 8});
   if (ways < (p.bits == 4 ? 4 : 2)) return 1;
   const int64_t per = (macro + ways - 1) / ways;  // macro steps per window; drop windows that would be empty
