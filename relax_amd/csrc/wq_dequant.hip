@@ -101,6 +101,10 @@ __global__ __launch_bounds__(256) void wq_dequant_quad_kernel(const uint32_t* __
   if (q < (idx_t)quads) *reinterpret_cast<u32x4*>(&words[wave][lane * 4]) = reinterpret_cast<const u32x4*>(wq)[q];
   if (lane < 64 / QPS && q0 + (idx_t)lane * QPS < (idx_t)quads)
     sc[wave][lane] = reinterpret_cast<const uint16_t*>(scales)[q0 / QPS + lane];
+  // (the loads below read other lanes' entries: the hardware runs a wavefront's LDS instructions in order, the
+  // fences keep the compiler from moving them across the stores)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
   for (int r = 0; r < UPQ; ++r) {
     const int u = 64 * r + lane;  // unit among this wavefront's 64 * UPQ

@@ -26,6 +26,12 @@ namespace wq {
 
 __device__ __forceinline__ bool m_ok_row(int row, int M) { return row < M; }
 
+// The wavefront-private LDS exchanges below (activations, canonical weights, scales) rely on two things: the
+// hardware executes a wavefront's LDS instructions in order, and every exchange is "all 64 lanes store, then all
+// load" with unconditional stores of the loaded type's size or more, which the compiler cannot move the loads
+// across or forward from (it must assume they alias).  Wavefront-scope fences between stores and loads state the
+// same explicitly but cost 2 - 4 % here (they also stop the scheduler from interleaving the exchanges of
+// neighbouring k-steps); the staged builds are pinned bit for bit against the direct ones by the tests instead.
 template <int BITS, int R, int MT, int U>
 struct SkinnyBatch {
   static constexpr int NJ = (128 / BITS) / 8;
