@@ -348,7 +348,6 @@ void launch_one(const Problem& p, int group_shift) {
 
 template <int BITS, int MT>
 bool dispatch_variant(const Problem& p, int group_shift, int variant) {
-  if (variant > 20 && MT < 2) return false;  // (one row block: the direct loads)
   // the staged builds on canonical weights load a k-step's scales by row: standard quantizations, whole k-steps;
   // anything else runs the direct form of the same shape
   if (variant > 20 && !p.tiled && (group_shift != (BITS == 4 ? 0 : 3) || (BITS == 4 && p.k % 128 != 0))) variant -= 20;
@@ -443,8 +442,12 @@ int launch_skinny(const Problem& p, int variant) {
     // workgroup pay: eight on one int4 tile (4096 x 4096 at 32 rows 8.9 -> 8.0 us, 4096 x 11008 at 64 rows
     // 36.7 -> 30.4), eight on four tiles with 513 - 1024 tiles (12288 x 4096 at 48 rows 21.8 -> 20.6; not at
     // four row blocks of int4, whose staging areas fill the LDS; there tile-major weights keep the direct loads).
+    // One row block (up to 16 rows, where the decode kernel does not apply): the staged loads pay on the two
+    // ends -- at most one tile per CU from 9 rows on and for int8 (2048 x 2048 int8: 4.7 - 5.9 -> 4.2 - 4.6 us),
+    // and with several rounds of workgroups (a 152064 x 4096 vocabulary projection: 108 - 153 -> 91 - 102 us,
+    // tile-major 75 - 106 -> 70 - 76).
     const bool staged = mt >= 2;
-    if (tiles <= 256) variant = staged ? (p.bits == 4 ? 26 : 21) : 1;
+    if (tiles <= 256) variant = staged ? (p.bits == 4 ? 26 : 21) : (p.bits == 8 || p.m >= 9) ? 26 : 1;
     // (one tile per workgroup is 1.5 - 1.8x slower here; int8 at up to 4 rows on tile-major weights:
     // eight wavefronts, 3 - 5 % ahead)
     else if (tiles <= 512) variant = staged ? 25 : ((p.bits == 4 || (p.tiled && p.m <= 4)) ? 5 : 2);
@@ -455,7 +458,7 @@ int launch_skinny(const Problem& p, int variant) {
     }
     // several rounds of workgroups: eight tiles share one pass over the activations; staged from 17 rows
     // on for int8 (27648 x 5120 tile-major at 32 rows 43.4 -> 38.5 us) and for canonical int4 up to 48 rows
-    else if (!staged) variant = 5;
+    else if (!staged) variant = 27;
     else if (p.bits == 8) variant = slices > 1 ? 27 : 31;  // (10240 x 5120 at 96 rows: 36 against 44 us)
     else variant = (!p.tiled && mt <= 3) ? 27 : 11;
   }

@@ -207,8 +207,10 @@ def test_skinny_kernel_with_staged_activations(variant, bits, m, n, k):
         tiled = relax_amd.wq_matmul(_dev(x), wt, st, bits, g, tiled_n=n, kernel=lib.KERNEL_SKINNY, variant=variant)
         torch.cuda.synchronize()
         assert np.array_equal(tiled.cpu().numpy().view(np.uint16), got.view(np.uint16))
-    with pytest.raises(lib.WqError, match="unknown variant"):
-        run_matmul(x[:8], wq, s, bits, g, kernel=lib.KERNEL_SKINNY, variant=variant)
+    # one row block: the same builds, bit-equal to the direct form as well
+    few = run_matmul(x[:8], wq, s, bits, g, kernel=lib.KERNEL_SKINNY, variant=variant)
+    few_direct = run_matmul(x[:8], wq, s, bits, g, kernel=lib.KERNEL_SKINNY, variant=variant - 20)
+    assert np.array_equal(few.view(np.uint16), few_direct.view(np.uint16))
 
 
 @pytest.mark.parametrize("bits,m,n,k", [
