@@ -127,9 +127,6 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
   Problem p{nullptr, nullptr, nullptr, nullptr, m, d->n, d->k, d->bits, d->group, d->zero_point, nullptr};
   if (gemv_applicable(p)) {
     // The GEMV kernel stages the activations in LDS, in K phases when they do not fit in one piece.
-    // (A rule that sent such problems with at most one row tile per CU to the register-activation
-    // kernel dated from a slower staging path: 16 rows on 4096 x 11008 now take 15.5 against 16.7 us,
-    // 8 rows 12.7 against 12.8 us.)
     const int64_t tiles = (d->n + 15) / 16;
     // (with at most 2048 columns of K and 256 row tiles the matrix is so small -- 4 MB -- that the
     // staging kernel's start-up costs more than it saves: 4096 x 2048, 5.6 against 4.9 us)
@@ -149,6 +146,11 @@ int select_kernel(const mi355x_wq_desc* d, int64_t m, bool tiled = false) {
     // (rows of 16384 and more, one tile per CU: the staging kernel at batch 1 - 4, 17.7 against 19.8 us, the
     // other at 8 - 12 rows, 14.7 against 16.7 us)
     if (tiled && d->k >= 16384 && tiles <= cu_count() && m >= 8 && m <= 12) few_tiles = true;
+    // int4 from 9 rows on with activations beyond the LDS (K phases in the staging kernel) and at most two row
+    // tiles per CU: the register-activation kernel with its staged loads, on both layouts (4096 x 11008 at
+    // 9 - 16 rows: 13.0 - 14.3 against 14.7 - 15.6 us, tile-major 11.9 - 12.8 against 13.2 - 14.0;
+    // 5120 x 13824: 21 - 22 against 24 - 25 us)
+    if (d->bits == 4 && m >= 9 && m * d->k * 2 > 144 * 1024 && tiles <= 2 * cu_count() && d->k < 16384) few_tiles = true;
     if (!tiny && !few_tiles) return MI355X_WQ_KERNEL_GEMV;
   }
   if (m > 64) {

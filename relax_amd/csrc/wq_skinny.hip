@@ -450,7 +450,7 @@ int launch_skinny(const Problem& p, int variant) {
     if (tiles <= 256) variant = staged ? (p.bits == 4 ? 26 : 21) : (p.bits == 8 || p.m >= 9) ? 26 : 1;
     // (one tile per workgroup is 1.5 - 1.8x slower here; int8 at up to 4 rows on tile-major weights:
     // eight wavefronts, 3 - 5 % ahead)
-    else if (tiles <= 512) variant = staged ? 25 : ((p.bits == 4 || (p.tiled && p.m <= 4)) ? 5 : 2);
+    else if (tiles <= 512) variant = (staged || p.m >= 9) ? 25 : ((p.bits == 4 || (p.tiled && p.m <= 4)) ? 5 : 2);
     else if (tiles <= 1024) {
       if (!staged) variant = 7;
       else if (p.bits == 8 || mt <= 3) variant = 28;

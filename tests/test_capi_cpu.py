@@ -127,8 +127,11 @@ def test_kernel_selection_by_rows():
     assert L.mi355x_wq_select_kernel(d, 8) == lib.KERNEL_GEMV
     # 16 rows x 4096 = 128 KB of activations still fit the LDS in one piece
     assert L.mi355x_wq_select_kernel(d, 16) == lib.KERNEL_GEMV
-    # 16 rows x 8192 = 256 KB: staged in K phases
-    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 8192), 16) == lib.KERNEL_GEMV
+    # 16 rows x 8192 = 256 KB would be staged in K phases: int4 from 9 rows on goes to the register-activation kernel
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 8192), 16) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 8192), 9) == lib.KERNEL_GEMV   # 144 KB: one piece
+    assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 11008), 9) == lib.KERNEL_SKINNY
+    assert L.mi355x_wq_select_kernel(lib.make_desc(8, 128, 5120, 13824), 16) == lib.KERNEL_GEMV
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 22016, 4096), 16) == lib.KERNEL_GEMV
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 11008), 2) == lib.KERNEL_GEMV
     assert L.mi355x_wq_select_kernel(lib.make_desc(4, 32, 4096, 11008), 8) == lib.KERNEL_GEMV
