@@ -56,21 +56,35 @@ struct GemvBuf {
   uint32_t sc[SPL > 1 ? SPL / 2 : 1];  // SPL float16 scales, packed two per register
 };
 
-struct GemvArgs {
+// What a wavefront walks in one K phase: of every tile of its workgroup the super steps start .. start + cnt - 1
+// (the phase's super steps dealt out evenly: the first `nsuper % WAVES` wavefronts take one more).
+struct GemvCtx {
+  int chunk_base;  // first chunk of the phase
+  int nsuper;      // super steps of the phase
+  int start, cnt;
+};
+
+// The kernel's argument segment as a struct (arguments are laid out in order with their natural alignment):
+// the kernel reads the arguments that only its last section needs -- the output, the epilogue, the K split's
+// workspace -- through the segment pointer, behind an optimisation barrier at the start of that section.  Left to
+// itself the compiler fetches them at the top of the kernel and, in the builds that run short of scalar registers,
+// waits for that fetch (a trip to host-visible memory) to spill them: ahead of the first weight request.
+struct GemvKernArgs {
   const half_t* x;
   const uint32_t* wq;
   const half_t* scales;
+  int M, N, K, shift_and_zero, max_tiles, phase_chunks, ksplit, grid;
   half_t* y;
-  int M, N, K;
-  int group_shift, zero_point;
-  int lds_stride;    // halves per staged activation row
-  int tiles;         // ceil(N / 16)
-  int max_tiles;     // tiles per workgroup, upper bound (slot array extent)
-  int phase_chunks;  // chunks per K phase (multiple of 4*D)
   Epilogue ep;
+  float* partials;
+  unsigned int* counters;
 };
 
-template <int BITS, int WAVES, int D, int SPL, bool TILED, bool ROWS, bool KSPLIT>
+template <int BITS, int WAVES, int D, int SPL, bool TILED, bool ROWS, bool KSPLIT, bool PHASES>
+// PHASES: the launch walks K in more than one phase (activations beyond the LDS).  The host knows; as a template
+// flag it keeps the second phase description out of the build that runs the common launches, whose first memory
+// requests otherwise wait behind that bookkeeping (and behind the late kernel arguments, which the compiler
+// fetched early and spilled when the scalar registers ran out).
 // Scalar kernel arguments instead of one struct, and in this order: the first 14 dwords of the
 // argument segment are preloaded into SGPRs at wavefront launch (16 user SGPRs less the segment
 // pointer); anything after them is fetched by a scalar load from host-visible memory.
@@ -78,32 +92,24 @@ template <int BITS, int WAVES, int D, int SPL, bool TILED, bool ROWS, bool KSPLI
 // plan and the grid size (gridDim.x is itself a load from the end of the segment), 14 dwords --
 // therefore comes first, and what only the final store needs (y, the epilogue, the K split's
 // workspace) after it.
-__global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
+// (at least two wavefronts per SIMD as far as registers go, also for the 4-wavefront builds: with 512
+// registers to hand the compiler keeps the accumulator in AGPRs and copies it to and from VGPRs around the
+// stream loop, and a copy out of the AGPRs that a taken branch puts right behind the last MFMA reads the
+// registers before the MFMA has written them -- the wait states are missing on that path; the 4-wavefront
+// builds lost part of a super step's sum in two of four accumulator registers that way)
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8))) void wq_gemv_kernel(
     const half_t* x_, const uint32_t* wq_, const half_t* scales_, int M_, int N_, int K_,
-    int shift_and_zero_, int max_tiles_, int phase_chunks_, int ksplit_, int grid_, half_t* y_, const Epilogue ep_,
-    float* partials_, unsigned int* counters_) {
+    int shift_and_zero_, int max_tiles_, int phase_chunks_, int ksplit_, int grid_, half_t* y_late, const Epilogue ep_late,
+    float* partials_late, unsigned int* counters_late) {
+  static_assert(!KSPLIT || !PHASES, "the cross-workgroup K split walks one window of K");
+  constexpr bool XPRE = PHASES && ROWS;  // (up to eight rows) a phase's activations are requested a phase ahead
   const int group_shift_ = shift_and_zero_ & 0xFF, zero_point_ = (shift_and_zero_ >> 8) & 0xFF;
   const bool gated = (shift_and_zero_ >> 16) & 1;  // fused multiply(nn.silu(gate), up): rows walked interleaved
   const int tiles_ = (N_ + 15) >> 4;
-  const int lds_stride_ = phase_chunks_ * (128 / BITS) + 8;  // halves per staged row (launch_one's plan)
-  GemvArgs a;
-  a.x = x_;
-  a.wq = wq_;
-  a.scales = scales_;
-  a.y = y_;
-  a.M = M_;
-  a.N = N_;
-  a.K = K_;
-  a.group_shift = group_shift_;
-  a.zero_point = zero_point_;
-  a.lds_stride = lds_stride_;
-  a.tiles = tiles_;
-  a.max_tiles = max_tiles_;
-  a.phase_chunks = phase_chunks_;
-  a.ep = ep_;
   constexpr int CH = 128 / BITS;  // k per 16-byte lane load
   constexpr int NJ = CH / 8;      // MFMAs per lane load
   constexpr int NT = WAVES * 64;
+  const int lds_stride = phase_chunks_ * CH + 8;  // halves per staged row (launch_one's plan)
   static_assert(SPL == 1 || SPL == D, "one scale per super step, or one per chunk");
   static_assert(!TILED || D == 2, "the tile-major layout is written for super steps of eight chunks");
   static_assert(SPL == 1 || (SPL % 2 == 0 && SPL <= 8), "scale vector is 4, 8 or 16 bytes");
@@ -111,21 +117,21 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps loop control scalar
   const int col = lane & 15, kq = lane >> 4;
-  const int M = a.M, N = a.N, K = a.K;
+  const int M = M_, N = N_, K = K_;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char wq_gemv_smem[];
   // [max_tiles][WAVES][4][64] float partial tiles, then [M][lds_stride] staged activations
   float* slots = reinterpret_cast<float*>(wq_gemv_smem);
-  half_t* xs = reinterpret_cast<half_t*>(wq_gemv_smem + (size_t)a.max_tiles * WAVES * 1024);
+  half_t* xs = reinterpret_cast<half_t*>(wq_gemv_smem + (size_t)max_tiles_ * WAVES * 1024);
 
   const uint32_t row_bytes = (uint32_t)K * BITS / 8;
   const int nchunks = K / CH;
-  const uint32_t groups_per_row = (uint32_t)nchunks >> a.group_shift;
+  const uint32_t groups_per_row = (uint32_t)nchunks >> group_shift_;
   // (the tile-major buffers hold whole tiles: rows up to the next multiple of 16, zero filled)
-  const uint32_t n_stored = TILED ? (uint32_t)a.tiles * 16u : (uint32_t)N;
-  const rsrc_t rw = make_rsrc(a.wq, n_stored * row_bytes);
-  const rsrc_t rs = make_rsrc(a.scales, n_stored * groups_per_row * 2u);
-  const rsrc_t rx = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
+  const uint32_t n_stored = TILED ? (uint32_t)tiles_ * 16u : (uint32_t)N;
+  const rsrc_t rw = make_rsrc(wq_, n_stored * row_bytes);
+  const rsrc_t rs = make_rsrc(scales_, n_stored * groups_per_row * 2u);
+  const rsrc_t rx = make_rsrc(x_, (uint32_t)M * (uint32_t)K * 2u);
 
   // Tiles of this workgroup: tile0, tile0 + tstride, ...  With the K split, R consecutive workgroups
   // share a tile list and each walks its own window of K (phase_chunks chunks from kr * phase_chunks).
@@ -135,21 +141,44 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
   const int tile0 = KSPLIT ? (int)blockIdx.x / R : (int)blockIdx.x;
   const int tstride = KSPLIT ? G / R : G;
   // (= ceil((tiles - tile0) / tstride) without the division: max_tiles is the ceiling for tile0 = 0)
-  const int my_tiles = a.max_tiles - (tile0 + (a.max_tiles - 1) * tstride >= a.tiles ? 1 : 0);
+  const int my_tiles = max_tiles_ - (tile0 + (max_tiles_ - 1) * tstride >= tiles_ ? 1 : 0);
 
-  const Q4Consts qc = make_q4_consts(a.zero_point);
-  const half_t* xrow = xs + (size_t)(col < M ? col : 0) * a.lds_stride;
+  const Q4Consts qc = make_q4_consts(zero_point_);
+  const half_t* xrow = xs + (size_t)(col < M ? col : 0) * lds_stride;
 
-  // weights of (tile index i, super step ss of the current phase) -> registers
-  auto load_super = [&](GemvBuf<D, SPL>& b, int i, int ss, int chunk_base, int ss_end) {
+  auto make_ctx = [&](int chunk_base) -> GemvCtx {
+    GemvCtx c;
+    c.chunk_base = chunk_base;
+    const int ph_chunks = min(phase_chunks_, nchunks - chunk_base);
+    c.nsuper = ph_chunks > 0 ? (ph_chunks + 4 * D - 1) / (4 * D) : 0;
+    const int base = c.nsuper / WAVES, extra = c.nsuper % WAVES;
+    c.cnt = base + (wave < extra ? 1 : 0);
+    c.start = wave * base + min(wave, extra);
+    return c;
+  };
+  const GemvCtx dead_ctx = GemvCtx{nchunks, 0, 0, 0};
+  // the items of a phase in the order a wavefront walks them: (tile index i, step s); i = my_tiles: no item
+  auto first_tile = [&](const GemvCtx& c) { return c.cnt > 0 ? 0 : my_tiles; };
+  auto advance = [&](const GemvCtx& c, int& i, int& s) {
+    if (++s >= c.cnt) {
+      s = 0;
+      ++i;
+    }
+  };
+
+  // weights of item (i, s) of phase `c` -> registers; anything that is no item loads zeros
+  auto load_super = [&](GemvBuf<D, SPL>& b, const GemvCtx& c, int i, int s) {
+    const int ss = c.start + s;  // super step within the phase
+    const int tile = tile0 + i * tstride;
+    bool ok = i < my_tiles;
     if constexpr (TILED) {
       // Tile-major stream: the D 1 KB blocks of (tile, super step) are consecutive and lane l owns
       // bytes 16 l .. 16 l + 15 of each -- every load instruction of the wavefront reads 1 KB
       // contiguously.  Scales: int4 / group 32 one 4-byte pair per lane, int8 / group 128 one
       // float16 per (row, super step).
       const uint32_t nsuper_all = (uint32_t)nchunks / (4 * D);
-      const uint32_t item = (uint32_t)(tile0 + i * tstride) * nsuper_all + (uint32_t)(chunk_base / (4 * D) + ss);
-      const bool ok = (i < my_tiles) && (ss < ss_end) && (chunk_base + ss * 4 * D < nchunks);
+      const uint32_t item = (uint32_t)tile * nsuper_all + (uint32_t)(c.chunk_base / (4 * D) + ss);
+      ok = ok && (c.chunk_base + ss * 4 * D < nchunks);
       const uint32_t woff = ok ? item * (D * 1024u) + (uint32_t)lane * 16u : kOobOffset;
 #pragma unroll
       for (int d = 0; d < D; ++d) b.w[d] = load_b128(rw, woff + d * 1024u);
@@ -157,15 +186,15 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
       else b.sc[0] = load_b32(rs, ok ? (item * 64u + (uint32_t)lane) * 4u : kOobOffset);
       return;
     }
-    int n = min((tile0 + i * tstride) * 16 + col, N - 1);  // rows past N: computed, not stored
+    int n = min(tile * 16 + col, N - 1);      // rows past N: computed, not stored
     if (gated) n = gated_physical_row(n, N);  // even columns of a tile: gate rows, odd columns: their up rows
-    const int chunk0 = chunk_base + ss * 4 * D + kq * D;
+    const int chunk0 = c.chunk_base + ss * 4 * D + kq * D;
     // D > 1 is only launched when K is a multiple of 4*D chunks, so a lane's D
     // chunks are valid together; D == 1 checks its single chunk.
-    const bool ok = (i < my_tiles) && (ss < ss_end) && (chunk0 < nchunks);
+    ok = ok && (chunk0 < nchunks);
     const uint32_t woff = ok ? (uint32_t)n * row_bytes + (uint32_t)chunk0 * 16u : kOobOffset;
     const uint32_t soff =
-        ok ? ((uint32_t)n * groups_per_row + ((uint32_t)chunk0 >> a.group_shift)) * 2u : kOobOffset;
+        ok ? ((uint32_t)n * groups_per_row + ((uint32_t)chunk0 >> group_shift_)) * 2u : kOobOffset;
 #pragma unroll
     for (int d = 0; d < D; ++d) b.w[d] = load_b128(rw, woff + d * 16u);
     if constexpr (SPL == 1) {
@@ -183,11 +212,13 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     }
   };
 
+  // staged activations of step s of the phase
+  auto x_of = [&](const GemvCtx& c, int s) -> const half_t* { return xrow + ((c.start + s) * 4 * D + kq * D) * CH; };
+
   float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  // one super step of MFMAs; `ss_local` addresses the staged activations of this phase
-  auto compute_super = [&](const GemvBuf<D, SPL>& b, int ss_local) {
-    const half_t* xp = xrow + (ss_local * 4 * D + kq * D) * CH;
+  // one super step of MFMAs on the staged activations at xp
+  auto compute_super = [&](const GemvBuf<D, SPL>& b, const half_t* xp) {
     half8_t av[2][NJ];  // activations of chunk d+1 are read from LDS while chunk d is consumed
 #pragma unroll
     for (int j = 0; j < NJ; ++j) av[0][j] = *reinterpret_cast<const half8_t*>(xp + j * 8);
@@ -228,90 +259,124 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
     acc = float4_t{0.f, 0.f, 0.f, 0.f};
   };
 
+  // The weight stream is one software pipeline over all K phases: the register set that a phase's last trip
+  // frees is filled with the first item of the next phase, so that the phase boundary (a barrier, the
+  // activations of the next K range into LDS, a barrier) does not find the memory pipeline empty.
+  GemvBuf<D, SPL> b0, b1;
+  // (the late arguments: fetched from the argument segment once the first phase's requests are out, see GemvKernArgs)
+  half_t* y_ = nullptr;
+  Epilogue ep_ = Epilogue{nullptr, nullptr, 0};
+  float* partials_ = nullptr;
+  unsigned int* counters_ = nullptr;
+  u32x4 xn[XPRE ? 8 : 1];  // XPRE: this thread's column of the next phase's activations, requested a phase ahead
+
+  auto permute_x = [&](u32x4 v) -> u32x4 {
+    if constexpr (BITS == 4) {
+      u32x4 p;
+      p[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
+      p[1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
+      p[2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
+      p[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
+      return p;
+    } else {
+      return v;
+    }
+  };
+  // 16-byte vector kv of activation row m in the phase that starts at chunk `chunk_base` (zeros past the
+  // phase, the row or K), and its place in LDS
+  auto x_load_of = [&](const GemvCtx& c, int m, int kv) -> u32x4 {
+    const int kbase = c.chunk_base * CH;
+    const int vec_per_row = ((c.nsuper * 4 * D + 3) / 4) * 4 * CH / 8;
+    const bool ok = m < M && kv < vec_per_row && kbase + kv * 8 < K;
+    return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
+  };
+  auto x_store_of = [&](const GemvCtx& c, int m, int kv, u32x4 v) {
+    const int vec_per_row = ((c.nsuper * 4 * D + 3) / 4) * 4 * CH / 8;
+    if (m >= M || kv >= vec_per_row) return;
+    *reinterpret_cast<u32x4*>(xs + (size_t)m * lds_stride + kv * 8) = permute_x(v);
+  };
+
+  // behind the first phase's requests: the scalar loads' latency runs beside that of the activations
+  auto fetch_late_arguments = [&]() {
+    typedef const __attribute__((address_space(4))) GemvKernArgs* kernarg_ptr_t;
+    kernarg_ptr_t late = (kernarg_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(late));
+    y_ = late->y;
+    ep_ = Epilogue{late->ep.bias, late->ep.residual, late->ep.activation};
+    if constexpr (KSPLIT) {
+      partials_ = late->partials;
+      counters_ = late->counters;
+    }
+  };
+
   // One K phase: stage its activations, stream every tile of the workgroup over it.  The first phase
   // is a copy of its own ahead of the loop over the others: inside a loop the compiler hoists the
   // stream's constants in front of it, i.e. in front of the kernel's first requests.
-  auto run_phase = [&](const int ph) {
-    const int chunk_base = (KSPLIT ? kr : ph) * a.phase_chunks;
-    const int ph_chunks = min(a.phase_chunks, nchunks - chunk_base);
-    const int nsuper = (ph_chunks + 4 * D - 1) / (4 * D);
-    const int per_wave = (nsuper + WAVES - 1) / WAVES;
-    const int ss_begin = wave * per_wave;
-    const int ss_end = min(ss_begin + per_wave, nsuper);
-    const int cnt = max(ss_end - ss_begin, 0);  // super steps per tile for this wavefront
-
+  // b0_loaded: the previous phase's last trip has requested this phase's first item.
+  auto run_phase = [&](const int ph, const GemvCtx& c, const GemvCtx& cn, const bool b0_loaded) {
     // ---- stage this phase's activations (zero padded to a whole k-step) ---------------
     // The first batch of vectors per thread is requested before the first weights and
     // stored after them: global loads retire in order, so the LDS fill does not wait
     // for the much slower first weight loads.
-    GemvBuf<D, SPL> b0, b1;
-    {
-      const int kbase = chunk_base * CH;
-      const int kpad = ((ph_chunks + 3) / 4) * 4 * CH;
-      const int vec_per_row = kpad / 8;
-      auto permute_x = [&](u32x4 v) -> u32x4 {
-        if constexpr (BITS == 4) {
-          u32x4 p;
-          p[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
-          p[1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
-          p[2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
-          p[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
-          return p;
-        } else {
-          return v;
-        }
-      };
-      if (ph > 0) __syncthreads();  // every wavefront is done reading the previous phase
+    const int vec_per_row = ((c.nsuper * 4 * D + 3) / 4) * 4 * CH / 8;
+    if (ph == 0) {
       if constexpr (!ROWS) {
         // one or two rows, or rows longer than the workgroup has threads: a flat index over (row, column),
-        // two vectors per thread ahead of the weights
-        // (every extra request, even one that is masked off, takes its turn in the memory pipeline
-        // ahead of the first weights: the batch-1 start-up is kept as short as it can be)
+        // up to three vectors per thread ahead of the weights -- as many as the activations have, each
+        // further one under a wave-uniform branch.  (Every request, even one that is masked off, takes its
+        // turn in the memory pipeline ahead of the first weights, and a request behind the first weights
+        // comes back after them, a cold trip to HBM later: 4096 x 11008 at batch 1 has 2.7 vectors per
+        // thread and waited 2.3 us for its activations with two ahead, 1.3 us with three.)
         const int total = M * vec_per_row;
-        auto x_load = [&](int idx) -> u32x4 {
-          const int m = idx / vec_per_row, kv = idx - m * vec_per_row;
-          const bool ok = idx < total && kbase + kv * 8 < K;
-          return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
+        auto at = [&](int idx, int& m, int& kv) {
+          m = idx / vec_per_row;
+          kv = idx - m * vec_per_row;
         };
-        auto x_store = [&](int idx, u32x4 v) {
-          if (idx >= total) return;
-          const int m = idx / vec_per_row, kv = idx - m * vec_per_row;
-          *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = permute_x(v);
-        };
-        // (the first two vectors without the division when a row has at least as many vectors as the
-        // workgroup has threads -- K >= 4096: they are in row 0 or 1; the start-up of a 5 us kernel is
+        // (the first vectors without the division when a row has at least as many vectors as the
+        // workgroup has threads -- K >= 4096: they are in rows 0 to 2; the start-up of a 5 us kernel is
         // a few hundred instructions, and a division is forty of them)
-        int m0, kv0, m1, kv1;
-        if (vec_per_row >= NT) {
-          m0 = 0;
-          kv0 = tid;
-          m1 = tid + NT >= vec_per_row ? 1 : 0;
-          kv1 = tid + NT - m1 * vec_per_row;
-        } else {
-          m0 = tid / vec_per_row;
-          kv0 = tid - m0 * vec_per_row;
-          m1 = (tid + NT) / vec_per_row;
-          kv1 = tid + NT - m1 * vec_per_row;
+        const bool wide = vec_per_row >= NT, second = total > NT, third = total > 2 * NT;
+        int m0 = 0, kv0 = tid, m1 = 0, kv1 = 0, m2 = 0, kv2 = 0;
+        if (!wide) at(tid, m0, kv0);
+        const u32x4 x0 = x_load_of(c, m0, kv0);
+        u32x4 x1 = u32x4{0u, 0u, 0u, 0u}, x2 = u32x4{0u, 0u, 0u, 0u};
+        if (second) {
+          if (wide) {
+            m1 = tid + NT >= vec_per_row ? 1 : 0;
+            kv1 = tid + NT - m1 * vec_per_row;
+          } else {
+            at(tid + NT, m1, kv1);
+          }
+          x1 = x_load_of(c, m1, kv1);
         }
-        auto x_load_at = [&](int m, int kv) -> u32x4 {
-          const bool ok = m < M && kbase + kv * 8 < K;
-          return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
-        };
-        auto x_store_at = [&](int m, int kv, u32x4 v) {
-          if (m < M) *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = permute_x(v);
-        };
-        const u32x4 x0 = x_load_at(m0, kv0), x1 = x_load_at(m1, kv1);
+        if (third) {
+          if (wide) {
+            m2 = (tid + 2 * NT >= vec_per_row ? 1 : 0) + (tid + 2 * NT >= 2 * vec_per_row ? 1 : 0);
+            kv2 = tid + 2 * NT - m2 * vec_per_row;
+          } else {
+            at(tid + 2 * NT, m2, kv2);
+          }
+          x2 = x_load_of(c, m2, kv2);
+        }
         __builtin_amdgcn_sched_barrier(0);
-        load_super(b0, 0, ss_begin, chunk_base, ss_end);
+        load_super(b0, c, first_tile(c), 0);
         __builtin_amdgcn_sched_barrier(0);
-        x_store_at(m0, kv0, x0);
-        x_store_at(m1, kv1, x1);
-        for (int idx = tid + 2 * NT; idx < total; idx += 4 * NT) {
-          const u32x4 v0 = x_load(idx), v1 = x_load(idx + NT), v2 = x_load(idx + 2 * NT), v3 = x_load(idx + 3 * NT);
-          x_store(idx, v0);
-          x_store(idx + NT, v1);
-          x_store(idx + 2 * NT, v2);
-          x_store(idx + 3 * NT, v3);
+        fetch_late_arguments();
+        x_store_of(c, m0, kv0, x0);
+        if (second) x_store_of(c, m1, kv1, x1);
+        if (third) x_store_of(c, m2, kv2, x2);
+        for (int idx = tid + 3 * NT; idx < total; idx += 4 * NT) {
+          int ma, ka, mb, kb, mc, kc, md, kd;
+          at(idx, ma, ka);
+          at(idx + NT, mb, kb);
+          at(idx + 2 * NT, mc, kc);
+          at(idx + 3 * NT, md, kd);
+          const u32x4 v0 = x_load_of(c, ma, ka), v1 = x_load_of(c, mb, kb), v2 = x_load_of(c, mc, kc),
+                      v3 = x_load_of(c, md, kd);
+          x_store_of(c, ma, ka, v0);
+          x_store_of(c, mb, kb, v1);
+          x_store_of(c, mc, kc, v2);
+          x_store_of(c, md, kd, v3);
         }
       } else {
         // more rows, and a phase of at most one vector per thread and row (launch_one checks): a thread
@@ -321,73 +386,122 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
         // slower: part of the batch behind the weights -- it returns after them, i.e. after a cold trip
         // to HBM; sixteen in flight; requests under per-vector branches, which the wait-count
         // insertion serialises.)
-        auto x_load = [&](int m, int kv) -> u32x4 {
-          const bool ok = m < M && kv < vec_per_row && kbase + kv * 8 < K;
-          return load_b128(rx, ok ? ((uint32_t)m * (uint32_t)K + (uint32_t)(kbase + kv * 8)) * 2u : kOobOffset);
-        };
-        auto x_store = [&](int m, int kv, u32x4 v) {
-          if (m >= M || kv >= vec_per_row) return;
-          *reinterpret_cast<u32x4*>(xs + (size_t)m * a.lds_stride + kv * 8) = permute_x(v);
-        };
         auto stage = [&](auto rmc) {
           constexpr int RM = decltype(rmc)::value;
           u32x4 xv[RM];
 #pragma unroll
-          for (int r = 0; r < RM; ++r) xv[r] = x_load(r, tid);
+          for (int r = 0; r < RM; ++r) xv[r] = x_load_of(c, r, tid);
           __builtin_amdgcn_sched_barrier(0);
-          load_super(b0, 0, ss_begin, chunk_base, ss_end);
+          load_super(b0, c, first_tile(c), 0);
           __builtin_amdgcn_sched_barrier(0);
+          fetch_late_arguments();
 #pragma unroll
-          for (int r = 0; r < RM; ++r) x_store(r, tid, xv[r]);
+          for (int r = 0; r < RM; ++r) x_store_of(c, r, tid, xv[r]);
           for (int m0 = RM; m0 < M; m0 += RM) {
 #pragma unroll
-            for (int r = 0; r < RM; ++r) xv[r] = x_load(m0 + r, tid);
+            for (int r = 0; r < RM; ++r) xv[r] = x_load_of(c, m0 + r, tid);
 #pragma unroll
-            for (int r = 0; r < RM; ++r) x_store(m0 + r, tid, xv[r]);
+            for (int r = 0; r < RM; ++r) x_store_of(c, m0 + r, tid, xv[r]);
           }
         };
         if (M <= 4) stage(std::integral_constant<int, 4>{});
         else stage(std::integral_constant<int, 8>{});
       }
+    } else {
+      __syncthreads();  // every wavefront is done reading the previous phase
+      auto restage_rows = [&]() {
+        for (int m0 = 0; m0 < M; m0 += 8) {
+          u32x4 xv[8];
+#pragma unroll
+          for (int r = 0; r < 8; ++r) xv[r] = x_load_of(c, m0 + r, tid);
+#pragma unroll
+          for (int r = 0; r < 8; ++r) x_store_of(c, m0 + r, tid, xv[r]);
+        }
+      };
+      if constexpr (XPRE) {
+        if (M <= 8) {
+          // (requested at the start of the previous phase: here long since)
+#pragma unroll
+          for (int r = 0; r < 8; ++r) x_store_of(c, r, tid, xn[r]);
+        } else {
+          restage_rows();
+        }
+      } else if constexpr (ROWS) {
+        restage_rows();
+      } else {
+        const int total = M * vec_per_row;
+        for (int idx = tid; idx < total; idx += 2 * NT) {
+          const int ma = idx / vec_per_row, ka = idx - ma * vec_per_row;
+          const int mb = (idx + NT) / vec_per_row, kb = idx + NT - mb * vec_per_row;
+          const u32x4 v0 = x_load_of(c, ma, ka), v1 = x_load_of(c, mb, kb);
+          x_store_of(c, ma, ka, v0);
+          x_store_of(c, mb, kb, v1);
+        }
+      }
+      if (!b0_loaded) load_super(b0, c, first_tile(c), 0);
     }
     __syncthreads();
+    if constexpr (XPRE) {
+      // the next phase's column of this thread, behind the one item that is in flight
+      if (M <= 8) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) xn[r] = x_load_of(cn, r, tid);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
 
     // ---- the weight stream: a flat software pipeline over (tile, super step) ----------
     // Two items per trip, unconditionally (with an early exit in between, the compiler
     // sinks the prefetch below the compute).  Items past the end load zeros from an
-    // out-of-range offset and are not flushed.
-    const int items = my_tiles * cnt;
-    int ci = 0, cs = 0;  // tile / local super step of the item being consumed
-    int pi = 0, ps = 0;  // ... of the item being prefetched
-    auto advance = [&](int& i, int& s) {
-      if (++s >= cnt) {
-        s = 0;
-        ++i;
-      }
-    };
+    // out-of-range offset and are not computed.
+    const int items = my_tiles * c.cnt;
+    int ci = first_tile(c), cs = 0;  // tile / step of the item being consumed
+    int pi = ci, ps = 0;             // ... of the item being prefetched
     for (int j = 0; j < items; j += 2) {
-      advance(pi, ps);
-      load_super(b1, pi, ss_begin + ps, chunk_base, ss_end);
+      advance(c, pi, ps);
+      load_super(b1, c, pi, ps);
       __builtin_amdgcn_sched_barrier(0);
-      compute_super(b0, ss_begin + cs);
-      if (cs == cnt - 1) flush_tile(ci, ph == 0);
-      advance(ci, cs);
+      compute_super(b0, x_of(c, cs));
+      if (cs == c.cnt - 1) flush_tile(ci, ph == 0);
+      advance(c, ci, cs);
       __builtin_amdgcn_sched_barrier(0);
-      advance(pi, ps);
-      load_super(b0, pi, ss_begin + ps, chunk_base, ss_end);
+      // the item after next, or behind the last trip the first item of the next phase
+      advance(c, pi, ps);
+      if constexpr (PHASES) {
+        const bool wrap = j + 2 >= items;
+        GemvCtx lc;
+        lc.chunk_base = wrap ? cn.chunk_base : c.chunk_base;
+        lc.nsuper = wrap ? cn.nsuper : c.nsuper;
+        lc.start = wrap ? cn.start : c.start;
+        lc.cnt = wrap ? cn.cnt : c.cnt;
+        load_super(b0, lc, wrap ? first_tile(cn) : pi, wrap ? 0 : ps);
+      } else {
+        load_super(b0, c, pi, ps);  // (behind the last trip: no item, zeros)
+      }
       __builtin_amdgcn_sched_barrier(0);
-      compute_super(b1, min(ss_begin + cs, nsuper - 1));
-      if (ci < my_tiles && cs == cnt - 1) flush_tile(ci, ph == 0);
-      advance(ci, cs);
+      if (ci < my_tiles) {
+        compute_super(b1, x_of(c, cs));
+        if (cs == c.cnt - 1) flush_tile(ci, ph == 0);
+      }
+      advance(c, ci, cs);
       __builtin_amdgcn_sched_barrier(0);
     }
-    // a wavefront without work in this phase still owns slots that the epilogue sums
-    if (cnt == 0 && ph == 0)
+    // a wavefront without work in the first phase still owns slots that the epilogue sums
+    if (ph == 0 && c.cnt == 0)
       for (int i = 0; i < my_tiles; ++i) flush_tile(i, true);
+    return items > 0;
   };
-  run_phase(0);
-  if constexpr (!KSPLIT)
-    for (int ph = 1; ph * a.phase_chunks < nchunks; ++ph) run_phase(ph);
+  if constexpr (!PHASES) {
+    run_phase(0, make_ctx(KSPLIT ? kr * phase_chunks_ : 0), dead_ctx, false);
+  } else {
+    GemvCtx c = phase_chunks_ < nchunks ? make_ctx(phase_chunks_) : dead_ctx;
+    bool loaded = run_phase(0, make_ctx(0), c, false);
+    for (int ph = 1; ph * phase_chunks_ < nchunks; ++ph) {
+      const GemvCtx cn = (ph + 1) * phase_chunks_ < nchunks ? make_ctx((ph + 1) * phase_chunks_) : dead_ctx;
+      loaded = run_phase(ph, c, cn, loaded);
+      c = cn;
+    }
+  }
 
   // ---- sum the wavefronts' partial tiles, convert, store -----------------------------
   __syncthreads();
@@ -406,10 +520,10 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
             float up = 0.f;
 #pragma unroll
             for (int w = 0; w < WAVES; ++w) up += slots[((size_t)(i * WAVES + w) * 4 + r) * 64 + l + 1];
-            store_gated(a.y, m, n >> 1, N >> 1, sum, up);
+            store_gated(y_, m, n >> 1, N >> 1, sum, up);
           }
         } else {
-          store_out(a.ep, a.y, m, n, N, sum);
+          store_out(ep_, y_, m, n, N, sum);
         }
       }
     }
@@ -453,7 +567,7 @@ __global__ __launch_bounds__(WAVES * 64) void wq_gemv_kernel(
       float* const part = partials_ + (size_t)(tile0 + i * tstride) * R * 256 + (idx & 255);
       float sum = 0.f;
       for (int q = 0; q < R; ++q) sum += __hip_atomic_load(part + q * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (m < M && n < N) store_out(a.ep, a.y, m, n, N, sum);
+      if (m < M && n < N) store_out(ep_, y_, m, n, N, sum);
     }
     __syncthreads();
     if (tid < my_tiles && last[tid])
@@ -518,43 +632,38 @@ enum { kNotApplicable = 0, kLaunched = 1, kFailed = -1 };
 
 template <int BITS, int WAVES, int D, int SPL, bool TILED = false, bool KSPLIT = false>
 int launch_one(const Problem& p, int group_shift, const Plan& plan, int ksplit = 1, void* workspace = nullptr) {
-  GemvArgs a;
-  a.x = (const half_t*)p.x;
-  a.wq = (const uint32_t*)p.wq;
-  a.scales = (const half_t*)p.scales;
-  a.y = (half_t*)p.y;
-  a.M = (int)p.m;
-  a.N = (int)p.n;
-  a.K = (int)p.k;
-  a.group_shift = group_shift;
-  a.zero_point = p.zero_point;
-  a.lds_stride = plan.lds_stride;
-  a.tiles = (int)((p.n + 15) / 16);
-  a.max_tiles = plan.max_tiles;
-  a.phase_chunks = plan.phase_chunks;
-  a.ep = Epilogue{(const half_t*)p.bias, (const half_t*)p.residual, p.activation};
+  const Epilogue ep{(const half_t*)p.bias, (const half_t*)p.residual, p.activation};
   // workspace of the K split: kSplitMaxTiles arrival counters at a fixed place -- a workspace shared by
   // projections of different shapes keeps them apart from the partial tiles, whose leftovers are not
   // zero -- then [tiles][ksplit][256] float partial tiles
   unsigned int* const counters = static_cast<unsigned int*>(workspace);
   float* const partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kSplitCounterBytes);
-  // two builds of the kernel, by the way the activations are staged: flat index / a column per thread
-  auto go = [&](auto rows) -> int {
-    constexpr bool ROWS = decltype(rows)::value;
+  // the builds of the kernel: by the way the activations are staged (flat index / a column per thread) and by
+  // whether K is walked in several phases
+  auto go = [&](auto rows, auto phases) -> int {
+    constexpr bool ROWS = decltype(rows)::value, PHASES = decltype(phases)::value;
     static std::atomic<bool> lds_ok[kMaxDevices];
-    if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT>, (int)kLdsPerWgMax,
+    if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT, PHASES>, (int)kLdsPerWgMax,
                             lds_ok))
       return kFailed;
-    hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT>), dim3(plan.grid), dim3(WAVES * 64),
-                       plan.lds_bytes, p.stream, a.x, a.wq, a.scales, a.M, a.N, a.K,
-                       a.group_shift | (a.zero_point << 8) | (p.activation == kActGated ? 1 << 16 : 0), a.max_tiles, a.phase_chunks, ksplit, plan.grid, a.y, a.ep, partials,
-                       counters);
+    hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT, PHASES>), dim3(plan.grid), dim3(WAVES * 64),
+                       plan.lds_bytes, p.stream, (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
+                       (int)p.m, (int)p.n, (int)p.k,
+                       group_shift | (p.zero_point << 8) | (p.activation == kActGated ? 1 << 16 : 0),
+                       plan.max_tiles, plan.phase_chunks, ksplit, plan.grid, (half_t*)p.y, ep,
+                       partials, counters);
     return kLaunched;
   };
   constexpr int ch = 128 / BITS;
   const int phase_vectors = (plan.phase_chunks + 3) / 4 * 4 * ch / 8;  // 16-byte vectors per staged row
-  if (p.m <= 2 || phase_vectors > WAVES * 64) return go(std::false_type{});
-  return go(std::true_type{});
+  const bool flat = p.m <= 2 || phase_vectors > WAVES * 64;
+  if constexpr (KSPLIT) {
+    return flat ? go(std::false_type{}, std::false_type{}) : go(std::true_type{}, std::false_type{});
+  } else {
+    if ((int64_t)plan.phase_chunks * ch < p.k)
+      return flat ? go(std::false_type{}, std::true_type{}) : go(std::true_type{}, std::true_type{});
+    return flat ? go(std::false_type{}, std::false_type{}) : go(std::true_type{}, std::false_type{});
+  }
 }
 
 // D chunks per lane need K to be a multiple of 4*D chunks, and the lane's D
