@@ -24,8 +24,9 @@
  * the module; device constants are borrowed (the caller keeps them alive, as the const loader
  * does).  With MI355X_WQ_MODULE_TILE_WEIGHTS the weights are converted once, at init, to the
  * tile-major layout of mi355x_wq_tile_weights and every call runs mi355x_wq_matmul_tiled on the
- * module's own copy (bit-identical results, 4-18 % faster decode).  Init allocates device memory;
- * calls allocate nothing.
+ * module's own copy (bit-identical results, 4-18 % faster decode); a composite with the gated tail
+ * (silu_mul), which is computed on canonical weights only, keeps its canonical constants.  Init allocates
+ * device memory; calls allocate nothing.
  */
 #ifndef MI355X_WQ_MODULE_H_
 #define MI355X_WQ_MODULE_H_
@@ -47,7 +48,10 @@ typedef int (*mi355x_wq_packed_cfunc)(mi355x_tvm_value* args, int* type_codes, i
 
 enum {
   MI355X_WQ_MODULE_TILE_WEIGHTS = 1, /* convert bound weights to the tile-major layout at init (where it is defined) */
-  MI355X_WQ_MODULE_LIBRARY_SCRATCH = 2, /* decode calls may split K on the library's scratch array (mi355x_wq_matmul_static_ws) */
+  MI355X_WQ_MODULE_LIBRARY_SCRATCH = 2, /* decode calls may split K on the library's scratch array (mi355x_wq_matmul_static_ws);
+                                           a split that needs more than the array holds runs unsplit */
+  MI355X_WQ_MODULE_OWN_WORKSPACE = 4,   /* init allocates the K split's workspace for calls of up to
+                                           mi355x_wq_module_set_workspace_rows rows; calls run mi355x_wq_matmul_ws on it */
   MI355X_DL_CPU = 1                  /* kDLCPU */
 };
 
@@ -65,7 +69,18 @@ MI355X_WQ_API int mi355x_wq_module_create(const char* symbol, const mi355x_wq_ca
                                          const char* const* const_names, const int32_t* const_args,
                                          int32_t num_consts, int32_t flags, mi355x_wq_module** out);
 
-/* Frees the module and the device memory it owns (copies of host constants, tile-major weights). */
+/* With MI355X_WQ_MODULE_OWN_WORKSPACE: the row count up to which calls may split K across workgroups.  Init
+ * (which knows N and K from the bound weights) allocates mi355x_wq_workspace_bytes maximised over 1 .. rows and
+ * zeroes it; calls of up to `rows` rows then go through mi355x_wq_matmul_ws on that buffer and still allocate
+ * nothing, calls of more rows run as without a workspace.  The reference's counterpart is the split-K workspace
+ * its generated host code allocates inside every call (python/tvm/contrib/cutlass/gemm_operation.py:294-295,
+ * sized at python/tvm/contrib/cutlass/build.py:335), which an unchanged Relax module gets without asking; here it
+ * is the module that owns it, so that a call can be captured in a HIP graph.  To be set before
+ * __init_<symbol> runs; the count is part of the saved module.  Calls on one module must not overlap in time
+ * (they share the buffer).  Returns 0 or -1. */
+MI355X_WQ_API int mi355x_wq_module_set_workspace_rows(mi355x_wq_module* mod, int32_t rows);
+
+/* Frees the module and the device memory it owns (copies of host constants, tile-major weights, workspace). */
 MI355X_WQ_API void mi355x_wq_module_destroy(mi355x_wq_module* mod);
 
 /* "get_symbol" / "get_const_vars" / "get_json" of the reference module

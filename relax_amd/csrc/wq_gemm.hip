@@ -235,7 +235,24 @@ int launch_gemm(const Problem& p, int variant) {
   if (p.activation != kActGelu) return launch_gemm_any(p, variant, true);
   // gelu: fused by the LDS-staged kernels; behind the direct-weight kernel as a pass of its own -- unless the
   // residual is the output buffer itself, which the first pass would overwrite: then the fused kernels run.
-  if (p.residual == p.y) return launch_gemm_any(p, variant, false);
+  if (p.residual == p.y) {
+    // On tile-major weights only the direct-weight kernel and the register-activation kernel read the layout;
+    // the latter fuses gelu, so it runs the rows here, in blocks of as many rows as it takes (rows of the
+    // output are independent; an in-place residual is read by the thread that then writes the element).
+    if (p.tiled && variant == 0) {
+      for (int64_t m0 = 0; m0 < p.m; m0 += kSkinnyMaxM) {
+        Problem part = p;
+        part.m = std::min<int64_t>(kSkinnyMaxM, p.m - m0);
+        part.x = static_cast<const half_t*>(p.x) + m0 * p.k;
+        part.y = static_cast<half_t*>(p.y) + m0 * p.n;
+        part.residual = part.y;
+        const int rc = launch_skinny(part, 0);
+        if (rc != 0) return rc;
+      }
+      return 0;
+    }
+    return launch_gemm_any(p, variant, false);
+  }
   Problem first = p;
   first.activation = 0;
   first.residual = nullptr;

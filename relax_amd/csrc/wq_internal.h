@@ -78,8 +78,11 @@ namespace wq {
 // mi355x_wq_packed_call; when `wq_tiled` is given, a matmul reads these tile-major copies instead of
 // the canonical tensors in the wq / scales slots (which are still validated and give N, K and group).
 // `library_scratch`: decode matmuls go through mi355x_wq_matmul_static_ws (K split on the library's scratch array).
+// `workspace`: device memory of the caller for the K split (mi355x_wq_matmul_ws); it takes precedence over the
+// library's scratch array.
 int packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes, int num_args,
-                             const void* wq_tiled, const void* scales_tiled, bool library_scratch = false);
+                             const void* wq_tiled, const void* scales_tiled, bool library_scratch = false,
+                             void* workspace = nullptr, int64_t workspace_bytes = 0);
 // Forwards the recorded error to TVM's error slot when the process has one; returns -1.
 int packed_fail();
 }  // namespace wq

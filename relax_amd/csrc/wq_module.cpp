@@ -40,6 +40,9 @@ struct mi355x_wq_module {
   std::vector<BoundConst> bound;
   void* wq_tiled = nullptr;
   void* scales_tiled = nullptr;
+  int32_t workspace_rows = 0;  // MI355X_WQ_MODULE_OWN_WORKSPACE: calls of up to this many rows may split K
+  void* workspace = nullptr;
+  int64_t workspace_bytes = 0;
   int device = -1;
 };
 
@@ -53,9 +56,10 @@ std::string make_json(const mi355x_wq_module& m) {
   int n = snprintf(buf, sizeof(buf),
                    "{\"version\": 1, \"op\": \"%s\", \"bits\": %d, \"group\": %d, \"zero_point\": %d, "
                    "\"num_args\": %d, \"arg_x\": %d, \"arg_wq\": %d, \"arg_scales\": %d, \"arg_out\": %d, "
-                   "\"arg_bias\": %d, \"arg_residual\": %d, \"activation\": %d, \"flags\": %d, \"const_args\": [",
+                   "\"arg_bias\": %d, \"arg_residual\": %d, \"activation\": %d, \"flags\": %d, \"workspace_rows\": %d, "
+                   "\"const_args\": [",
                    op_name(s.op), s.bits, s.group, s.zero_point, s.num_args, s.arg_x, s.arg_wq, s.arg_scales,
-                   s.arg_out, s.arg_bias, s.arg_residual, s.activation, m.flags);
+                   s.arg_out, s.arg_bias, s.arg_residual, s.activation, m.flags, m.workspace_rows);
   std::string out(buf, n);
   for (size_t i = 0; i < m.const_args.size(); ++i) {
     out += (i ? ", " : "") + std::to_string(m.const_args[i]);
@@ -112,7 +116,8 @@ struct JsonReader {
   }
 };
 
-bool parse_json(const std::string& text, mi355x_wq_callspec* spec, std::vector<int32_t>* const_args, int32_t* flags) {
+bool parse_json(const std::string& text, mi355x_wq_callspec* spec, std::vector<int32_t>* const_args, int32_t* flags,
+                int32_t* workspace_rows) {
   JsonReader r{text.data(), text.data() + text.size()};
   memset(spec, 0, sizeof(*spec));
   spec->op = -1;
@@ -150,7 +155,8 @@ bool parse_json(const std::string& text, mi355x_wq_callspec* spec, std::vector<i
                      : key == "arg_x" ? &spec->arg_x : key == "arg_wq" ? &spec->arg_wq
                      : key == "arg_scales" ? &spec->arg_scales : key == "arg_out" ? &spec->arg_out
                      : key == "arg_bias" ? &spec->arg_bias : key == "arg_residual" ? &spec->arg_residual
-                     : key == "activation" ? &spec->activation : key == "flags" ? flags : nullptr;
+                     : key == "activation" ? &spec->activation : key == "flags" ? flags
+                     : key == "workspace_rows" ? workspace_rows : nullptr;
       if (key == "version") version = v;
       else if (field != nullptr) *field = (int32_t)v;
       else return false;
@@ -222,7 +228,7 @@ bool validate(const char* symbol, const mi355x_wq_callspec* spec, const int32_t*
     wq::set_error("module: between 0 and %d constants, got %d", (int)kMaxConsts, num_consts);
     return false;
   }
-  if ((flags & ~(MI355X_WQ_MODULE_TILE_WEIGHTS | MI355X_WQ_MODULE_LIBRARY_SCRATCH)) != 0) {
+  if ((flags & ~(MI355X_WQ_MODULE_TILE_WEIGHTS | MI355X_WQ_MODULE_LIBRARY_SCRATCH | MI355X_WQ_MODULE_OWN_WORKSPACE)) != 0) {
     wq::set_error("module: unknown flags 0x%x", flags);
     return false;
   }
@@ -245,6 +251,10 @@ bool validate(const char* symbol, const mi355x_wq_callspec* spec, const int32_t*
   }
   if ((flags & MI355X_WQ_MODULE_TILE_WEIGHTS) && !(is_matmul && has_wq && has_scales)) {
     wq::set_error("module: tile-major conversion needs a matmul whose wq and scales are both constants");
+    return false;
+  }
+  if ((flags & MI355X_WQ_MODULE_OWN_WORKSPACE) && !(is_matmul && has_wq && has_scales)) {
+    wq::set_error("module: a workspace is sized from N and K at init, which needs a matmul whose wq and scales are both constants");
     return false;
   }
   return true;
@@ -271,7 +281,9 @@ void release_device_memory(mi355x_wq_module* m) {
   m->bound.clear();
   if (m->wq_tiled != nullptr) (void)hipFree(m->wq_tiled);
   if (m->scales_tiled != nullptr) (void)hipFree(m->scales_tiled);
-  m->wq_tiled = m->scales_tiled = nullptr;
+  if (m->workspace != nullptr) (void)hipFree(m->workspace);
+  m->wq_tiled = m->scales_tiled = m->workspace = nullptr;
+  m->workspace_bytes = 0;
 }
 
 bool hip_ok(hipError_t e, const char* what) {
@@ -345,9 +357,9 @@ bool bind_constants(mi355x_wq_module* m, const mi355x_dl_tensor* const* consts, 
     }
   }
   m->device = cur;
-  if (!(m->flags & MI355X_WQ_MODULE_TILE_WEIGHTS)) return true;
+  if (!(m->flags & (MI355X_WQ_MODULE_TILE_WEIGHTS | MI355X_WQ_MODULE_OWN_WORKSPACE))) return true;
 
-  // One-off conversion to the tile-major layout; the canonical tensors stay bound for validation.
+  // N, K and the group of the bound weights (both flags need wq and scales among the constants)
   const BoundConst *bw = nullptr, *bs = nullptr;
   for (int i = 0; i < num_consts; ++i) {
     if (m->const_args[i] == m->spec.arg_wq) bw = &m->bound[i];
@@ -372,27 +384,49 @@ bool bind_constants(mi355x_wq_module* m, const mi355x_dl_tensor* const* consts, 
     return false;
   }
   if (d.n == 0) return true;
+  // One-off conversion to the tile-major layout; the canonical tensors stay bound for validation.
   // The flag is a request, not a promise: where the tile-major layout is not defined for this
-  // (bits, group, K) -- e.g. int4 with K not a multiple of 256 -- the canonical constants stay bound
-  // and calls run on them, exactly as they would without the flag.
-  if (!wq::tiled_layout_defined(d.bits, d.group, d.k)) return true;
-  int64_t wq_bytes = 0, sc_bytes = 0;
-  if (mi355x_wq_tiled_sizes(&d, &wq_bytes, &sc_bytes) != 0) return false;
-  if (!hip_ok(hipMalloc(&m->wq_tiled, wq_bytes), "hipMalloc") || !hip_ok(hipMalloc(&m->scales_tiled, sc_bytes), "hipMalloc"))
-    return false;
-  const void* pw = static_cast<const char*>(tw.data) + tw.byte_offset;
-  const void* ps = static_cast<const char*>(ts.data) + ts.byte_offset;
-  if (mi355x_wq_tile_weights(&d, pw, ps, m->wq_tiled, m->scales_tiled, nullptr) != 0) return false;
-  if (!hip_ok(hipStreamSynchronize(nullptr), "hipStreamSynchronize")) return false;
-  // The module's own canonical copies (of host constants) are not read again: calls take N, K and the
-  // group from the headers and the data from the tile-major buffers, which have at least as many rows.
-  for (int i = 0; i < num_consts; ++i) {
-    BoundConst& b = m->bound[i];
-    const bool is_wq = m->const_args[i] == m->spec.arg_wq, is_scales = m->const_args[i] == m->spec.arg_scales;
-    if (b.owned == nullptr || !(is_wq || is_scales)) continue;
-    (void)hipFree(b.owned);
-    b.owned = nullptr;
-    b.tensor.data = is_wq ? m->wq_tiled : m->scales_tiled;
+  // (bits, group, K) -- e.g. int4 with K not a multiple of 256 -- or for this composite -- the gated tail is
+  // computed on canonical weights only -- the canonical constants stay bound and calls run on them, exactly as
+  // they would without the flag.
+  if ((m->flags & MI355X_WQ_MODULE_TILE_WEIGHTS) && m->spec.activation != MI355X_WQ_ACT_SILU_MUL &&
+      wq::tiled_layout_defined(d.bits, d.group, d.k)) {
+    int64_t wq_bytes = 0, sc_bytes = 0;
+    if (mi355x_wq_tiled_sizes(&d, &wq_bytes, &sc_bytes) != 0) return false;
+    if (!hip_ok(hipMalloc(&m->wq_tiled, wq_bytes), "hipMalloc") || !hip_ok(hipMalloc(&m->scales_tiled, sc_bytes), "hipMalloc"))
+      return false;
+    const void* pw = static_cast<const char*>(tw.data) + tw.byte_offset;
+    const void* ps = static_cast<const char*>(ts.data) + ts.byte_offset;
+    if (mi355x_wq_tile_weights(&d, pw, ps, m->wq_tiled, m->scales_tiled, nullptr) != 0) return false;
+    if (!hip_ok(hipStreamSynchronize(nullptr), "hipStreamSynchronize")) return false;
+    // The module's own canonical copies (of host constants) are not read again: calls take N, K and the
+    // group from the headers and the data from the tile-major buffers, which have at least as many rows.
+    for (int i = 0; i < num_consts; ++i) {
+      BoundConst& b = m->bound[i];
+      const bool is_wq = m->const_args[i] == m->spec.arg_wq, is_scales = m->const_args[i] == m->spec.arg_scales;
+      if (b.owned == nullptr || !(is_wq || is_scales)) continue;
+      (void)hipFree(b.owned);
+      b.owned = nullptr;
+      b.tensor.data = is_wq ? m->wq_tiled : m->scales_tiled;
+    }
+  }
+  // The K split's workspace, where this projection has a use for one at any row count up to workspace_rows:
+  // allocated and zeroed here, once, so that calls allocate nothing (what the reference's generated host code
+  // does per call, python/tvm/contrib/cutlass/gemm_operation.py:294-295).
+  if ((m->flags & MI355X_WQ_MODULE_OWN_WORKSPACE) && m->workspace_rows > 0) {
+    const int tiled = m->wq_tiled != nullptr ? 1 : 0;
+    int64_t need = 0;
+    for (int64_t rows = 1; rows <= m->workspace_rows; ++rows) {
+      const int64_t b = mi355x_wq_workspace_bytes(&d, rows, tiled);
+      if (b < 0) return false;
+      if (b > need) need = b;
+    }
+    if (need > 0) {
+      if (!hip_ok(hipMalloc(&m->workspace, need), "hipMalloc")) return false;
+      if (!hip_ok(hipMemset(m->workspace, 0, need), "hipMemset") || !hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize"))
+        return false;
+      m->workspace_bytes = need;
+    }
   }
   return true;
 }
@@ -533,8 +567,21 @@ int mi355x_wq_module_call(mi355x_wq_module* mod, mi355x_tvm_value* args, int* ty
       ++next;
     }
   }
+  // (a call of more rows than the workspace was sized for runs as the plain call)
+  int64_t rows = 0;
+  if (mod->workspace != nullptr && mod->spec.op == 0) {
+    const int tc = codes[mod->spec.arg_x];
+    const mi355x_dl_tensor* tx = (tc == MI355X_TVM_DLTENSOR_HANDLE || tc == MI355X_TVM_NDARRAY_HANDLE)
+                                     ? static_cast<const mi355x_dl_tensor*>(full[mod->spec.arg_x].v_handle) : nullptr;
+    if (tx != nullptr && tx->shape != nullptr && tx->ndim >= 1 && tx->ndim <= 8) {
+      rows = 1;
+      for (int d = 0; d + 1 < tx->ndim; ++d) rows = tx->shape[d] > 0 && rows <= mod->workspace_rows ? rows * tx->shape[d] : rows;
+    }
+  }
+  const bool use_ws = mod->workspace != nullptr && rows >= 1 && rows <= mod->workspace_rows;
   return wq::packed_call_with_weights(&mod->spec, full, codes, total, mod->wq_tiled, mod->scales_tiled,
-                                      (mod->flags & MI355X_WQ_MODULE_LIBRARY_SCRATCH) != 0);
+                                      (mod->flags & MI355X_WQ_MODULE_LIBRARY_SCRATCH) != 0,
+                                      use_ws ? mod->workspace : nullptr, use_ws ? mod->workspace_bytes : 0);
 }
 
 int64_t mi355x_wq_module_save_to_binary(const mi355x_wq_module* mod, void* buffer, int64_t capacity) {
@@ -595,8 +642,8 @@ int mi355x_wq_module_create_from_json(const char* symbol, const char* json, cons
   *out = nullptr;
   mi355x_wq_callspec spec;
   std::vector<int32_t> const_args;
-  int32_t flags = 0;
-  if (!parse_json(json, &spec, &const_args, &flags)) {
+  int32_t flags = 0, workspace_rows = 0;
+  if (!parse_json(json, &spec, &const_args, &flags, &workspace_rows)) {
     wq::set_error("module load: the call description is not one this library wrote: %.200s", json);
     return -1;
   }
@@ -604,7 +651,36 @@ int mi355x_wq_module_create_from_json(const char* symbol, const char* json, cons
     wq::set_error("module load: %d constant names for %d constant slots", num_consts, (int)const_args.size());
     return -1;
   }
-  return mi355x_wq_module_create(symbol, &spec, const_names, const_args.data(), num_consts, flags, out);
+  if (mi355x_wq_module_create(symbol, &spec, const_names, const_args.data(), num_consts, flags, out) != 0) return -1;
+  if (workspace_rows != 0 && mi355x_wq_module_set_workspace_rows(*out, workspace_rows) != 0) {
+    mi355x_wq_module_destroy(*out);
+    *out = nullptr;
+    return -1;
+  }
+  return 0;
+}
+
+int mi355x_wq_module_set_workspace_rows(mi355x_wq_module* mod, int32_t rows) {
+  if (mod == nullptr) {
+    wq::set_error("module is NULL");
+    return -1;
+  }
+  std::lock_guard<std::mutex> guard(mod->mutex);
+  if (!(mod->flags & MI355X_WQ_MODULE_OWN_WORKSPACE)) {
+    wq::set_error("module: workspace rows go with MI355X_WQ_MODULE_OWN_WORKSPACE");
+    return -1;
+  }
+  if (rows < 0 || rows > (1 << 20)) {
+    wq::set_error("module: workspace rows must be between 0 and %d, got %d", 1 << 20, rows);
+    return -1;
+  }
+  if (mod->initialized && !mod->const_names.empty()) {
+    wq::set_error("module: the workspace is sized at init; set the rows before __init_%s runs", mod->symbol.c_str());
+    return -1;
+  }
+  mod->workspace_rows = rows;
+  mod->json = make_json(*mod);
+  return 0;
 }
 
 }  // extern "C"

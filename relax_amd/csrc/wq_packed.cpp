@@ -34,9 +34,12 @@ constexpr Dtype kU8{1, 8, "uint8"};
 
 // Checks one tensor argument; on success stores the (byte_offset adjusted) pointer.
 // `vector_ok`: the tensor may be 1-d [N] (reported as rows = 1, cols = N).
+// `fold_leading`: any rank from 1 on, compact row-major; the extents before the last are folded into the rows
+// (x[B, S, K] is B * S rows of K: relax.matmul broadcasts the leading extents of x over a 2-d weight,
+// src/relax/op/tensor/linear_algebra.cc:46-114).
 bool take_tensor(mi355x_tvm_value* args, int* type_codes, int idx, const char* role, Dtype want,
                  int device_id_expected, const mi355x_dl_tensor** out, void** ptr,
-                 bool vector_ok = false, int64_t* rows = nullptr, int64_t* cols = nullptr) {
+                 bool vector_ok = false, int64_t* rows = nullptr, int64_t* cols = nullptr, bool fold_leading = false) {
   const int tc = type_codes[idx];
   if (tc != MI355X_TVM_DLTENSOR_HANDLE && tc != MI355X_TVM_NDARRAY_HANDLE) {
     wq::set_error("argument %d (%s): expected a tensor (type code 7 or 13), got type code %d", idx,
@@ -69,6 +72,47 @@ bool take_tensor(mi355x_tvm_value* args, int* type_codes, int idx, const char* r
     *ptr = static_cast<char*>(t->data) + t->byte_offset;
     if (rows != nullptr) *rows = 1;
     if (cols != nullptr) *cols = t->shape[0];
+    return true;
+  }
+  if (fold_leading && t->shape != nullptr && t->ndim >= 1 && t->ndim != 2) {
+    if (t->dtype.code != want.code || t->dtype.bits != want.bits || t->dtype.lanes != 1) {
+      wq::set_error("argument %d (%s): expected dtype %s, got code=%d bits=%d lanes=%d", idx, role,
+                    want.name, t->dtype.code, t->dtype.bits, t->dtype.lanes);
+      return false;
+    }
+    if (t->device.device_type != MI355X_DL_ROCM ||
+        (device_id_expected >= 0 && t->device.device_id != device_id_expected)) {
+      wq::set_error("argument %d (%s): expected a ROCm tensor on device %d, got device type %d id %d",
+                    idx, role, device_id_expected, t->device.device_type, t->device.device_id);
+      return false;
+    }
+    if (t->ndim > 8) {
+      wq::set_error("argument %d (%s): at most 8 dimensions, got %d", idx, role, t->ndim);
+      return false;
+    }
+    int64_t lead = 1, expect = 1;
+    bool compact = true;
+    for (int d = t->ndim - 1; d >= 0; --d) {
+      if (t->shape[d] < 0 || (d < t->ndim - 1 && t->shape[d] != 0 && lead > (int64_t)0x7FFFFFFF / t->shape[d])) {
+        wq::set_error("argument %d (%s): negative or oversized extent", idx, role);
+        return false;
+      }
+      if (t->strides != nullptr && t->shape[d] > 1 && t->strides[d] != expect) compact = false;
+      expect *= t->shape[d];
+      if (d < t->ndim - 1) lead *= t->shape[d];
+    }
+    if (!compact) {
+      wq::set_error("argument %d (%s): a %d-d tensor must be compact row-major", idx, role, t->ndim);
+      return false;
+    }
+    if (t->data == nullptr && expect != 0) {
+      wq::set_error("argument %d (%s): NULL data pointer", idx, role);
+      return false;
+    }
+    *out = t;
+    *ptr = static_cast<char*>(t->data) + t->byte_offset;
+    if (rows != nullptr) *rows = lead;
+    if (cols != nullptr) *cols = t->shape[t->ndim - 1];
     return true;
   }
   if (t->ndim != 2 || t->shape == nullptr) {
@@ -138,7 +182,8 @@ int mi355x_wq_packed_call_scratch(const mi355x_wq_callspec* spec, mi355x_tvm_val
 int wq::packed_fail() { return fail(); }
 
 int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_value* args, int* type_codes,
-                                 int num_args, const void* wq_tiled, const void* scales_tiled, bool library_scratch) {
+                                 int num_args, const void* wq_tiled, const void* scales_tiled, bool library_scratch,
+                                 void* workspace, int64_t workspace_bytes) {
   if (spec == nullptr) {
     wq::set_error("call spec is NULL");
     return fail();
@@ -184,9 +229,19 @@ int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_valu
   if (!take_tensor(args, type_codes, spec->arg_wq, "wq", kU32, -1, &tw, &pw)) return fail();
   const int dev = tw->device.device_id;
   if (!take_tensor(args, type_codes, spec->arg_scales, "scales", kF16, dev, &ts, &ps)) return fail();
-  if (!take_tensor(args, type_codes, spec->arg_out, is_matmul ? "y" : "wd", kF16, dev, &to, &po))
+  int64_t out_rows = 0, out_cols = 0, x_rows = 0, x_cols = 0;
+  if (!take_tensor(args, type_codes, spec->arg_out, is_matmul ? "y" : "wd", kF16, dev, &to, &po, false, &out_rows, &out_cols,
+                   is_matmul))
     return fail();
-  if (is_matmul && !take_tensor(args, type_codes, spec->arg_x, "x", kF16, dev, &tx, &px)) return fail();
+  if (is_matmul && !take_tensor(args, type_codes, spec->arg_x, "x", kF16, dev, &tx, &px, false, &x_rows, &x_cols, true))
+    return fail();
+  // the output (and the residual) repeat the leading extents of x
+  auto same_leading = [](const mi355x_dl_tensor* a, const mi355x_dl_tensor* b) {
+    if (a->ndim != b->ndim) return false;
+    for (int d = 0; d + 1 < a->ndim; ++d)
+      if (a->shape[d] != b->shape[d]) return false;
+    return true;
+  };
 
   const int per_word = 32 / (spec->bits == 8 ? 8 : 4);
   mi355x_wq_desc d;
@@ -217,9 +272,9 @@ int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_valu
 
   int64_t m = 0;
   if (is_matmul) {
-    m = tx->shape[0];
-    if (tx->shape[1] != d.k) {
-      wq::set_error("x has %lld columns but the weights have K=%lld", (long long)tx->shape[1],
+    m = x_rows;
+    if (x_cols != d.k) {
+      wq::set_error("x has %lld columns but the weights have K=%lld", (long long)x_cols,
                     (long long)d.k);
       return fail();
     }
@@ -229,10 +284,11 @@ int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_valu
       wq::set_error("the gated tail (silu_mul) needs an even N, got %lld", (long long)d.n);
       return fail();
     }
-    const int64_t out_cols = gated_out ? d.n / 2 : d.n;
-    if (to->shape[0] != m || to->shape[1] != out_cols) {
-      wq::set_error("y has shape (%lld, %lld), expected (%lld, %lld)", (long long)to->shape[0],
-                    (long long)to->shape[1], (long long)m, (long long)out_cols);
+    const int64_t want_cols = gated_out ? d.n / 2 : d.n;
+    if (out_rows != m || out_cols != want_cols || !same_leading(to, tx)) {
+      wq::set_error("y has shape (%lld, %lld), expected (%lld, %lld)%s", (long long)out_rows,
+                    (long long)out_cols, (long long)m, (long long)want_cols,
+                    same_leading(to, tx) ? "" : " with the leading extents of x");
       return fail();
     }
   } else if (to->shape[0] != d.n || to->shape[1] != d.k) {
@@ -247,7 +303,7 @@ int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_valu
     const mi355x_dl_tensor* tb = nullptr;
     void* pb = nullptr;
     int64_t br = 0, bc = 0;
-    if (!take_tensor(args, type_codes, spec->arg_bias, "bias", kF16, dev, &tb, &pb, true, &br, &bc))
+    if (!take_tensor(args, type_codes, spec->arg_bias, "bias", kF16, dev, &tb, &pb, true, &br, &bc, true))
       return fail();
     if (br != 1 || bc != d.n) {
       wq::set_error("bias has shape (%lld, %lld), expected (%lld) or (1, %lld)", (long long)br,
@@ -259,10 +315,12 @@ int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_valu
   if (has_res) {
     const mi355x_dl_tensor* tr = nullptr;
     void* pr = nullptr;
-    if (!take_tensor(args, type_codes, spec->arg_residual, "residual", kF16, dev, &tr, &pr)) return fail();
-    if (tr->shape[0] != m || tr->shape[1] != d.n) {
-      wq::set_error("residual has shape (%lld, %lld), expected (%lld, %lld)", (long long)tr->shape[0],
-                    (long long)tr->shape[1], (long long)m, (long long)d.n);
+    int64_t rr = 0, rc = 0;
+    if (!take_tensor(args, type_codes, spec->arg_residual, "residual", kF16, dev, &tr, &pr, false, &rr, &rc, true))
+      return fail();
+    if (rr != m || rc != d.n || !same_leading(tr, tx)) {
+      wq::set_error("residual has shape (%lld, %lld), expected (%lld, %lld)%s", (long long)rr,
+                    (long long)rc, (long long)m, (long long)d.n, same_leading(tr, tx) ? "" : " with the leading extents of x");
       return fail();
     }
     ep.residual = pr;
@@ -280,11 +338,20 @@ int wq::packed_call_with_weights(const mi355x_wq_callspec* spec, mi355x_tvm_valu
     wq::set_error("tensors live on ROCm device %d but the current HIP device is %d", dev, cur);
     return fail();
   }
-  if (library_scratch && is_matmul) {
-    // decode calls may split K across workgroups on the library's own scratch array (no allocation)
+  if (workspace != nullptr && is_matmul) {
+    // a workspace the caller (the subgraph module) owns: the K split of decode and prefill calls where it pays;
+    // anything else, and a workspace that is too small, runs as the plain call
     const bool tiled = wq_tiled != nullptr;
-    return mi355x_wq_matmul_static_ws(&d, px, tiled ? wq_tiled : pw, tiled ? scales_tiled : ps, &ep, po, m, g_stream,
-                                      tiled ? 1 : 0) == 0 ? 0 : fail();
+    return mi355x_wq_matmul_ws(&d, px, tiled ? wq_tiled : pw, tiled ? scales_tiled : ps, &ep, po, m, g_stream,
+                               tiled ? 1 : 0, workspace, workspace_bytes) == 0 ? 0 : fail();
+  }
+  if (library_scratch && is_matmul) {
+    // decode calls may split K across workgroups on the library's own scratch array (no allocation); a split
+    // that would need more than the array holds runs unsplit -- the option is a speed-up, never a reason to fail
+    const bool tiled = wq_tiled != nullptr;
+    if (mi355x_wq_workspace_bytes(&d, m, tiled ? 1 : 0) <= mi355x_wq_static_ws_bytes())
+      return mi355x_wq_matmul_static_ws(&d, px, tiled ? wq_tiled : pw, tiled ? scales_tiled : ps, &ep, po, m, g_stream,
+                                        tiled ? 1 : 0) == 0 ? 0 : fail();
   }
   if (wq_tiled != nullptr && is_matmul)
     return mi355x_wq_matmul_tiled(&d, px, wq_tiled, scales_tiled, &ep, po, m, g_stream) == 0 ? 0 : fail();

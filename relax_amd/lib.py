@@ -32,7 +32,7 @@ EXPORTED_SYMBOLS = (
     "mi355x_wq_module_num_consts", "mi355x_wq_module_const_name", "mi355x_wq_module_json",
     "mi355x_wq_module_initialized", "mi355x_wq_module_get_function", "mi355x_wq_module_init",
     "mi355x_wq_module_call", "mi355x_wq_module_save_to_binary", "mi355x_wq_module_load_from_binary",
-    "mi355x_wq_module_create_from_json",
+    "mi355x_wq_module_create_from_json", "mi355x_wq_module_set_workspace_rows",
 )
 PACKED_ENTRIES = tuple(s for s in EXPORTED_SYMBOLS if s.startswith(("mi355x_q4f16_", "mi355x_q8f16_")))
 
@@ -123,6 +123,7 @@ def load() -> C.CDLL:
     L.mi355x_wq_module_save_to_binary.restype = i64
     L.mi355x_wq_module_load_from_binary.argtypes = [vp, i64, C.POINTER(i64), C.POINTER(vp)]
     L.mi355x_wq_module_create_from_json.argtypes = [C.c_char_p, C.c_char_p, C.POINTER(C.c_char_p), i32, C.POINTER(vp)]
+    L.mi355x_wq_module_set_workspace_rows.argtypes = [vp, i32]
     _lib = L
     return L
 

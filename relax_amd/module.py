@@ -30,6 +30,7 @@ from .vm_harness import (K_TVM_NDARRAY_HANDLE, K_TVM_NULLPTR, CallSpec, PackedEr
 
 TILE_WEIGHTS = 1
 LIBRARY_SCRATCH = 2
+OWN_WORKSPACE = 4
 ND_ARRAY_MAGIC = 0xDD5E40F096B4A13F  # kTVMNDArrayMagic, include/tvm/runtime/ndarray.h:447
 _PACKED_CFUNC = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_void_p, C.c_void_p)
 
@@ -138,14 +139,20 @@ class SubgraphModule:
         self._keep = []  # device constants borrowed by the module must outlive it
 
     @classmethod
-    def create(cls, symbol: str, spec: CallSpec, const_names=(), const_args=(), flags: int = 0) -> "SubgraphModule":
+    def create(cls, symbol: str, spec: CallSpec, const_names=(), const_args=(), flags: int = 0,
+               workspace_rows: int = 0) -> "SubgraphModule":
+        """`workspace_rows` (with OWN_WORKSPACE among the flags): init allocates the K split's workspace for calls
+        of up to that many rows."""
         L = _lib.load()
         n = len(const_names)
         names = (C.c_char_p * max(n, 1))(*[s.encode() for s in const_names])
         slots = (C.c_int32 * max(n, 1))(*const_args)
         out = C.c_void_p()
         _lib.check(L.mi355x_wq_module_create(symbol.encode(), C.addressof(spec), names, slots, n, flags, C.byref(out)))
-        return cls(out.value)
+        mod = cls(out.value)
+        if workspace_rows:
+            _lib.check(L.mi355x_wq_module_set_workspace_rows(mod._h, workspace_rows))
+        return mod
 
     @classmethod
     def load_from_binary(cls, data: bytes, pos: int = 0):

@@ -18,16 +18,19 @@ activation)` describes for its CUTLASS backend (python/tvm/relax/dpl/pattern.py:
 or by the gated tail of a Llama MLP, whose gate and up projections share one weight matrix (gate rows,
 then as many up rows):
 
-    sp  = R.split(y, 2, axis=-1)
-    out = R.multiply(R.nn.silu(sp[0]), sp[1])      # [M, N/2]
+    sp  = R.split(y, 2, axis=-1)                   # the last axis, by either of its two indices
+    out = R.multiply(R.nn.silu(sp[0]), sp[1])      # [M, N/2]; multiply is matched in both operand orders
+
+x may carry leading extents, `x[B, S, K]` against the 2-d weight (src/relax/op/tensor/linear_algebra.cc:46-114):
+the kernels see M = B * S rows.
 
 `matmul(x, permute_dims(W))` is what `relax.op.linear` expands to
 (python/tvm/relax/op/linear_algebra.py:54-90).  The pattern name's prefix before the
 first "." becomes the `Codegen` attribute, i.e. the backend name
 (src/relax/transform/fuse_ops.cc:1039-1044).
 
-Verified by reading, not by running: TVM cannot be built or imported in this build's
-environment.
+TVM cannot be built or imported in this build's environment; the table is executed against a stand-in
+`tvm.relax.dpl` whose matcher follows src/relax/ir/dataflow_matcher.cc (tests/support/fake_dpl.py).
 """
 from __future__ import annotations
 
@@ -43,6 +46,7 @@ DECODE_FUNCS = {
 def patterns():
     """[(name, DFPattern)] for FuseOpsByPattern(patterns, annotate_codegen=True)."""
     from tvm.relax.dpl import is_call_tir, is_op, is_tuple_get_item, wildcard  # python/tvm/relax/dpl/pattern.py:678-837
+    from tvm.tir import IntImm
 
     def core(fn_name):
         # Only the float32-accumulating form is taken: with out_dtype "" or "float16" the CPU path
@@ -62,9 +66,19 @@ def patterns():
         add1 = lambda: is_op("relax.add")(core(fn_name), wildcard())  # noqa: E731
         relu = lambda: is_op("relax.nn.relu")(add1())                 # noqa: E731
         gelu = lambda: is_op("relax.nn.gelu")(add1())                 # noqa: E731
-        halves = lambda: is_op("relax.split")(core(fn_name)).has_attr({"indices_or_sections": 2})  # noqa: E731
-        gated = is_op("relax.multiply")(is_op("relax.nn.silu")(is_tuple_get_item(halves(), 0)),
-                                        is_tuple_get_item(halves(), 1))
+        # The section count of relax.op.split is an int64 IntImm (python/tvm/relax/op/manipulate.py:238-240) and an
+        # object-valued attribute is compared structurally, dtype included (src/relax/ir/dataflow_matcher.cc:139-147):
+        # a Python 2 would arrive as an int32 IntImm and never match.  The axis is an `int` field, compared by value
+        # (:110-114) and stored as written: the last axis of a 2-d or 3-d output is -1, 1 or 2 -- an attribute
+        # pattern holds one value per key, hence the alternatives.  (A 3-d output split along axis 1 would match
+        # too; the hook refuses it.)  One pattern object for the split: both halves must come from the same one.
+        split = is_op("relax.split")(core(fn_name))
+        two = IntImm("int64", 2)
+        halves = (split.has_attr({"indices_or_sections": two, "axis": -1})
+                  | split.has_attr({"indices_or_sections": two, "axis": 1})
+                  | split.has_attr({"indices_or_sections": two, "axis": 2}))
+        gated = is_op("relax.multiply")(is_op("relax.nn.silu")(is_tuple_get_item(halves, 0)),
+                                        is_tuple_get_item(halves, 1))
         table.append((base + "_silu_mul", gated))
         table.append((base + "_add_relu_add", is_op("relax.add")(relu(), wildcard())))
         table.append((base + "_add_add", is_op("relax.add")(add1(), wildcard())))

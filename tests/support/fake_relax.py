@@ -16,10 +16,34 @@ class StructInfo:
 
 
 class Attrs:
-    """Call attributes with attribute access, like an Attrs node (MatmulAttrs.out_dtype, ...)."""
+    """Call attributes with attribute access, like an Attrs node (MatmulAttrs.out_dtype, ...).  The Python type
+    of a field stands for the C++ type of the reference's field, which decides how a pattern's attribute test
+    compares it (src/relax/ir/dataflow_matcher.cc:108-150): `int` for an int field (SplitAttrs.axis), `DataType`
+    for a DataType field (MatmulAttrs.out_dtype, AstypeAttrs.dtype), `IntImm` / list for an object-valued field
+    (SplitAttrs.indices_or_sections, PermuteDimsAttrs.axes)."""
 
     def __init__(self, **fields):
         self.__dict__.update(fields)
+
+
+class IntImm:
+    """tvm.tir.IntImm: a value with a dtype; structural equality tells int32 from int64."""
+
+    def __init__(self, dtype, value):
+        self.dtype, self.value = str(dtype), int(value)
+
+    def __int__(self):
+        return self.value
+
+    def __index__(self):
+        return self.value
+
+    def __repr__(self):
+        return f"IntImm({self.dtype!r}, {self.value})"
+
+
+class DataType(str):
+    """A DataType attribute field: reads back as its string in Python."""
 
 
 class Var(Expr):
@@ -110,7 +134,7 @@ class Function(Expr):
 def as_module():
     """A module object usable as `tvm` with a `relax` attribute."""
     relax = types.ModuleType("tvm.relax")
-    for cls in (Var, Call, Function, Tuple, GlobalVar, SeqExpr, BindingBlock, DataflowBlock, VarBinding, Constant, ExternFunc, TupleGetItem):
+    for cls in (Var, Call, Function, Tuple, GlobalVar, SeqExpr, BindingBlock, DataflowBlock, VarBinding, Constant, ExternFunc, TupleGetItem, Op):
         setattr(relax, cls.__name__, cls)
     tvm = types.ModuleType("tvm")
     tvm.relax = relax
@@ -131,32 +155,37 @@ def quantized_linear(decode="decode_q4f16", m=4, n=48, k=128, tail=(), outer_ord
     wq = Constant([n, k // per], dtype="uint32") if "wq" in bound else Var("wq", [n, k // per], "uint32")
     s = Constant([n, k // group], dtype="float16") if "scales" in bound else Var("s", [n, k // group], "float16")
     x = Var("x", x_shape or [m, k], x_dtype)
+    lead = list(x_shape[:-1]) if x_shape else [m]  # matmul broadcasts the leading extents of x over the 2-d weight
     params = [p for p in (wq, s, x) if isinstance(p, Var)]
     binds = []
     wd = Var("wd", [n, k], "float16")
     binds.append(VarBinding(wd, Call(Op("relax.call_tir"), [GlobalVar(decode), Tuple([wq, s])])))
     wt = Var("wt", [k, n], "float16")
     binds.append(VarBinding(wt, Call(Op("relax.permute_dims"), [wd], Attrs(axes=axes))))
-    y32 = Var("y32", [m, n], out_dtype or x_dtype)
-    binds.append(VarBinding(y32, Call(Op("relax.matmul"), [x, wt], Attrs(out_dtype=out_dtype))))
-    cur = Var("y", [m, n], astype_dtype)
-    binds.append(VarBinding(cur, Call(Op("relax.astype"), [y32], Attrs(dtype=astype_dtype))))
+    y32 = Var("y32", lead + [n], out_dtype or x_dtype)
+    binds.append(VarBinding(y32, Call(Op("relax.matmul"), [x, wt], Attrs(out_dtype=DataType(out_dtype)))))
+    cur = Var("y", lead + [n], astype_dtype)
+    binds.append(VarBinding(cur, Call(Op("relax.astype"), [y32], Attrs(dtype=DataType(astype_dtype)))))
     for i, step in enumerate(tail):
-        nxt = Var(f"t{i}", [m, n], "float16")
+        nxt = Var(f"t{i}", lead + [n], "float16")
         if step[0] == "silu_mul":
             # sp = split(y, 2, axis); out = multiply(nn.silu(sp[0]), sp[1]); step = ("silu_mul", sections, axis, swapped)
             sections = step[1] if len(step) > 1 else 2
             axis = step[2] if len(step) > 2 else -1
             swapped = len(step) > 3 and step[3]
             sp = Var("sp")
-            binds.append(VarBinding(sp, Call(Op("relax.split"), [cur], Attrs(indices_or_sections=sections, axis=axis))))
-            h0, h1 = Var("gate", [m, n // 2], "float16"), Var("up", [m, n // 2], "float16")
+            # (relax.op.split stores a section count as an int64 IntImm and the axis as given,
+            # python/tvm/relax/op/manipulate.py:238-240, src/relax/op/tensor/manipulate.cc:635-660)
+            binds.append(VarBinding(sp, Call(Op("relax.split"), [cur],
+                                             Attrs(indices_or_sections=IntImm("int64", sections), axis=int(axis)))))
+            h0, h1 = Var("gate", lead + [n // 2], "float16"), Var("up", lead + [n // 2], "float16")
             binds.append(VarBinding(h0, TupleGetItem(sp, 1 if swapped else 0)))
             binds.append(VarBinding(h1, TupleGetItem(sp, 0 if swapped else 1)))
-            act = Var("act", [m, n // 2], "float16")
+            act = Var("act", lead + [n // 2], "float16")
             binds.append(VarBinding(act, Call(Op("relax.nn.silu"), [h0])))
-            nxt = Var(f"t{i}", [m, n // 2], "float16")
-            binds.append(VarBinding(nxt, Call(Op("relax.multiply"), [act, h1])))
+            nxt = Var(f"t{i}", lead + [n // 2], "float16")
+            flipped = len(step) > 4 and step[4]  # multiply(up, silu(gate)): the same product
+            binds.append(VarBinding(nxt, Call(Op("relax.multiply"), [h1, act] if flipped else [act, h1])))
             cur = nxt
             continue
         if step[0] == "add":
@@ -180,7 +209,7 @@ def quantized_linear(decode="decode_q4f16", m=4, n=48, k=128, tail=(), outer_ord
     order = outer_order or list(range(len(outer)))
     outer_params = [outer[i] for i in order]
     local = Var("gv1" if golden_names else "local_func")
-    gv = Var("gv11" if golden_names else "gv", [m, n], "float16")
+    gv = Var("gv11" if golden_names else "gv", list(cur.struct_info.shape), "float16")
     body = SeqExpr([BindingBlock([VarBinding(local, composite), VarBinding(gv, Call(local, outer))])], gv)
     return Function(outer_params, body, {"Codegen": "mi355x", "global_symbol": symbol})
 

@@ -27,7 +27,7 @@ def declared_symbols():
 def test_library_exports_every_declared_symbol():
     L = lib.load()
     names = declared_symbols()
-    assert len(names) == 57 and set(names) == set(lib.EXPORTED_SYMBOLS)
+    assert len(names) == 58 and set(names) == set(lib.EXPORTED_SYMBOLS)
     for n in names:
         assert hasattr(L, n), n
     assert L.mi355x_wq_version() >= 100
@@ -237,9 +237,17 @@ def test_packed_dtype_shape_and_stride_checks():
         vm_harness.call_packed("mi355x_q4f16_matmul", _args(x, wq, s, y[:, :8].contiguous(), **dev))
     with pytest.raises(vm_harness.PackedError, match="scales has 8 rows but wq has 16"):
         vm_harness.call_packed("mi355x_q4f16_matmul", _args(x, wq, s[:8].contiguous(), y, **dev))
-    with pytest.raises(vm_harness.PackedError, match="expected a 2-d tensor"):
+    # a 1-d x is one row of its length (leading extents fold into the rows): 128 columns against K = 64
+    with pytest.raises(vm_harness.PackedError, match="x has 128 columns but the weights have K=64"):
         vm_harness.call_packed("mi355x_q4f16_matmul", _args(x.reshape(-1), wq, s, y, **dev)[:1] +
                                _args(x, wq, s, y, **dev)[1:])
+    # the weights stay 2-d
+    with pytest.raises(vm_harness.PackedError, match=r"argument 1 \(wq\): expected a 2-d tensor"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", _args(x, wq, s, y, **dev)[:1] +
+                               [vm_harness.TensorArg(wq.reshape(2, 8, -1), as_uint32=True, **dev)] + _args(x, wq, s, y, **dev)[2:])
+    # x[1, 2, K] with a 2-d output: the leading extents must repeat
+    with pytest.raises(vm_harness.PackedError, match="with the leading extents of x"):
+        vm_harness.call_packed("mi355x_q4f16_matmul", _args(x.reshape(1, 2, -1), wq, s, y, **dev))
     xt = torch.zeros((64, 2), dtype=torch.float16).t()  # shape (2, 64), strides (1, 2)
     with pytest.raises(vm_harness.PackedError, match="not compact row-major"):
         vm_harness.call_packed("mi355x_q4f16_matmul", [
@@ -297,7 +305,7 @@ def test_fused_entries_check_their_extra_operand():
             vm_harness.TensorArg(torch.zeros(16, dtype=torch.float32), **dev), a[3]])
     with pytest.raises(vm_harness.PackedError, match=r"residual has shape \(1, 16\), expected \(2, 16\)"):
         vm_harness.call_packed("mi355x_q4f16_matmul_residual", a[:3] + [bias2d, a[3]])
-    with pytest.raises(vm_harness.PackedError, match=r"argument 3 \(residual\): expected a 2-d tensor"):
+    with pytest.raises(vm_harness.PackedError, match=r"residual has shape \(1, 16\), expected \(2, 16\)"):
         vm_harness.call_packed("mi355x_q4f16_matmul_residual", a[:3] + [bias, a[3]])
     if not torch.cuda.is_available():  # every check passes; only the missing device stops the calls
         for sym, extra in (("mi355x_q4f16_matmul_bias", bias), ("mi355x_q4f16_matmul_bias", bias2d),

@@ -124,6 +124,30 @@ def test_gelu_with_the_residual_in_the_output_buffer(bits, m, n, k):
                                 out=h, kernel=lib.KERNEL_GEMM, variant=21)
 
 
+@pytest.mark.parametrize("bits,m,n,k", [(4, 300, 520, 512), (8, 129, 260, 1024), (4, 600, 136, 768)])
+def test_gelu_in_place_on_tile_major_weights(bits, m, n, k):
+    """The same on tile-major weights, which only the direct-weight and the register-activation kernel read: the
+    rows run through the latter, which fuses gelu, in blocks of as many rows as it takes.  (A module with bound
+    weights converts them to this layout when it loads.)"""
+    import relax_amd
+    from tests.test_gpu_parity import _dev
+
+    x, wq, s, g = O.make_case(2100 + m, m, n, k, bits)
+    bias, res = _fused_operands(m + n + 1, m, n)
+    wt, st = relax_amd.wq_tile_weights(_dev(wq), _dev(s), bits, g)
+    h = _dev(res).clone()
+    relax_amd.wq_matmul(_dev(x), wt, st, bits, g, bias=_dev(bias), activation="gelu", residual=h, out=h, tiled_n=n)
+    torch.cuda.synchronize()
+    want = c_oracle.wq_matmul_fused(x, wq, s, bits, g, bias=bias, activation="gelu", residual=res, nthreads=16).astype(np.float64)
+    err = np.abs(h.cpu().numpy().astype(np.float64) - want)
+    assert np.all(err <= 1.5 * (ATOL + RTOL * np.abs(want)) + 2.0 ** -9 * np.abs(want)), (bits, m, float(err.max()))
+    # and with the residual in a buffer of its own the same values come out (two passes on the direct-weight kernel)
+    sep = relax_amd.wq_matmul(_dev(x), wt, st, bits, g, bias=_dev(bias), activation="gelu", residual=_dev(res), tiled_n=n)
+    torch.cuda.synchronize()
+    err2 = np.abs(sep.cpu().numpy().astype(np.float64) - want)
+    assert np.all(err2 <= 1.5 * (ATOL + RTOL * np.abs(want)) + 2.0 ** -9 * np.abs(want)), (bits, m, float(err2.max()))
+
+
 def test_tail_golden_fixtures():
     """The committed fixtures of the gelu and gated tails: at least 99.9 % of the outputs equal the fixture's tail
     applied to this kernel's own matmul output bit for bit, and everything within the matmul tolerance of the fixture."""

@@ -271,3 +271,181 @@ def test_library_scratch_flag_and_packed_call_scratch():
     vm_harness.call_packed("mi355x_wq_packed_call_scratch", targs, spec=spec)
     torch.cuda.synchronize()
     assert torch.equal(y.view(torch.int16), want.view(torch.int16))
+
+
+def test_gated_composite_with_bound_weights():
+    """A gate+up projection whose weights are bound constants -- the normal case of an LLM -- with the tile-major
+    request on: the gated tail runs on canonical weights only, so init keeps the canonical constants and the calls
+    compute; decode and prefill row counts, host and device constants, through export -> load."""
+    import relax_amd
+
+    vm_harness.set_stream()
+    for bits, n, k, rows in ((4, 512, 1024, (1, 8, 160)), (8, 256, 1280, (3, 16))):
+        x_all, wq, s, g = O.make_case(46 + bits, max(rows), n, k, bits)
+        dw, ds = _dev(wq), _dev(s)
+        mod = M.SubgraphModule.create("gu", spec_for(bits, ("wq", "scales", "x", "out"), activation=lib.ACT_SILU_MUL),
+                                      ["w", "s"], [0, 1], M.TILE_WEIGHTS)
+        mod, _ = M.SubgraphModule.load_from_binary(mod.save_to_binary())
+        mod.get_function("__init_gu")(wq, s)  # host arrays, as after load_module
+        for m in rows:
+            dx = _dev(np.ascontiguousarray(x_all[:m]))
+            y = torch.empty((m, n // 2), dtype=torch.float16, device="cuda")
+            mod.get_function("gu")(dx, y)
+            direct = relax_amd.wq_matmul(dx, dw, ds, bits, g, activation="silu_mul")
+            torch.cuda.synchronize()
+            assert torch.equal(y.view(torch.int16), direct.view(torch.int16)), (bits, m)
+            ref = c_oracle.wq_matmul_fused(x_all[:m], wq, s, bits, g, activation="silu_mul", nthreads=8).astype(np.float64)
+            h = np.abs(c_oracle.wq_matmul(x_all[:m], wq, s, bits, g, nthreads=8).astype(np.float64))
+            err = np.abs(y.cpu().numpy().astype(np.float64) - ref)
+            assert np.all(err <= (1e-2 + 1e-2 * np.abs(ref)) * 2 * (1.0 + h[:, :n // 2] + h[:, n // 2:])), (bits, m, float(err.max()))
+        mod.close()
+
+
+@pytest.mark.parametrize("bits, n, k, rows", [(8, 15360, 5120, (256,)), (8, 5120, 5120, (256, 1)), (8, 27648, 5120, (256,)),
+                                              (8, 5120, 13824, (256, 16, 1)), (4, 4096, 11008, (8, 16, 200))])
+@pytest.mark.parametrize("flags", [M.OWN_WORKSPACE, M.OWN_WORKSPACE | M.TILE_WEIGHTS])
+def test_module_owned_workspace(bits, n, k, rows, flags):
+    """MI355X_WQ_MODULE_OWN_WORKSPACE: init allocates and zeroes the K split's workspace for calls of up to
+    `workspace_rows` rows; calls equal the caller-workspace entry bit for bit and match the oracle; the buffer's
+    counters are back at zero after every call; a call of more rows than it was sized for runs as the plain call;
+    the setting survives export -> load."""
+    import relax_amd
+
+    vm_harness.set_stream()
+    tiled = bool(flags & M.TILE_WEIGHTS)
+    x_all, wq, s, g = O.make_case(60 + bits + n % 7, max(rows), n, k, bits)
+    dw, ds = _dev(wq), _dev(s)
+    wt, st = relax_amd.wq_tile_weights(dw, ds, bits, g) if tiled else (dw, ds)
+    mod = M.SubgraphModule.create("f", spec_for(bits, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1], flags, workspace_rows=256)
+    mod, _ = M.SubgraphModule.load_from_binary(mod.save_to_binary())
+    mod.get_function("__init_f")(dw, ds)
+    split_somewhere = False
+    for m in rows:
+        x = np.ascontiguousarray(x_all[:m])
+        dx = _dev(x)
+        y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+        mod.get_function("f")(dx, y)
+        mod.get_function("f")(dx, y)  # (a second call finds the counters at zero again)
+        need = relax_amd.wq_workspace_bytes(bits, g, n, k, m, tiled=tiled)
+        split_somewhere |= need > 0
+        ws = relax_amd.wq_workspace(max(need, 16))
+        ref = relax_amd.wq_matmul(dx, wt, st, bits, g, workspace=ws, **({"tiled_n": n} if tiled else {}))
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), ref.view(torch.int16)), (bits, n, k, m, flags)
+        want = c_oracle.wq_matmul(x[:4], wq, s, bits, g, nthreads=16)
+        assert_close(y[:4].cpu().numpy(), want, (bits, n, k, m, flags), ulp_fraction=0.01)
+    if m >= 64:  # every tile against float32 torch on the bit-exact dequantized weights
+        wd = relax_amd.wq_dequantize(dw, ds, bits, g).float()
+        full = (dx.float() @ wd.t())
+        err = (y.float() - full).abs()
+        assert bool((err <= 2e-2 + 1e-2 * full.abs()).all()), float(err.max())
+    assert split_somewhere or (bits == 8 and n == 27648), "these shapes are meant to split K at some row count"
+    # more rows than the workspace was sized for: the plain call
+    m = 300
+    x, _, _, _ = O.make_case(61, m, 16, k, bits)
+    dx = _dev(x)
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    mod.get_function("f")(dx, y)
+    plain_y = relax_amd.wq_matmul(dx, wt, st, bits, g, **({"tiled_n": n} if tiled else {}))
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), plain_y.view(torch.int16))
+    mod.close()
+
+
+def test_module_owned_workspace_in_a_hip_graph():
+    """Calls on the module's workspace allocate nothing: captured, replayed, equal to eager."""
+    vm_harness.set_stream()
+    bits, m, n, k = 8, 256, 5120, 13824
+    x, wq, s, g = O.make_case(63, m, n, k, bits)
+    mod = M.SubgraphModule.create("f", spec_for(bits, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1], M.OWN_WORKSPACE,
+                                  workspace_rows=m)
+    mod.get_function("__init_f")(_dev(wq), _dev(s))
+    dx = _dev(x)
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    run = mod.get_function("f")
+    run(dx, y)
+    torch.cuda.synchronize()
+    eager = y.clone()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        vm_harness.set_stream(stream)
+        with torch.cuda.graph(graph, stream=stream):
+            run(dx, y)
+    vm_harness.set_stream()
+    for _ in range(3):
+        y.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager)
+
+
+def test_scratch_option_falls_back_where_the_array_is_too_small():
+    """A decode split that would need more than the library's 4 MB array runs unsplit through the packed and module
+    paths (the option is a speed-up, not a reason to fail); the direct entry point still refuses."""
+    import relax_amd
+
+    vm_harness.set_stream()
+    bits, m, n, k = 8, 1, 17408, 8192
+    x, wq, s, g = O.make_case(64, m, n, k, bits)
+    dx, dw, ds = _dev(x), _dev(wq), _dev(s)
+    L = lib.load()
+    need = relax_amd.wq_workspace_bytes(bits, g, n, k, m)
+    assert need > L.mi355x_wq_static_ws_bytes(), "the case is meant to exceed the scratch array"
+    want = relax_amd.wq_matmul(dx, dw, ds, bits, g)
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    targs = [vm_harness.TensorArg(t, as_uint32=(t.dtype == torch.int32)) for t in (dx, dw, ds, y)]
+    vm_harness.call_packed("mi355x_wq_packed_call_scratch", targs, spec=spec_for(bits, ("x", "wq", "scales", "out")))
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), want.view(torch.int16))
+    mod = M.SubgraphModule.create("f", spec_for(bits, ("wq", "scales", "x", "out")), ["w", "s"], [0, 1], M.LIBRARY_SCRATCH)
+    mod.get_function("__init_f")(dw, ds)
+    y.zero_()
+    mod.get_function("f")(dx, y)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), want.view(torch.int16))
+    desc = lib.make_desc(bits, g, n, k)
+    assert L.mi355x_wq_matmul_static_ws(desc, dx.data_ptr(), dw.data_ptr(), ds.data_ptr(), None, y.data_ptr(), m, None, 0) == -1
+    assert "use mi355x_wq_matmul_ws" in lib.last_error()
+
+
+def test_activations_with_leading_extents():
+    """x[B, S, K] against the 2-d weight (src/relax/op/tensor/linear_algebra.cc:46-114): B * S rows; the output, the
+    residual and (with unit extents) the bias carry the same leading extents."""
+    vm_harness.set_stream()
+    bits, n, k = 4, 96, 512
+    x, wq, s, g = O.make_case(65, 10, n, k, bits)
+    rng = np.random.default_rng(6)
+    bias = rng.standard_normal(n).astype(np.float16)
+    res = rng.standard_normal((10, n)).astype(np.float16)
+    dw, ds = _dev(wq), _dev(s)
+    x3 = _dev(x).reshape(2, 5, k)
+    y3 = vm_harness.call_dps("mi355x_q4f16_matmul", [x3, dw, ds], (2, 5, n))
+    torch.cuda.synchronize()
+    assert_close(y3.reshape(10, n).cpu().numpy(), c_oracle.wq_matmul(x, wq, s, bits, g), "x[2, 5, K]")
+    spec = spec_for(bits, ("x", "wq", "scales", "bias", "residual", "out"), activation=lib.ACT_RELU)
+    y = torch.empty((2, 5, n), dtype=torch.float16, device="cuda")
+    targs = [vm_harness.TensorArg(t, as_uint32=(t.dtype == torch.int32))
+             for t in (x3, dw, ds, _dev(bias).reshape(1, 1, n), _dev(res).reshape(2, 5, n), y)]
+    vm_harness.call_packed("mi355x_wq_packed_call", targs, spec=spec)
+    torch.cuda.synchronize()
+    want = c_oracle.wq_matmul_fused(x, wq, s, bits, g, bias=bias, activation="relu", residual=res)
+    assert_close(y.reshape(10, n).cpu().numpy(), want, "fused tail on x[2, 5, K]")
+    # a 1-d x is one row; the gated tail halves the last extent
+    y1 = vm_harness.call_dps("mi355x_q4f16_matmul", [x3[0, 0], dw, ds], (n,))
+    yg = vm_harness.call_dps("mi355x_q4f16_matmul_silu_mul", [x3, dw, ds], (2, 5, n // 2))
+    torch.cuda.synchronize()
+    assert torch.equal(y1, y3[0, 0])
+    assert yg.shape == (2, 5, n // 2)
+    for bad_shape, message in (((10, n), "leading extents of x"), ((5, 2, n), "leading extents of x"), ((2, 5, n + 1), "expected")):
+        with pytest.raises(PackedError, match=message):
+            vm_harness.call_dps("mi355x_q4f16_matmul", [x3, dw, ds], bad_shape)
+    with pytest.raises(PackedError, match="leading extents of x"):
+        targs[4] = vm_harness.TensorArg(_dev(res))  # a 2-d residual beside a 3-d x
+        vm_harness.call_packed("mi355x_wq_packed_call", targs, spec=spec)
+    with pytest.raises(PackedError, match="compact"):
+        wide = torch.zeros((2, 5, 2 * k), dtype=torch.float16, device="cuda")
+        vm_harness.call_packed("mi355x_wq_packed_call",
+                               [vm_harness.TensorArg(wide[:, :, :k], with_strides=True)] + targs[1:3] + [vm_harness.TensorArg(y)],
+                               spec=spec_for(bits, ("x", "wq", "scales", "out")))

@@ -47,7 +47,11 @@ def test_call_before_init_reports_the_reference_message():
     (dict(const_names=["a", "b"], const_args=[0, 0]), "bound by two constants"),
     (dict(const_names=["a"], const_args=[7]), "not the slot"),
     (dict(const_names=["a"], const_args=[0], flags=M.TILE_WEIGHTS), "wq and scales are both constants"),
-    (dict(const_names=["a", "b"], const_args=[0, 1], flags=6), "unknown flags"),
+    (dict(const_names=["a", "b"], const_args=[0, 1], flags=8), "unknown flags"),
+    (dict(const_names=["a"], const_args=[0], flags=M.OWN_WORKSPACE), "needs a matmul whose wq and scales are both constants"),
+    (dict(const_names=["a", "b"], const_args=[0, 1], flags=M.TILE_WEIGHTS, workspace_rows=8), "go with MI355X_WQ_MODULE_OWN_WORKSPACE"),
+    (dict(const_names=["a", "b"], const_args=[0, 1], flags=M.OWN_WORKSPACE, workspace_rows=-1), "workspace rows must be between"),
+    (dict(const_names=["a", "b"], const_args=[0, 1], flags=M.OWN_WORKSPACE, workspace_rows=(1 << 20) + 1), "workspace rows must be between"),
     (dict(const_names=["a", ""], const_args=[0, 1]), "has no name"),
 ])
 def test_create_rejects(kwargs, message):
@@ -78,7 +82,7 @@ def test_binary_form_is_the_documented_stream_encoding():
     m = M.SubgraphModule.create("f0", spec, ["w", "s", "b"], [1, 2, 3], M.TILE_WEIGHTS)
     json = ('{"version": 1, "op": "matmul", "bits": 8, "group": 0, "zero_point": 0, "num_args": 5, "arg_x": 0, '
             '"arg_wq": 1, "arg_scales": 2, "arg_out": 4, "arg_bias": 3, "arg_residual": -1, "activation": 1, '
-            '"flags": 1, "const_args": [1, 2, 3]}')
+            '"flags": 1, "workspace_rows": 0, "const_args": [1, 2, 3]}')
     assert m.json == json
     expect = dmlc_string("f0") + dmlc_string(json) + struct.pack("<Q", 3) + dmlc_string("w") + dmlc_string("s") + dmlc_string("b")
     assert m.save_to_binary() == expect
@@ -86,6 +90,11 @@ def test_binary_form_is_the_documented_stream_encoding():
     assert used == len(expect)
     assert (back.symbol, back.const_names, back.json, back.initialized) == ("f0", ["w", "s", "b"], json, False)
     assert back.save_to_binary() == expect
+    # the rows a module's own workspace is sized for travel with it (a description without the key: none)
+    ws = M.SubgraphModule.create("f1", spec_matmul(), ["w", "s"], [0, 1], M.TILE_WEIGHTS | M.OWN_WORKSPACE, workspace_rows=256)
+    assert '"flags": 5, "workspace_rows": 256,' in ws.json
+    ws_back, _ = M.SubgraphModule.load_from_binary(ws.save_to_binary())
+    assert ws_back.json == ws.json and ws_back.save_to_binary() == ws.save_to_binary()
     # JSON written by another producer: other key order and white space
     other = '{ "const_args":[1,2,3],"flags":1,"activation":1,"arg_residual":-1,"arg_bias":3,"arg_out":4,\n"arg_scales":2,' \
             '"arg_wq":1,"arg_x":0,"num_args":5,"zero_point":0,"group":0,"bits":8,"op":"matmul","version":1 }'

@@ -253,6 +253,11 @@ def test_bound_weights_give_a_module_plan(fake_tvm):
     assert module_plan(f, constants_of(f)).flags == MODULE_TILE_WEIGHTS
     f = fake_tvm.quantized_linear(bound=("wq", "scales"), k=256)
     assert module_plan(f, constants_of(f), tile_weights=False).flags == 0
+    # the gated tail is computed on canonical weights only: a gate+up composite keeps its canonical constants (a
+    # module that converted them would refuse every call)
+    f = fake_tvm.quantized_linear(bound=("wq", "scales"), k=256, tail=[("silu_mul",)])
+    plan = module_plan(f, constants_of(f))
+    assert plan.flags == 0 and plan.spec.activation == 2 and (plan.spec.arg_x, plan.spec.arg_out, plan.spec.num_args) == (2, 3, 4)
     # only the weights bound, scales a parameter: no tile-major conversion (it needs both)
     f = fake_tvm.quantized_linear(bound=("wq",))
     plan = module_plan(f, constants_of(f))
@@ -350,7 +355,6 @@ def test_bound_constants_stay_inside_the_composite(fake_tvm):
     (dict(out_dtype="float16"), "out_dtype float32"),
     (dict(astype_dtype="float32"), "must produce float16"),
     (dict(axes=[0, 1]), "2-d transpose"),
-    (dict(x_shape=[2, 4, 128]), "x must be a 2-d tensor"),
     (dict(x_dtype="float32"), "x must be float16"),
 ])
 def test_role_derivation_rejects_composites_the_kernels_do_not_compute(fake_tvm, kwargs, message):
@@ -389,16 +393,29 @@ def test_hook_honours_its_options(fake_tvm, monkeypatch):
     # defaults: tile-major conversion on, no scratch
     mods = codegen.relax_ext_mi355x([bound, free], None, names)
     assert [m[0] for m in mods] == ["module", "csource"]
-    assert created[0][-1] == codegen.MODULE_TILE_WEIGHTS and "mi355x_wq_packed_call(&spec" in created[1][1]
+    # (the creator's last two arguments: the module's flags and the rows its workspace is sized for)
+    assert created[0][-2:] == (codegen.MODULE_TILE_WEIGHTS, 0) and "mi355x_wq_packed_call(&spec" in created[1][1]
     created.clear()
+    # workspace: a function with bound weights gets a workspace of its own, sized at load for 2048 rows unless the
+    # options say otherwise; a function whose weights are parameters goes through the library's scratch array
     codegen.relax_ext_mi355x([bound, free], {"tile_weights": False, "workspace": True}, names)
-    assert created[0][-1] == codegen.MODULE_LIBRARY_SCRATCH
+    assert created[0][-2:] == (codegen.MODULE_OWN_WORKSPACE, 2048)
     assert "mi355x_wq_packed_call_scratch(&spec" in created[1][1] and created[1][3] == ["free_mi355x"]
     created.clear()
-    codegen.relax_ext_mi355x([bound], {"workspace": 1}, names)  # integers as TVM passes them
-    assert created[0][-1] == codegen.MODULE_TILE_WEIGHTS | codegen.MODULE_LIBRARY_SCRATCH
+    codegen.relax_ext_mi355x([bound], {"workspace": 1, "workspace_rows": 64}, names)  # integers as TVM passes them
+    assert created[0][-2:] == (codegen.MODULE_TILE_WEIGHTS | codegen.MODULE_OWN_WORKSPACE, 64)
+    created.clear()
+    codegen.relax_ext_mi355x([bound], {"workspace_rows": 64}, names)  # rows without the switch: no workspace
+    assert created[0][-2:] == (codegen.MODULE_TILE_WEIGHTS, 0)
+    created.clear()
+    # only the packed weights bound: N and K are known at load, the group is not -- the library's scratch array
+    half_bound = fake_tvm.quantized_linear(bound=("wq",), k=256, symbol="half_mi355x")
+    codegen.relax_ext_mi355x([half_bound], {"workspace": True}, constants_of(half_bound))
+    assert created[0][-2:] == (codegen.MODULE_LIBRARY_SCRATCH, 0)
     with pytest.raises(ValueError, match="unknown option 'tile_weight'"):
         codegen.relax_ext_mi355x([free], {"tile_weight": True}, {})
+    with pytest.raises(ValueError, match="workspace_rows must be between"):
+        codegen.relax_ext_mi355x([bound], {"workspace": True, "workspace_rows": 0}, names)
 
 
 def test_gated_tail_of_a_gate_up_projection(fake_tvm):
