@@ -32,33 +32,36 @@ HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
 GEMV_PROFILE = os.path.join(ROOT, "profiles", "gemv_decode_llama7b.md")
 GEMV_KERNEL_SOURCES = ("relax_amd/csrc/wq_gemv.hip", "relax_amd/csrc/wq_device.h")
+GEMM_PROFILE = os.path.join(ROOT, "profiles", "gemm_prefill_llama7b.md")
+GEMM_KERNEL_SOURCES = ("relax_amd/csrc/wq_gemm_direct.hip", "relax_amd/csrc/wq_device.h")
+PROBE_SO = os.path.join(ROOT, "relax_amd", "csrc", "libmi355x_probe.so")
 
 
-def kernel_sources_digest() -> str:
-    """sha256 over the decode kernel's source files (what a counter summary is valid for)."""
+def kernel_sources_digest(sources=GEMV_KERNEL_SOURCES) -> str:
+    """sha256 over a kernel's source files (what a counter summary is valid for)."""
     import hashlib
 
     h = hashlib.sha256()
-    for rel in GEMV_KERNEL_SOURCES:
+    for rel in sources:
         with open(os.path.join(ROOT, rel), "rb") as f:
             h.update(f.read())
     return h.hexdigest()
 
 
-def measured_traffic():
-    """HBM bytes per GEMV launch of this workload, from the tracked rocprofv3 counter summary
+def measured_traffic(profile=GEMV_PROFILE, sources=GEMV_KERNEL_SOURCES):
+    """HBM bytes per launch of a leg's dominant kernel, from the tracked rocprofv3 counter summary
     (FETCH_SIZE / WRITE_SIZE per dispatch, scaled by the copy of known size that runs first).
     The summary names the digest of the kernel sources it was taken on; when the sources have
     changed since, the figure is stale and None is returned."""
     import re
 
     try:
-        text = open(GEMV_PROFILE).read()
+        text = open(profile).read()
     except OSError:
         return None
     traffic = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", text, re.M)
     digest = re.search(r"^kernel_sources_sha256:\s*([0-9a-f]{64})", text, re.M)
-    if not traffic or not digest or digest.group(1) != kernel_sources_digest():
+    if not traffic or not digest or digest.group(1) != kernel_sources_digest(sources):
         return None
     return int(traffic.group(1))
 
@@ -317,6 +320,7 @@ def main() -> int:
     ap.add_argument("--no-ksplit", action="store_true", help="skip the caller-workspace (K split) leg")
     ap.add_argument("--no-tiled", action="store_true", help="skip the tile-major-weights decode leg")
     ap.add_argument("--no-streams", action="store_true", help="skip the two-stream (two independent chains) leg")
+    ap.add_argument("--no-read-floor", action="store_true", help="skip the read-only floor leg")
     ap.add_argument("--no-sustained", action="store_true",
                     help="skip the sustained-load segments that sample clock and power (use under a profiler)")
     ap.add_argument("--configs", action="store_true",
@@ -549,7 +553,8 @@ def main() -> int:
             result["gemm"]["tile_major_tflops"] = round(flops / (sum(ours_tiled) / len(ours_tiled) * 1e-3) / 1e12, 1)
         result["roofline_gemm"] = {"bound": "mfma", "achieved": round(tflops, 1),
                                    "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                   "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                                   "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4),
+                                   "traffic": measured_traffic(GEMM_PROFILE, GEMM_KERNEL_SOURCES),
                                    "kernel": "wq::wq_gemm_direct_kernel"}
         del wds, tiled_w
 
@@ -638,6 +643,56 @@ def main() -> int:
                         "do not add up to the step time -- `value` above stays the one-stream figure"
                         % launches_per_step}
         del sgraph
+
+    if not args.no_read_floor and os.path.exists(PROBE_SO):
+        # Context for the HBM fraction: a kernel that only reads -- the same packed weights and scales, one
+        # launch per matrix, the same number of launches in one HIP graph -- i.e. what launch gaps, cold starts
+        # and tails leave of the 8 TB/s for these byte counts with no arithmetic, staging or reduction.  The
+        # kernel lives in a measurement library of its own; without that file the leg is left out.
+        import ctypes
+
+        rd = ctypes.CDLL(PROBE_SO).mi355x_probe_stream_read
+        rd.argtypes = [ctypes.c_void_p, ctypes.c_longlong, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_void_p,
+                       ctypes.c_int, ctypes.c_void_p]
+        sink = torch.zeros(64, dtype=torch.int32, device=dev)
+        floor = {}
+        for blocks in (256, 512, 1024):
+            def read_pass():
+                sp = int(stream.cuda_stream)
+                for _ in DECODE_BATCHES:
+                    for mats in layers:
+                        for wq, s, n, k in mats:
+                            rc = rd(wq.data_ptr(), wq.numel() * 4, s.data_ptr(), s.numel() * 2, sink.data_ptr(), blocks, sp)
+                            if rc != 0:
+                                raise RuntimeError("read-only probe: HIP error %d" % rc)
+
+            with torch.cuda.stream(stream):
+                read_pass()
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=stream):
+                    read_pass()
+                gr.replay()
+                torch.cuda.synchronize()
+                r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                r0.record(stream)
+                for _ in range(args.steps):
+                    gr.replay()
+                r1.record(stream)
+                torch.cuda.synchronize()
+            floor[blocks] = r0.elapsed_time(r1) / args.steps
+            del gr
+        best_blocks = min(floor, key=floor.get)
+        weight_bytes = len(DECODE_BATCHES) * sum(wq.numel() * 4 + s.numel() * 2 for mats in layers for wq, s, _, _ in mats)
+        fgbs = weight_bytes / (floor[best_blocks] * 1e-3) / 1e9
+        result["read_floor"] = {
+            "value": round(fgbs, 1), "unit": "GB/s", "frac": round(fgbs / HBM_PEAK_GBS, 4),
+            "ms_per_step": round(floor[best_blocks], 4), "avg_launch_us": round(floor[best_blocks] * 1e3 / launches_per_step, 3),
+            "workgroups": best_blocks, "ms_per_step_by_workgroups": {str(b): round(t, 4) for b, t in floor.items()},
+            "decode_step_over_floor": round(ms_per_step / floor[best_blocks], 3),
+            "workload": "a kernel that only reads the same packed weights and scales (1 KB contiguous per wavefront "
+                        "instruction, four requests in flight per thread), one launch per matrix, the same %d launches "
+                        "in one HIP graph; best of 256 / 512 / 1024 workgroups of 512 threads" % launches_per_step}
 
     if not args.no_ksplit:
         # the down projection (4096 x 11008) of every layer at 8 rows: the one case of this step where a
