@@ -35,6 +35,7 @@ GEMV_KERNEL_SOURCES = ("relax_amd/csrc/wq_gemv.hip", "relax_amd/csrc/wq_device.h
 GEMM_PROFILE = os.path.join(ROOT, "profiles", "gemm_prefill_llama7b.md")
 GEMM_KERNEL_SOURCES = ("relax_amd/csrc/wq_gemm_direct.hip", "relax_amd/csrc/wq_device.h")
 PROBE_SO = os.path.join(ROOT, "relax_amd", "csrc", "libmi355x_probe.so")
+STAMPS_SO = os.path.join(ROOT, "relax_amd", "csrc", "libmi355x_wq_stamps.so")
 
 
 def kernel_sources_digest(sources=GEMV_KERNEL_SOURCES) -> str:
@@ -308,6 +309,84 @@ def config_table(torch, dev, args) -> int:
     return 0
 
 
+def stamp_budget(torch, dev, args, L) -> int:
+    """Where a decode launch spends its time, from the wavefronts' own clock readings.
+
+    Runs the headline chain (the four projections per layer, one HIP graph per batch size) on the build of the
+    library whose decode kernel records the 100 MHz real-time counter at eight points of every wavefront's life,
+    reads back the last layer's four launches and prints, per shape and batch size, the distribution over
+    wavefronts of each point relative to the launch's first wavefront entry, the pause since the previous
+    launch's last acknowledged store, and the graph's time per launch with the hooks in (HIP events)."""
+    import ctypes
+
+    import numpy as np
+
+    import relax_amd
+
+    points = ["entry", "first requests issued", "activations in LDS", "first super step done", "weight stream end",
+              "before the last barrier", "after the last barrier", "stores acknowledged"]
+    launches, waves, npoints = 4, 4096, len(points)
+    L.mi355x_wq_stamps_read.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    torch.manual_seed(0)
+    layers = []
+    for _ in range(args.layers):
+        layers.append([(torch.randint(-2**31, 2**31 - 1, (n, k // 8), dtype=torch.int32, device=dev),
+                        (torch.rand((n, k // 32), device=dev) * 0.015 + 0.005).to(torch.float16), n, k)
+                       for _, n, k in LLAMA7B])
+    stream = torch.cuda.Stream()
+    for m in DECODE_BATCHES:
+        xs = {k: torch.randn((m, k), device=dev).to(torch.float16) for k in (4096, 11008)}
+        ys = {n: torch.empty((m, n), dtype=torch.float16, device=dev) for _, n, _ in LLAMA7B}
+
+        def chain():
+            for mats in layers:
+                for wq, sc, n, k in mats:
+                    relax_amd.wq_matmul(xs[k], wq, sc, 4, 32, out=ys[n])
+
+        with torch.cuda.stream(stream):
+            chain()
+            torch.cuda.synchronize()
+            if L.mi355x_wq_stamps_reset() != 0:
+                raise RuntimeError("resetting the stamp array failed")
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                chain()  # (the launch count, hence the slot, is fixed at capture: layer l, shape j -> slot j)
+            for _ in range(3):
+                g.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(10):
+                g.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+        per_launch = e0.elapsed_time(e1) * 1e3 / (10 * len(layers) * len(LLAMA7B))
+        buf = (ctypes.c_ulonglong * (launches * waves * npoints))()
+        if L.mi355x_wq_stamps_read(buf, launches * waves * npoints) != 0:
+            raise RuntimeError("reading the stamp array failed")
+        a = np.array(buf[:], dtype=np.int64).reshape(launches, waves, npoints)
+        print(f"batch {m}: {per_launch:.2f} us per launch with the hooks in ({len(layers) * len(LLAMA7B)} launches per graph)")
+        print("| shape | wavefronts | pause before | " + " | ".join(points[1:]) + " | first entry -> last end |")
+        print("|---|---|---|" + "---|" * len(points))
+        prev_end = None
+        for j, (name, n, k) in enumerate(LLAMA7B):
+            r = a[j]
+            r = r[r[:, 0] > 0]
+            r = r[r[:, 7] > r[:, 7].max() - 5000]  # the last replay's wavefronts (50 us window)
+            t0 = r[:, 0].min()
+            rel = (r - t0) / 100.0
+            pause = "" if prev_end is None else f"{(t0 - prev_end) / 100.0:.2f}"
+            cells = []
+            for q in range(1, npoints):
+                c = rel[:, q]
+                cells.append(f"{np.median(c):.2f} ({c.min():.2f}-{c.max():.2f})")
+            print(f"| {name} {n}x{k} | {len(r)} | {pause} | " + " | ".join(cells) + f" | {rel[:, 7].max():.2f} |")
+            prev_end = r[:, 7].max()
+        sys.stdout.flush()
+        del g
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -327,6 +406,9 @@ def main() -> int:
                     help="instead of the benchmark: time every shape of the decode, prefill and q8f16 "
                          "configurations on its own (weights rotated through more than 2 GB, one HIP "
                          "graph per case) and print one line per case")
+    ap.add_argument("--stamps", action="store_true",
+                    help="instead of the benchmark: the decode chain on the library build with time-stamp hooks "
+                         "(libmi355x_wq_stamps.so); prints where the wavefronts of a launch spend their time")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the hot path is a single-GPU kernel and this build has no "
@@ -338,10 +420,15 @@ def main() -> int:
     import relax_amd
     from relax_amd import lib
 
-    lib.load()  # fails loudly if the HIP library is missing
+    if args.stamps:
+        lib.SO_PATH = STAMPS_SO  # the same library with the decode kernel's measurement hooks compiled in
+    L = lib.load()  # fails loudly if the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     torch.manual_seed(0)
+
+    if args.stamps:
+        return stamp_budget(torch, dev, args, L)
 
     if args.configs:
         return config_table(torch, dev, args)

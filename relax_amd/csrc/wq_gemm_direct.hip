@@ -495,6 +495,9 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
     // returns the counter to zero for the next launch.  Partials and counters are only touched by accesses that
     // are performed at the memory side of the chip's L2s (sc1), and a workgroup's stores have completed before
     // the barrier after which its count goes out.
+    // What would break it: one plain load or store (no sc1) of a partial or a counter word, here or in any kernel
+    // that shares the workspace -- it may be served from a stale line of the reader's L2 or stay dirty in the
+    // writer's.  A source-level test refuses such an access.
     const bool owner = GROUPS == 1 || grp == 0;
     constexpr uint32_t kWaveFloats = TM * 2 * 16 * 64;  // accumulators of one wavefront
     const rsrc_t rp = make_rsrc(partials + (size_t)tile_lin * S * WAVES * kWaveFloats, (uint32_t)S * WAVES * kWaveFloats * 4u);

@@ -34,10 +34,14 @@
 // exactly what a wavefront reads per instruction (D = 2): every load of the weight stream
 // is 1 KB contiguous.  Same lanes, same chunks, same order: bit-identical results.
 //
-// ROWS: how the activations reach LDS.  false: a flat index over (row, 16-byte column), two requests
-// per thread ahead of the first weights (batch 1 - 2, or rows longer than the workgroup has
-// threads); true: a thread stages its own column of four or eight rows, all requested ahead of
-// the first weights.
+// XS: how the first phase's activations reach LDS, a build each -- the start-up of a launch runs on a cold
+// instruction cache, and every alternative it has to jump over costs a fetch from memory (with all of them in one
+// build a batch-1 launch took 0.3 us longer).  0: a flat index over (row, 16-byte column) of any shape, up to
+// three requests per thread ahead of the first weights, the rest in a loop (batch 1 - 2, or rows longer than
+// the workgroup has threads); 1, 2, 3: the same for exactly that many requests per thread and rows of at least as
+// many vectors as the workgroup has threads (K >= 4096 with eight wavefronts) -- straight-line code, no division;
+// 4, 8, 16: a thread stages its own column of up to that many rows, the first four or eight requested ahead of the
+// first weights.
 //
 // KSPLIT: K is split over R workgroups per tile list as well (caller workspace): each writes a
 // float32 partial tile, the last to arrive adds them in the order of the K windows and stores.
@@ -49,6 +53,19 @@
 #include "wq_internal.h"
 
 namespace wq {
+
+// Measurement build (-DWQ_GEMV_STAMPS, linked into a library of its own that only bench.py --stamps loads): every
+// wavefront records the 100 MHz real-time counter at eight points of its life -- entry, first requests issued,
+// activations staged, first super step computed, end of the weight stream, before and after the barrier ahead of the
+// slot sum, stores acknowledged -- into a device array with one slot per launch modulo four, so that the last four
+// launches of a replayed graph can be read back.  In the product build the hooks expand to nothing.
+#ifdef WQ_GEMV_STAMPS
+constexpr int kStampLaunches = 4, kStampWaves = 4096, kStampPoints = 8;
+__device__ unsigned long long g_gemv_stamps[kStampLaunches * kStampWaves * kStampPoints];
+#define WQ_STAMP(i) (stamps_[i] = __builtin_amdgcn_s_memrealtime())
+#else
+#define WQ_STAMP(i) ((void)0)
+#endif
 
 template <int D, int SPL>
 struct GemvBuf {
@@ -66,7 +83,7 @@ struct GemvCtx {
 
 // The kernel's argument segment as a struct (arguments are laid out in order with their natural alignment):
 // the kernel reads the arguments that only its last section needs -- the output, the epilogue, the K split's
-// workspace -- through the segment pointer, behind an optimisation barrier at the start of that section.  Left to
+// workspace -- through the segment pointer, at a place of the kernel's choosing (fetch_late_arguments).  Left to
 // itself the compiler fetches them at the top of the kernel and, in the builds that run short of scalar registers,
 // waits for that fetch (a trip to host-visible memory) to spill them: ahead of the first weight request.
 struct GemvKernArgs {
@@ -80,7 +97,7 @@ struct GemvKernArgs {
   unsigned int* counters;
 };
 
-template <int BITS, int WAVES, int D, int SPL, bool TILED, bool ROWS, bool KSPLIT, bool PHASES>
+template <int BITS, int WAVES, int D, int SPL, bool TILED, int XS, bool KSPLIT, bool PHASES>
 // PHASES: the launch walks K in more than one phase (activations beyond the LDS).  The host knows; as a template
 // flag it keeps the second phase description out of the build that runs the common launches, whose first memory
 // requests otherwise wait behind that bookkeeping (and behind the late kernel arguments, which the compiler
@@ -102,7 +119,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
     int shift_and_zero_, int max_tiles_, int phase_chunks_, int ksplit_, int grid_, half_t* y_late, const Epilogue ep_late,
     float* partials_late, unsigned int* counters_late) {
   static_assert(!KSPLIT || !PHASES, "the cross-workgroup K split walks one window of K");
-  constexpr bool XPRE = PHASES && ROWS;  // (up to eight rows) a phase's activations are requested a phase ahead
+  static_assert(XS == 0 || XS == 1 || XS == 2 || XS == 3 || XS == 4 || XS == 8 || XS == 16, "staging mode");
+  constexpr bool ROWS = XS >= 4;
+  constexpr bool XPRE = PHASES && (XS == 4 || XS == 8);  // (up to eight rows) a phase's activations are requested a phase ahead
   const int group_shift_ = shift_and_zero_ & 0xFF, zero_point_ = (shift_and_zero_ >> 8) & 0xFF;
   const bool gated = (shift_and_zero_ >> 16) & 1;  // fused multiply(nn.silu(gate), up): rows walked interleaved
   const int tiles_ = (N_ + 15) >> 4;
@@ -117,6 +136,10 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps loop control scalar
   const int col = lane & 15, kq = lane >> 4;
+#ifdef WQ_GEMV_STAMPS
+  unsigned long long stamps_[kStampPoints] = {};
+#endif
+  WQ_STAMP(0);
   const int M = M_, N = N_, K = K_;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char wq_gemv_smem[];
@@ -132,6 +155,24 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
   const rsrc_t rw = make_rsrc(wq_, n_stored * row_bytes);
   const rsrc_t rs = make_rsrc(scales_, n_stored * groups_per_row * 2u);
   const rsrc_t rx = make_rsrc(x_, (uint32_t)M * (uint32_t)K * 2u);
+
+  // XS = 1, 2, 3: the activation requests ahead of everything else -- they need nothing but the thread index and the
+  // shape.  Vector q of this thread is index tid + q * NT of the flat order, in row 0, 1 or 2 (rows have at least
+  // NT vectors, launch_one checks); one phase: a vector inside K is inside the phase.
+  constexpr int XQ = (XS >= 1 && XS <= 3) ? XS : 1;
+  int mq[XQ], kvq[XQ];
+  u32x4 xq[XQ];
+  if constexpr (XS >= 1 && XS <= 3) {
+    const int vec_per_row = (nchunks + 4 * D - 1) / (4 * D) * (4 * D) * CH / 8;
+#pragma unroll
+    for (int q = 0; q < XS; ++q) {
+      mq[q] = q == 0 ? 0 : (tid + q * NT >= vec_per_row ? 1 : 0) + (tid + q * NT >= 2 * vec_per_row ? 1 : 0);
+      kvq[q] = tid + q * NT - mq[q] * vec_per_row;
+      const bool ok = mq[q] < M && kvq[q] * 8 < K;
+      xq[q] = load_b128(rx, ok ? ((uint32_t)mq[q] * (uint32_t)K + (uint32_t)(kvq[q] * 8)) * 2u : kOobOffset);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   // Tiles of this workgroup: tile0, tile0 + tstride, ...  With the K split, R consecutive workgroups
   // share a tile list and each walks its own window of K (phase_chunks chunks from kr * phase_chunks).
@@ -263,7 +304,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
   // frees is filled with the first item of the next phase, so that the phase boundary (a barrier, the
   // activations of the next K range into LDS, a barrier) does not find the memory pipeline empty.
   GemvBuf<D, SPL> b0, b1;
-  // (the late arguments: fetched from the argument segment once the first phase's requests are out, see GemvKernArgs)
+  // (the late arguments: fetched from the argument segment by fetch_late_arguments, see GemvKernArgs and below)
   half_t* y_ = nullptr;
   Epilogue ep_ = Epilogue{nullptr, nullptr, 0};
   float* partials_ = nullptr;
@@ -296,7 +337,6 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
     *reinterpret_cast<u32x4*>(xs + (size_t)m * lds_stride + kv * 8) = permute_x(v);
   };
 
-  // behind the first phase's requests: the scalar loads' latency runs beside that of the activations
   auto fetch_late_arguments = [&]() {
     typedef const __attribute__((address_space(4))) GemvKernArgs* kernarg_ptr_t;
     kernarg_ptr_t late = (kernarg_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();
@@ -307,6 +347,20 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
       partials_ = late->partials;
       counters_ = late->counters;
     }
+  };
+
+  // Where the fetch goes.  The loads are plain loads from constant memory, which the compiler moves freely: placed
+  // behind the first weight requests they sank below the first activation store, i.e. behind the wait for the
+  // first activations, and the barrier that ends the staging then waited for a scalar load issued a memory trip
+  // late (0.5 us per launch on a 4096 x 4096 projection at batch 1).  The builds that walk K in one phase have the
+  // scalar registers to hold the seven values from the top of the kernel, so they fetch there, and an empty asm
+  // ahead of the staging barrier names the values as inputs: the loads cannot sink past it, and that barrier's
+  // wait for the LDS stores covers them.  The K-phase builds are short of scalar registers (a fetch at the top makes
+  // them wait for it and spill the values ahead of their first request): they fetch behind their first requests.
+  if constexpr (!PHASES) fetch_late_arguments();
+  auto pin_late_arguments = [&]() {
+    asm volatile("" ::"s"(y_), "s"(ep_.bias), "s"(ep_.residual), "s"(ep_.activation));
+    if constexpr (KSPLIT) asm volatile("" ::"s"(partials_), "s"(counters_));
   };
 
   // One K phase: stage its activations, stream every tile of the workgroup over it.  The first phase
@@ -320,7 +374,17 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
     // for the much slower first weight loads.
     const int vec_per_row = ((c.nsuper * 4 * D + 3) / 4) * 4 * CH / 8;
     if (ph == 0) {
-      if constexpr (!ROWS) {
+      if constexpr (XS >= 1 && XS <= 3) {
+        // exactly XS vectors per thread, rows of at least NT vectors (launch_one checks): vector q of this thread
+        // is index tid + q * NT of the flat order, in row 0, 1 or 2
+        static_assert(!PHASES && !KSPLIT, "one phase over all of K");
+        // (the requests went out at the top of the kernel)
+        load_super(b0, c, first_tile(c), 0);
+        __builtin_amdgcn_sched_barrier(0);
+        WQ_STAMP(1);
+#pragma unroll
+        for (int q = 0; q < XS; ++q) x_store_of(c, mq[q], kvq[q], xq[q]);
+      } else if constexpr (!ROWS) {
         // one or two rows, or rows longer than the workgroup has threads: a flat index over (row, column),
         // up to three vectors per thread ahead of the weights -- as many as the activations have, each
         // further one under a wave-uniform branch.  (Every request, even one that is masked off, takes its
@@ -361,7 +425,8 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
         __builtin_amdgcn_sched_barrier(0);
         load_super(b0, c, first_tile(c), 0);
         __builtin_amdgcn_sched_barrier(0);
-        fetch_late_arguments();
+        if constexpr (PHASES) fetch_late_arguments();
+        WQ_STAMP(1);
         x_store_of(c, m0, kv0, x0);
         if (second) x_store_of(c, m1, kv1, x1);
         if (third) x_store_of(c, m2, kv2, x2);
@@ -394,18 +459,18 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
           __builtin_amdgcn_sched_barrier(0);
           load_super(b0, c, first_tile(c), 0);
           __builtin_amdgcn_sched_barrier(0);
-          fetch_late_arguments();
+          if constexpr (PHASES) fetch_late_arguments();
+          WQ_STAMP(1);
 #pragma unroll
           for (int r = 0; r < RM; ++r) x_store_of(c, r, tid, xv[r]);
-          for (int m0 = RM; m0 < M; m0 += RM) {
+          if constexpr (XS == 16) {  // rows 8 .. 15
 #pragma unroll
-            for (int r = 0; r < RM; ++r) xv[r] = x_load_of(c, m0 + r, tid);
+            for (int r = 0; r < RM; ++r) xv[r] = x_load_of(c, RM + r, tid);
 #pragma unroll
-            for (int r = 0; r < RM; ++r) x_store_of(c, m0 + r, tid, xv[r]);
+            for (int r = 0; r < RM; ++r) x_store_of(c, RM + r, tid, xv[r]);
           }
         };
-        if (M <= 4) stage(std::integral_constant<int, 4>{});
-        else stage(std::integral_constant<int, 8>{});
+        stage(std::integral_constant<int, XS == 4 ? 4 : 8>{});
       }
     } else {
       __syncthreads();  // every wavefront is done reading the previous phase
@@ -419,13 +484,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
         }
       };
       if constexpr (XPRE) {
-        if (M <= 8) {
-          // (requested at the start of the previous phase: here long since)
+        // (requested at the start of the previous phase: here long since)
 #pragma unroll
-          for (int r = 0; r < 8; ++r) x_store_of(c, r, tid, xn[r]);
-        } else {
-          restage_rows();
-        }
+        for (int r = 0; r < 8; ++r) x_store_of(c, r, tid, xn[r]);
       } else if constexpr (ROWS) {
         restage_rows();
       } else {
@@ -440,16 +501,16 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
       }
       if (!b0_loaded) load_super(b0, c, first_tile(c), 0);
     }
+    if (ph == 0) pin_late_arguments();
     __syncthreads();
     if constexpr (XPRE) {
       // the next phase's column of this thread, behind the one item that is in flight
-      if (M <= 8) {
 #pragma unroll
-        for (int r = 0; r < 8; ++r) xn[r] = x_load_of(cn, r, tid);
-      }
+      for (int r = 0; r < 8; ++r) xn[r] = x_load_of(cn, r, tid);
       __builtin_amdgcn_sched_barrier(0);
     }
 
+    if (ph == 0) WQ_STAMP(2);
     // ---- the weight stream: a flat software pipeline over (tile, super step) ----------
     // Two items per trip, unconditionally (with an early exit in between, the compiler
     // sinks the prefetch below the compute).  Items past the end load zeros from an
@@ -462,6 +523,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
       load_super(b1, c, pi, ps);
       __builtin_amdgcn_sched_barrier(0);
       compute_super(b0, x_of(c, cs));
+      if (ph == 0 && j == 0) WQ_STAMP(3);
       if (cs == c.cnt - 1) flush_tile(ci, ph == 0);
       advance(c, ci, cs);
       __builtin_amdgcn_sched_barrier(0);
@@ -486,6 +548,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
       advance(c, ci, cs);
       __builtin_amdgcn_sched_barrier(0);
     }
+    WQ_STAMP(4);
     // a wavefront without work in the first phase still owns slots that the epilogue sums
     if (ph == 0 && c.cnt == 0)
       for (int i = 0; i < my_tiles; ++i) flush_tile(i, true);
@@ -504,8 +567,13 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
   }
 
   // ---- sum the wavefronts' partial tiles, convert, store -----------------------------
+  WQ_STAMP(5);
   __syncthreads();
+  WQ_STAMP(6);
   if constexpr (!KSPLIT) {
+    // (the plain store first and on its own: the tails' code -- erf, exp -- is then a block the common launch never
+    // enters, instead of four stretches it jumps over on a cold instruction cache)
+    const bool plain = !gated && ep_.bias == nullptr && ep_.residual == nullptr && ep_.activation == 0;
     for (int idx = tid; idx < my_tiles * 256; idx += NT) {
       const int i = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
       const int m = 4 * (l >> 4) + r;
@@ -514,7 +582,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) sum += slots[((size_t)(i * WAVES + w) * 4 + r) * 64 + l];
-        if (gated) {
+        if (plain) {
+          y_[(size_t)m * N + n] = (half_t)sum;
+        } else if (gated) {
           // adjacent columns of the tile hold a gate / up pair: the even lane also sums its neighbour's
           if ((l & 1) == 0 && n + 1 < N) {
             float up = 0.f;
@@ -544,6 +614,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
     // the counters are only ever touched by device-scope atomic stores, loads and adds, which are
     // performed at the memory side of the L2s; a workgroup's stores have completed (vmcnt(0)) before
     // the barrier after which its count goes out.
+    // What would break it: one plain (non-atomic, or workgroup-scope) load or store of a partial or a counter
+    // word, in this kernel or any other that shares the workspace -- it may be served from a stale line of the
+    // reader's L2 or stay dirty in the writer's.  A source-level test refuses such an access.
     for (int idx = tid; idx < my_tiles * 256; idx += NT) {
       const int i = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
       float sum = 0.f;
@@ -573,6 +646,16 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
     if (tid < my_tiles && last[tid])
       __hip_atomic_store(&counters_[tile0 + tid * tstride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+#ifdef WQ_GEMV_STAMPS
+  // (the plain builds do not use ksplit_: the measurement build's launcher passes a launch counter there)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  WQ_STAMP(7);
+  if (!KSPLIT && lane == 0 && (int)blockIdx.x * WAVES + wave < kStampWaves) {
+    unsigned long long* t =
+        g_gemv_stamps + ((size_t)(ksplit_ & (kStampLaunches - 1)) * kStampWaves + (size_t)blockIdx.x * WAVES + wave) * kStampPoints;
+    for (int q = 0; q < kStampPoints; ++q) t[q] = stamps_[q];
+  }
+#endif
 }
 
 namespace {
@@ -630,6 +713,19 @@ bool make_plan(const Problem& p, int wgs_per_cu, Plan* out) {
 // the kernel was launched, or a runtime call failed (error already set).
 enum { kNotApplicable = 0, kLaunched = 1, kFailed = -1 };
 
+#ifdef WQ_GEMV_STAMPS
+int g_stamp_launches = 0;  // launches since the last reset: selects the slot a launch records into
+#endif
+
+// the kernel's ksplit argument (the measurement build numbers the plain launches there instead)
+inline int stamp_slot_or(int ksplit, bool split_build) {
+#ifdef WQ_GEMV_STAMPS
+  if (!split_build) return g_stamp_launches++;
+#endif
+  (void)split_build;
+  return ksplit;
+}
+
 template <int BITS, int WAVES, int D, int SPL, bool TILED = false, bool KSPLIT = false>
 int launch_one(const Problem& p, int group_shift, const Plan& plan, int ksplit = 1, void* workspace = nullptr) {
   const Epilogue ep{(const half_t*)p.bias, (const half_t*)p.residual, p.activation};
@@ -638,32 +734,46 @@ int launch_one(const Problem& p, int group_shift, const Plan& plan, int ksplit =
   // zero -- then [tiles][ksplit][256] float partial tiles
   unsigned int* const counters = static_cast<unsigned int*>(workspace);
   float* const partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kSplitCounterBytes);
-  // the builds of the kernel: by the way the activations are staged (flat index / a column per thread) and by
-  // whether K is walked in several phases
-  auto go = [&](auto rows, auto phases) -> int {
-    constexpr bool ROWS = decltype(rows)::value, PHASES = decltype(phases)::value;
+  // the builds of the kernel: by the way the activations are staged (the kernel's XS) and by whether K is walked in
+  // several phases
+  auto go = [&](auto xs, auto phases) -> int {
+    constexpr int XS = decltype(xs)::value;
+    constexpr bool PHASES = decltype(phases)::value;
     static std::atomic<bool> lds_ok[kMaxDevices];
-    if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT, PHASES>, (int)kLdsPerWgMax,
+    if (!ensure_dynamic_lds((const void*)wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, XS, KSPLIT, PHASES>, (int)kLdsPerWgMax,
                             lds_ok))
       return kFailed;
-    hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, ROWS, KSPLIT, PHASES>), dim3(plan.grid), dim3(WAVES * 64),
+    hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, XS, KSPLIT, PHASES>), dim3(plan.grid), dim3(WAVES * 64),
                        plan.lds_bytes, p.stream, (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                        (int)p.m, (int)p.n, (int)p.k,
                        group_shift | (p.zero_point << 8) | (p.activation == kActGated ? 1 << 16 : 0),
-                       plan.max_tiles, plan.phase_chunks, ksplit, plan.grid, (half_t*)p.y, ep,
+                       plan.max_tiles, plan.phase_chunks, stamp_slot_or(ksplit, KSPLIT), plan.grid, (half_t*)p.y, ep,
                        partials, counters);
     return kLaunched;
   };
-  constexpr int ch = 128 / BITS;
+  using std::integral_constant;
+  constexpr int ch = 128 / BITS, NT = WAVES * 64;
   const int phase_vectors = (plan.phase_chunks + 3) / 4 * 4 * ch / 8;  // 16-byte vectors per staged row
-  const bool flat = p.m <= 2 || phase_vectors > WAVES * 64;
-  if constexpr (KSPLIT) {
-    return flat ? go(std::false_type{}, std::false_type{}) : go(std::true_type{}, std::false_type{});
-  } else {
-    if ((int64_t)plan.phase_chunks * ch < p.k)
-      return flat ? go(std::false_type{}, std::true_type{}) : go(std::true_type{}, std::true_type{});
-    return flat ? go(std::false_type{}, std::false_type{}) : go(std::true_type{}, std::false_type{});
+  const bool flat = p.m <= 2 || phase_vectors > NT;
+  const bool phases = !KSPLIT && (int64_t)plan.phase_chunks * ch < p.k;
+  auto with_phases = [&](auto xs) -> int {
+    if constexpr (KSPLIT) return go(xs, std::false_type{});
+    else return phases ? go(xs, std::true_type{}) : go(xs, std::false_type{});
+  };
+  if (!flat) {
+    if (p.m <= 4) return with_phases(integral_constant<int, 4>{});
+    return p.m <= 8 ? with_phases(integral_constant<int, 8>{}) : with_phases(integral_constant<int, 16>{});
   }
+  if constexpr (!KSPLIT && WAVES == 8) {
+    // (the default shapes only: every exact build is a kernel more)
+    const int64_t total = p.m * (int64_t)phase_vectors;
+    if (!phases && phase_vectors >= NT && total <= 3 * NT) {
+      if (total <= NT) return go(integral_constant<int, 1>{}, std::false_type{});
+      if (total <= 2 * NT) return go(integral_constant<int, 2>{}, std::false_type{});
+      return go(integral_constant<int, 3>{}, std::false_type{});
+    }
+  }
+  return with_phases(integral_constant<int, 0>{});
 }
 
 // D chunks per lane need K to be a multiple of 4*D chunks, and the lane's D
@@ -999,3 +1109,17 @@ int launch_gemv_split_static(const Problem& p) {
 }
 
 }  // namespace wq
+
+#ifdef WQ_GEMV_STAMPS
+// The measurement build's two exports: copy the stamp array to the host (n values), clear it and restart the launch count.
+extern "C" __attribute__((visibility("default"))) int mi355x_wq_stamps_read(unsigned long long* host, int n) {
+  if (n < 0 || n > wq::kStampLaunches * wq::kStampWaves * wq::kStampPoints) return -1;
+  return hipMemcpyFromSymbol(host, HIP_SYMBOL(wq::g_gemv_stamps), (size_t)n * 8) == hipSuccess ? 0 : -1;
+}
+extern "C" __attribute__((visibility("default"))) int mi355x_wq_stamps_reset() {
+  void* p = nullptr;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(wq::g_gemv_stamps)) != hipSuccess) return -1;
+  wq::g_stamp_launches = 0;
+  return hipMemset(p, 0, sizeof(unsigned long long) * wq::kStampLaunches * wq::kStampWaves * wq::kStampPoints) == hipSuccess ? 0 : -1;
+}
+#endif
