@@ -958,7 +958,9 @@ bool split_plan_for(const Problem& p, int r, Plan* out, int64_t* path) {
 // 2 - 3 us.  A super step of a wavefront takes about 0.7 us, so the split must save at least five of
 // them on the critical path (5120 x 13824 int8: 28 -> 20, 21.8 -> 19.9 us at batch 1, 31.0 -> 22.8 us
 // at 16 rows), or spare a problem with one tile per CU the K phases that activations beyond the LDS
-// need (4096 x 11008 int4: 13.0 -> 11.7 us at 8 rows, 16.6 -> 13.7 us at 16).  On tile-major weights
+// need (4096 x 11008 int4: 12.9 -> 11.8 us at 10 rows, 13.9 -> 12.9 us at 16, int8 17.4 -> 13.8 us at 8 rows; int4
+// at up to 8 rows not: there the phases run with the next phase's activations requested a phase ahead, 10.3
+// against 11.1 us).  On tile-major weights
 // the register-activation kernel already covers the small batches of these shapes: there only from
 // 12 rows on.  Measured and excluded: 4096 x 4096 at 8 - 16 rows (5.7 -> 7.3 us), 5120 x 5120 (10.4 -> 12.1 us).
 template <int BITS>
@@ -986,7 +988,7 @@ bool choose_split(const Problem& p, int gs, SplitPlan* out) {
   }
   if (best == 1 || path1 - best_path < 5) {
     best = 1;
-    if (p.m * p.k * 2 > 160 * 1024 && tiles <= cu) {
+    if (p.m * p.k * 2 > 160 * 1024 && tiles <= cu && !(BITS == 4 && p.m <= 8)) {
       // the fewest windows whose activations fit, each wavefront keeping at least one super step
       for (int r = 2; r <= kSplitMaxR && best == 1; ++r) {
         Plan plan;

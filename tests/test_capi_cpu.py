@@ -64,7 +64,9 @@ def test_workspace_size_query_without_a_gpu():
     q = L.mi355x_wq_workspace_bytes
     assert q(lib.make_desc(8, 128, 5120, 13824), 1, 0) == 16384 + 320 * 3 * 1024         # three windows
     assert q(lib.make_desc(8, 128, 5120, 13824), 16, 0) == 16384 + 320 * 4 * 1024        # 16 rows: four fit the LDS
-    assert q(lib.make_desc(4, 32, 4096, 11008), 8, 0) == 16384 + 256 * 2 * 1024          # activations beyond the LDS
+    assert q(lib.make_desc(4, 32, 4096, 11008), 9, 0) == 16384 + 256 * 2 * 1024          # activations beyond the LDS
+    assert q(lib.make_desc(4, 32, 4096, 11008), 8, 0) == 0                                # (int4 up to 8 rows: K phases)
+    assert q(lib.make_desc(8, 128, 4096, 11008), 8, 0) == 16384 + 256 * 2 * 1024
     assert q(lib.make_desc(4, 32, 4096, 11008), 1, 0) == 0
     assert q(lib.make_desc(4, 32, 12288, 4096), 8, 0) == 0 and q(lib.make_desc(4, 32, 4096, 4096), 16, 0) == 0
     assert q(lib.make_desc(8, 128, 5120, 13824), 4, 1) == 0                              # tile-major: from 12 rows on
