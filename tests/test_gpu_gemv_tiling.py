@@ -82,3 +82,50 @@ def test_k_phases(bits, m, n, k):
         assert np.all(err <= ATOL + RTOL * np.abs(want.astype(np.float64))), (bits, m, n, k, variant, float(err.max()))
         ran += 1
     assert ran >= 2, ran
+
+
+# (bits, group, K, rows): the staging builds of the eight-wavefront kernel -- exactly one, two or three 16-byte
+# activation vectors per thread (rows of at least 512 vectors: K >= 4096), a column of up to four, eight or sixteen rows
+# per thread, the general flat index (rows of fewer than 512 vectors at batch 1 - 2; more than three vectors per thread)
+# -- for both scale layouts of each width (one scale per chunk / per super step).
+@pytest.mark.parametrize("bits,group,k,rows", [
+    (4, 32, 4096, (1, 2, 3, 4, 5, 8, 9, 16)),    # 1 and 2 vectors; columns of 4 / 8 / 16 rows
+    (4, 32, 6144, (1, 2)),                       # 768 vectors per row: 2 and 3 vectors
+    (4, 32, 11008, (1, 2)),                      # 1376 per row: 3 vectors; 2752 in all: flat index
+    (4, 128, 4096, (1, 2, 4, 8, 16)),            # one scale per super step
+    (4, 128, 6144, (1, 2)),
+    (4, 32, 2048, (1, 2, 7)),                    # rows of 256 vectors: flat index with the division
+    (8, 128, 4096, (1, 2, 3, 8, 16)),
+    (8, 128, 5120, (1, 2)),                      # 640 per row: 2 and 3 vectors
+    (8, 128, 11008, (1, 2)),
+    (8, 16, 4096, (1, 2, 6)),                    # int8 with one scale per chunk
+    (8, 128, 2048, (1, 2, 12)),
+])
+def test_activation_staging_builds(bits, group, k, rows):
+    import relax_amd
+    from relax_amd import lib
+
+    n = 530  # 34 tiles, the last one ragged
+    x_all, wq, s, g = O.make_case(7000 + bits * 131 + group + k, max(rows), n, k, bits, group=group)
+    want_all = c_oracle.wq_matmul(x_all, wq, s, bits, g, nthreads=16)
+    dwq, ds = _dev(wq), _dev(s)
+    standard = (bits, group) in ((4, 32), (8, 128)) and k % 256 == 0
+    tiled = relax_amd.wq_tile_weights(dwq, ds, bits, g) if standard else None
+    for m in rows:
+        dx = _dev(np.ascontiguousarray(x_all[:m]))
+        for variant in (15, 25):
+            y = relax_amd.wq_matmul(dx, dwq, ds, bits, g, kernel=lib.KERNEL_GEMV, variant=variant)
+            torch.cuda.synchronize()
+            _close(y.cpu().numpy(), want_all[:m], (bits, group, k, m, variant))
+            if tiled is not None:
+                yt = relax_amd.wq_matmul(dx, tiled[0], tiled[1], bits, g, tiled_n=n, kernel=lib.KERNEL_GEMV, variant=variant)
+                torch.cuda.synchronize()
+                assert torch.equal(yt.view(torch.int16), y.view(torch.int16)), ("tile-major", bits, group, k, m, variant)
+        # the fused tail behind the exact builds' plain-store fast path: bias + residual
+        bias = _dev(np.linspace(-1, 1, n).astype(np.float16))
+        res = _dev(np.full((m, n), 0.5, dtype=np.float16))
+        yf = relax_amd.wq_matmul(dx, dwq, ds, bits, g, kernel=lib.KERNEL_GEMV, variant=15, bias=bias, residual=res)
+        y0 = relax_amd.wq_matmul(dx, dwq, ds, bits, g, kernel=lib.KERNEL_GEMV, variant=15)
+        torch.cuda.synchronize()
+        want_f = ((y0.cpu().numpy() + bias.cpu().numpy()[None, :]).astype(np.float16) + np.float16(0.5)).astype(np.float16)
+        assert np.array_equal(yf.cpu().numpy().view(np.int16), want_f.view(np.int16)), ("fused", bits, group, k, m)
