@@ -124,7 +124,11 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
   constexpr bool XPRE = PHASES && (XS == 4 || XS == 8);  // (up to eight rows) a phase's activations are requested a phase ahead
   const int group_shift_ = shift_and_zero_ & 0xFF, zero_point_ = (shift_and_zero_ >> 8) & 0xFF;
   const bool gated = (shift_and_zero_ >> 16) & 1;  // fused multiply(nn.silu(gate), up): rows walked interleaved
-  const int tiles_ = (N_ + 15) >> 4;
+  // Weight rows per tile, 8 .. 16 (16 on tile-major weights, with the gated tail and with the K split): a tile is
+  // always 16 MFMA columns, of which the first tile_rows carry rows -- the host shortens the tiles where 16-row
+  // tiles would leave the workgroups unevenly loaded (5120 rows: 320 tiles on 256 workgroups, two for some and one
+  // for the others; 512 tiles of 10 rows: two for each).
+  const int tile_rows = (shift_and_zero_ >> 20) & 0x1F;
   constexpr int CH = 128 / BITS;  // k per 16-byte lane load
   constexpr int NJ = CH / 8;      // MFMAs per lane load
   constexpr int NT = WAVES * 64;
@@ -151,7 +155,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
   const int nchunks = K / CH;
   const uint32_t groups_per_row = (uint32_t)nchunks >> group_shift_;
   // (the tile-major buffers hold whole tiles: rows up to the next multiple of 16, zero filled)
-  const uint32_t n_stored = TILED ? (uint32_t)tiles_ * 16u : (uint32_t)N;
+  const uint32_t n_stored = TILED ? (uint32_t)((N_ + 15) >> 4) * 16u : (uint32_t)N;
   const rsrc_t rw = make_rsrc(wq_, n_stored * row_bytes);
   const rsrc_t rs = make_rsrc(scales_, n_stored * groups_per_row * 2u);
   const rsrc_t rx = make_rsrc(x_, (uint32_t)M * (uint32_t)K * 2u);
@@ -182,7 +186,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
   const int tile0 = KSPLIT ? (int)blockIdx.x / R : (int)blockIdx.x;
   const int tstride = KSPLIT ? G / R : G;
   // (= ceil((tiles - tile0) / tstride) without the division: max_tiles is the ceiling for tile0 = 0)
-  const int my_tiles = max_tiles_ - (tile0 + (max_tiles_ - 1) * tstride >= tiles_ ? 1 : 0);
+  const int my_tiles = max_tiles_ - ((tile0 + (max_tiles_ - 1) * tstride) * tile_rows >= N ? 1 : 0);
 
   const Q4Consts qc = make_q4_consts(zero_point_);
   const half_t* xrow = xs + (size_t)(col < M ? col : 0) * lds_stride;
@@ -227,7 +231,8 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
       else b.sc[0] = load_b32(rs, ok ? (item * 64u + (uint32_t)lane) * 4u : kOobOffset);
       return;
     }
-    int n = min(tile * 16 + col, N - 1);      // rows past N: computed, not stored
+    int n = min(tile * tile_rows + col, N - 1);  // rows past N: computed, not stored
+    ok = ok && col < tile_rows;                  // columns past the tile's rows: zeros, no request
     if (gated) n = gated_physical_row(n, N);  // even columns of a tile: gate rows, odd columns: their up rows
     const int chunk0 = c.chunk_base + ss * 4 * D + kq * D;
     // D > 1 is only launched when K is a multiple of 4*D chunks, so a lane's D
@@ -577,8 +582,8 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
     for (int idx = tid; idx < my_tiles * 256; idx += NT) {
       const int i = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
       const int m = 4 * (l >> 4) + r;
-      const int n = (tile0 + i * tstride) * 16 + (l & 15);
-      if (m < M && n < N) {
+      const int n = (tile0 + i * tstride) * tile_rows + (l & 15);
+      if (m < M && n < N && (l & 15) < tile_rows) {
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) sum += slots[((size_t)(i * WAVES + w) * 4 + r) * 64 + l];
@@ -636,7 +641,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 8
       const int i = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
       if (!last[i]) continue;
       const int m = 4 * (l >> 4) + r;
-      const int n = (tile0 + i * tstride) * 16 + (l & 15);
+      const int n = (tile0 + i * tstride) * tile_rows + (l & 15);  // (the split runs on 16-row tiles)
       float* const part = partials_ + (size_t)(tile0 + i * tstride) * R * 256 + (idx & 255);
       float sum = 0.f;
       for (int q = 0; q < R; ++q) sum += __hip_atomic_load(part + q * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -668,14 +673,39 @@ constexpr size_t kLdsPerWgMax = 159 * 1024;  // of the 160 KB a workgroup can ad
 struct Plan {
   int grid, max_tiles, phase_chunks, lds_stride;
   size_t lds_bytes;
+  int tile_rows = 16;  // weight rows per tile
 };
+
+// Rows per tile for N rows on `cap` CUs.  With 16-row tiles a tile count just above a multiple of the CUs leaves most of
+// them idle for a whole tile (5120 rows: 320 tiles on 256 CUs -- 64 walk two tiles, 192 one); shorter tiles even that
+// out (512 tiles of 10 rows: two each) at the price of load instructions whose lanes past the tile's rows request
+// nothing.  Cost of a choice: tiles per CU x (rows + 4) -- a tile costs its bytes plus about four rows' worth of
+// per-tile work -- and a shorter tile must win by an eighth.  Measured (us, 16 rows -> the rule's choice): int8
+// 5120 x 5120 at 1 / 16 rows 8.80 -> 7.92 / 12.41 -> 11.22, 5120 x 13824 19.44 -> 16.68 / 26.14 -> 24.09, int4
+// 5120 x 5120 6.31 -> 5.98; what counts is the balance over CUs, not over workgroups: 12288 rows on two workgroups
+// per CU (768 tiles: two for one workgroup, one for the other, three per CU) lose with 12-row tiles (7.36 -> 8.28).
+// `forced` (8 .. 16) overrides the rule.
+inline int pick_tile_rows(int64_t n, int cap, int forced) {
+  if (forced >= 8 && forced <= 16) return forced;
+  auto cost = [&](int tr) {
+    const int64_t tiles = (n + tr - 1) / tr, grid = std::min<int64_t>(tiles, cap);
+    return ((tiles + grid - 1) / grid) * (tr + 4);
+  };
+  int best = 16;
+  int64_t best_cost = cost(16);
+  for (int tr = 15; tr >= 8; --tr)
+    if (cost(tr) < best_cost) best = tr, best_cost = cost(tr);
+  return best_cost * 8 <= cost(16) * 7 ? best : 16;
+}
 
 // Chooses the grid (workgroups per CU), the tiles per workgroup and the K phase so
 // that partial-tile slots + staged activations fit in LDS.
 template <int BITS, int WAVES, int D>
-bool make_plan(const Problem& p, int wgs_per_cu, Plan* out) {
+bool make_plan(const Problem& p, int wgs_per_cu, Plan* out, int tile_rows = 0) {
   constexpr int ch = 128 / BITS;
-  const int tiles = (int)((p.n + 15) / 16);
+  // (tile-major weights are laid out in 16-row tiles, and the gated tail pairs adjacent columns of one)
+  const int tr = (p.tiled || p.activation == kActGated) ? 16 : pick_tile_rows(p.n, cu_count(), tile_rows);
+  const int tiles = (int)((p.n + tr - 1) / tr);
   const int nchunks = (int)(p.k / ch);
   const size_t budget = std::min(kLdsPerWgMax, kLdsPerCu / (size_t)wgs_per_cu - 1024);
   const int grid = std::min(tiles, cu_count() * wgs_per_cu);
@@ -703,6 +733,7 @@ bool make_plan(const Problem& p, int wgs_per_cu, Plan* out) {
   }
   out->grid = grid;
   out->max_tiles = max_tiles;
+  out->tile_rows = tr;
   out->phase_chunks = phase_chunks;
   out->lds_stride = phase_chunks * ch + 8;  // +16 bytes: consecutive rows start 4 banks apart
   out->lds_bytes = slot_bytes + (size_t)p.m * out->lds_stride * sizeof(half_t);
@@ -746,7 +777,7 @@ int launch_one(const Problem& p, int group_shift, const Plan& plan, int ksplit =
     hipLaunchKernelGGL((wq_gemv_kernel<BITS, WAVES, D, SPL, TILED, XS, KSPLIT, PHASES>), dim3(plan.grid), dim3(WAVES * 64),
                        plan.lds_bytes, p.stream, (const half_t*)p.x, (const uint32_t*)p.wq, (const half_t*)p.scales,
                        (int)p.m, (int)p.n, (int)p.k,
-                       group_shift | (p.zero_point << 8) | (p.activation == kActGated ? 1 << 16 : 0),
+                       group_shift | (p.zero_point << 8) | (p.activation == kActGated ? 1 << 16 : 0) | (plan.tile_rows << 20),
                        plan.max_tiles, plan.phase_chunks, stamp_slot_or(ksplit, KSPLIT), plan.grid, (half_t*)p.y, ep,
                        partials, counters);
     return kLaunched;
@@ -779,11 +810,11 @@ int launch_one(const Problem& p, int group_shift, const Plan& plan, int ksplit =
 // D chunks per lane need K to be a multiple of 4*D chunks, and the lane's D
 // chunks to share one scale (SPL = 1) or to have one each (SPL = D).
 template <int BITS, int WAVES, int D>
-int try_launch(const Problem& p, int group_shift, int wgs_per_cu) {
+int try_launch(const Problem& p, int group_shift, int wgs_per_cu, int tile_rows) {
   constexpr int ch = 128 / BITS;
   if (D > 1 && p.k % (4 * D * ch) != 0) return kNotApplicable;
   Plan plan;
-  if (!make_plan<BITS, WAVES, D>(p, wgs_per_cu, &plan)) return kNotApplicable;
+  if (!make_plan<BITS, WAVES, D>(p, wgs_per_cu, &plan, tile_rows)) return kNotApplicable;
   if (p.tiled) {
     // only the layout's own shape: super steps of eight chunks, scales per chunk (int4 / group 32)
     // or per super step (int8 / group 128)
@@ -798,20 +829,21 @@ int try_launch(const Problem& p, int group_shift, int wgs_per_cu) {
   return kNotApplicable;
 }
 
-// variant = 10 * workgroups-per-CU + shape index
+// variant = 100 * rows-per-tile (0: the rule's choice, else 8 .. 16) + 10 * workgroups-per-CU + shape index
 template <int BITS>
 int dispatch(const Problem& p, int gs, int variant) {
-  const int wpc = variant / 10, shape = variant % 10;
-  if (wpc < 1 || wpc > 8) return kNotApplicable;
+  const int tr = variant / 100, wpc = variant % 100 / 10, shape = variant % 10;
+  if (wpc < 1 || wpc > 8 || (tr != 0 && (tr < 8 || tr > 16))) return kNotApplicable;
+  if (tr != 0 && tr != 16 && (p.tiled || p.activation == kActGated)) return kNotApplicable;
   switch (shape) {
-    case 1: return try_launch<BITS, 4, 1>(p, gs, wpc);
-    case 2: return try_launch<BITS, 4, 2>(p, gs, wpc);
-    case 3: return try_launch<BITS, 4, 4>(p, gs, wpc);
-    case 4: return try_launch<BITS, 8, 1>(p, gs, wpc);
-    case 5: return try_launch<BITS, 8, 2>(p, gs, wpc);
-    case 6: return try_launch<BITS, 8, 4>(p, gs, wpc);
-    case 7: return try_launch<BITS, 16, 1>(p, gs, wpc);
-    case 8: return try_launch<BITS, 16, 2>(p, gs, wpc);
+    case 1: return try_launch<BITS, 4, 1>(p, gs, wpc, tr);
+    case 2: return try_launch<BITS, 4, 2>(p, gs, wpc, tr);
+    case 3: return try_launch<BITS, 4, 4>(p, gs, wpc, tr);
+    case 4: return try_launch<BITS, 8, 1>(p, gs, wpc, tr);
+    case 5: return try_launch<BITS, 8, 2>(p, gs, wpc, tr);
+    case 6: return try_launch<BITS, 8, 4>(p, gs, wpc, tr);
+    case 7: return try_launch<BITS, 16, 1>(p, gs, wpc, tr);
+    case 8: return try_launch<BITS, 16, 2>(p, gs, wpc, tr);
     default: return kNotApplicable;
   }
 }
@@ -972,7 +1004,13 @@ bool choose_split(const Problem& p, int gs, SplitPlan* out) {
   const int64_t tiles = (p.n + 15) / 16, cu = cu_count();
   if (tiles > kSplitMaxTiles) return false;
   const int nsuper = (int)(p.k / ch) / (4 * kSplitD);
-  const int64_t path1 = ((tiles + std::min(tiles, cu) - 1) / std::min(tiles, cu)) * ((nsuper + kSplitWaves - 1) / kSplitWaves);
+  // (paths in twentieths of a 16-row super step: the plain call may run shorter tiles, pick_tile_rows, whose super
+  // steps cost (rows + 4) / 20 of a 16-row one -- while its activations fit the LDS in one piece; the split's tiles
+  // have 16 rows)
+  const bool gated = p.activation == kActGated;
+  const int tr = (p.tiled || gated || (int64_t)p.m * p.k * 2 + 16384 > (int64_t)kLdsPerWgMax) ? 16 : pick_tile_rows(p.n, (int)cu, 0);
+  const int64_t tiles1 = (p.n + tr - 1) / tr;
+  const int64_t path1 = ((tiles1 + std::min(tiles1, cu) - 1) / std::min(tiles1, cu)) * ((nsuper + kSplitWaves - 1) / kSplitWaves) * (tr + 4);
   int best = 1;
   int64_t best_path = path1;
   Plan best_plan{};
@@ -980,13 +1018,13 @@ bool choose_split(const Problem& p, int gs, SplitPlan* out) {
     Plan plan;
     int64_t path;
     if (!split_plan_for<BITS>(p, r, &plan, &path)) continue;
-    if (path < best_path) {
+    if (path * 20 < best_path) {
       best = r;
-      best_path = path;
+      best_path = path * 20;
       best_plan = plan;
     }
   }
-  if (best == 1 || path1 - best_path < 5) {
+  if (best == 1 || path1 - best_path < 5 * 20) {
     best = 1;
     if (p.m * p.k * 2 > 160 * 1024 && tiles <= cu && !(BITS == 4 && p.m <= 8)) {
       // the fewest windows whose activations fit, each wavefront keeping at least one super step

