@@ -76,7 +76,8 @@ static void check_descriptors() {
   mi355x_wq_desc odd{4, 32, 7, 0, 100, 352};
   EXPECT(mi355x_wq_tiled_sizes(&odd, &wb, &sb) == -1);
   mi355x_wq_desc q8{8, 128, 0, 0, 5120, 13824};
-  EXPECT(mi355x_wq_workspace_bytes(&q8, 1, 0) > 0);
+  EXPECT(mi355x_wq_workspace_bytes(&q8, 8, 0) > 0);
+  EXPECT(mi355x_wq_workspace_bytes(&q8, 1, 0) == 0);
   EXPECT(mi355x_wq_workspace_bytes(&d, 1, 0) == 0);
   EXPECT(mi355x_wq_matmul_ws(&d, (void*)ok, (void*)ok, (void*)ok, nullptr, (void*)ok, 4, nullptr, 0, (void*)(ok + 4),
                              1 << 20) == -1);
