@@ -988,8 +988,9 @@ bool split_plan_for(const Problem& p, int r, Plan* out, int64_t* path) {
 // staging where one tile per CU makes every workgroup stage all of a large x.  What it costs: the last
 // workgroup's chain of three trips to the memory side of the L2s (partials out, count, partials in),
 // 2 - 3 us.  A super step of a wavefront takes about 0.7 us, so the split must save at least five of
-// them on the critical path (5120 x 13824 int8: 28 -> 20, 21.8 -> 19.9 us at batch 1, 31.0 -> 22.8 us
-// at 16 rows), or spare a problem with one tile per CU the K phases that activations beyond the LDS
+// them on the critical path (5120 x 13824 int8 on 16-row tiles: 28 -> 20 super steps; 22.7 -> 19.8 us at 8 rows,
+// 24.1 -> 21.3 us at 16 -- at up to 5 rows, where the activations fit the LDS in one piece, the plain call's 10-row
+// tiles do better, 16.7 against 18.4 us at batch 1), or spare a problem with one tile per CU the K phases that activations beyond the LDS
 // need (4096 x 11008 int4: 12.9 -> 11.8 us at 10 rows, 13.9 -> 12.9 us at 16, int8 17.4 -> 13.8 us at 8 rows; int4
 // at up to 8 rows not: there the phases run with the next phase's activations requested a phase ahead, 10.3
 // against 11.1 us).  On tile-major weights
