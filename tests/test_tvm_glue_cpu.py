@@ -439,3 +439,64 @@ def test_gated_tail_of_a_gate_up_projection(fake_tvm):
             spec_from_function(fake_tvm.quantized_linear(n=64, tail=tail))
     with pytest.raises(ValueError, match="no bias and no residual"):
         Spec(0, 4, 0, 7, 2, 0, 1, 4, 3, -1, ACT_SILU_MUL).validate()
+
+
+def test_finalize_compiles_and_links_what_the_hook_emitted(fake_tvm, monkeypatch, tmp_path):
+    """finalize() (counterpart of finalize_modules_relax, python/tvm/contrib/cutlass/build.py:856-879) run against a
+    stand-in for the two TVM calls it makes.  `export_library` is what it is in TVM for a module tree with C-source
+    modules (python/tvm/runtime/module.py:450-560): write each module's source, compile with `cc` and the caller's
+    `options`, link one shared object; `load_module` opens it.  The stand-in really compiles -- so the link options
+    finalize passes (library directory, -lmi355x_wq, rpath) and the generated source are exercised together -- and the
+    entry of the hook's C-source module is then called through the loaded object."""
+    import sys
+    import types
+
+    from relax_amd.tvm_glue import codegen
+
+    class CSourceModule:
+        def __init__(self, source, fmt, symbols, consts):
+            self.source, self.format, self.symbols = source, fmt, list(symbols)
+
+    class Executable:
+        class Mod:
+            def __init__(self, imports):
+                self.imports = imports
+
+            def export_library(self, path, cc="g++", options=()):
+                files = []
+                for i, m in enumerate(self.imports):
+                    src = tmp_path / f"lib{i}.{m.format}"  # "cc": compiled as C++, as export_library does
+                    src.write_text(m.source)
+                    files.append(str(src))
+                subprocess.check_call([cc, "-shared", "-fPIC", "-Wall", "-Werror", "-DMI355X_WQ_STANDALONE", "-o", path]
+                                      + files + list(options))
+
+        def __init__(self, imports):
+            self.mod = Executable.Mod(imports)
+
+    registry = {"runtime.CSourceModuleCreate": CSourceModule}
+    tvm = sys.modules["tvm"]
+    monkeypatch.setattr(tvm, "get_global_func", lambda name: registry[name], raising=False)
+    monkeypatch.setattr(tvm, "runtime", types.SimpleNamespace(load_module=lambda path: C.CDLL(path)), raising=False)
+
+    free = fake_tvm.quantized_linear(symbol="free_mi355x")
+    mods = codegen.relax_ext_mi355x([free], None, {})
+    assert len(mods) == 1 and mods[0].symbols == ["free_mi355x"] and mods[0].format == "cc"
+    out = str(tmp_path / "model.so")
+    loaded = codegen.finalize(Executable(mods), lib.SO_PATH, out)
+    assert os.path.exists(out)
+    lib.load()
+    # the loaded object exports the hook's symbol with the backend calling convention, bound to the library's entry:
+    # FuseOpsByPattern order (wq, scales, x, y); a float16 tensor in the wq slot is refused by the library's own check
+    x = torch.zeros((2, 64), dtype=torch.float16)
+    wq = torch.zeros((16, 8), dtype=torch.int32)
+    s = torch.zeros((16, 2), dtype=torch.float16)
+    y = torch.zeros((2, 16), dtype=torch.float16)
+    dev = dict(device_type=10)
+    t = [vm_harness.TensorArg(wq, as_uint32=True, **dev), vm_harness.TensorArg(s, **dev),
+         vm_harness.TensorArg(x, **dev), vm_harness.TensorArg(y, **dev)]
+    rc, _ = call_entry(loaded, "free_mi355x", [t[2], t[0], t[1], t[3]])
+    assert rc == -1 and "argument 0 (wq): expected dtype uint32" in lib.last_error()
+    if not torch.cuda.is_available():
+        rc, _ = call_entry(loaded, "free_mi355x", t)
+        assert rc == -1 and "no usable HIP device" in lib.last_error()
