@@ -382,6 +382,26 @@ def stamp_budget(torch, dev, args, L) -> int:
                 cells.append(f"{np.median(c):.2f} ({c.min():.2f}-{c.max():.2f})")
             print(f"| {name} {n}x{k} | {len(r)} | {pause} | " + " | ".join(cells) + f" | {rel[:, 7].max():.2f} |")
             prev_end = r[:, 7].max()
+        # the same launches by workgroup (a workgroup's wavefronts are eight consecutive slots), in eighths of the
+        # workgroup ids: does a workgroup that starts or ends late do so because of where it sits in the grid?
+        print("| shape | workgroups | eighth of the workgroup ids: entry of the first wavefront / weight stream end / "
+              "stores acknowledged of the last, mean us | corr(id, end) | sd of end - entry |")
+        print("|---|---|---|---|---|")
+        for j, (name, n, k) in enumerate(LLAMA7B):
+            r = a[j]
+            keep = (r[:, 0] > 0) & (r[:, 7] > r[:, 7].max() - 5000)
+            slot = np.nonzero(keep)[0]
+            r = r[keep]
+            rel = (r - r[:, 0].min()) / 100.0
+            wg = slot // 8
+            ids = np.unique(wg)
+            entry = np.array([rel[wg == w, 0].min() for w in ids])
+            s_end = np.array([rel[wg == w, 4].max() for w in ids])
+            end = np.array([rel[wg == w, 7].max() for w in ids])
+            eighth = (np.arange(len(ids)) * 8) // len(ids)
+            cells = " ; ".join(f"{entry[eighth == e].mean():.2f} / {s_end[eighth == e].mean():.2f} / {end[eighth == e].mean():.2f}"
+                               for e in range(8))
+            print(f"| {name} {n}x{k} | {len(ids)} | {cells} | {np.corrcoef(ids, end)[0, 1]:.2f} | {np.std(end - entry):.2f} |")
         sys.stdout.flush()
         del g
     return 0
