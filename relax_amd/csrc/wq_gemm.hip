@@ -281,7 +281,7 @@ int launch_gemm_any(const Problem& p, int variant, bool direct_ok) {
   }
   if (!direct_ok && (p.tiled || variant >= 21)) {
     set_error("gemm kernel: gelu with the residual in the output buffer is not available on the direct-weight kernel "
-              "(tile-major weights, variants 21..26); pass the residual in a buffer of its own");
+              "(tile-major weights, variants 21..29); pass the residual in a buffer of its own");
     return -1;
   }
   if (p.tiled) {
@@ -298,7 +298,7 @@ int launch_gemm_any(const Problem& p, int variant, bool direct_ok) {
       ok = launch_gemm_direct(p, group_shift, variant - 20);
     if (!ok) {
       set_error("gemm kernel: tile-major weights need the direct-weight kernel (K %% 256 == 0, operands below "
-                "1 GiB; variant 0 or 21..26), got M=%lld N=%lld K=%lld variant=%d", (long long)p.m,
+                "1 GiB; variant 0 or 21..29), got M=%lld N=%lld K=%lld variant=%d", (long long)p.m,
                 (long long)p.n, (long long)p.k, variant);
       return -1;
     }

@@ -21,7 +21,7 @@ def _families():
 
     gemv = [10 * wpc + shape for wpc in (1, 2, 4) for shape in range(1, 9)]
     skinny = list(range(1, 12)) + list(range(21, 32))
-    gemm = list(range(1, 7)) + [11, 12, 13] + list(range(21, 27))
+    gemm = list(range(1, 7)) + [11, 12, 13] + list(range(21, 30))
     return [("gemv", lib.KERNEL_GEMV, gemv, (1, 3, 8, 16)),
             ("skinny", lib.KERNEL_SKINNY, skinny, (2, 16, 20, 40, 64, 100)),
             ("gemm", lib.KERNEL_GEMM, gemm, (70, 150, 300))]

@@ -295,10 +295,13 @@ def test_gemm_kernel_matches_oracle(bits, m, n, k):
     (24, 4, 300, 200, 512), (24, 4, 65, 520, 1280), (24, 4, 70, 136, 768), (24, 8, 513, 260, 1024),
     (24, 8, 100, 64, 1792),
     (25, 4, 300, 200, 1024), (25, 4, 65, 520, 1280), (25, 4, 70, 136, 2304), (25, 8, 513, 260, 1024),
-    (25, 8, 100, 64, 1792)])
+    (25, 8, 100, 64, 1792),
+    (27, 8, 129, 72, 256), (27, 8, 513, 260, 1024), (28, 8, 513, 260, 1024), (28, 8, 100, 64, 1792),
+    (29, 8, 513, 260, 1024), (29, 8, 100, 64, 1792), (27, 4, 300, 200, 256)])
 def test_gemm_direct_weight_variants_match_oracle(variant, bits, m, n, k):
     """Direct-weight kernel, 128-row tiles with one (21) and two (22) K groups, 64-row tiles (23, 24) and
-    64 x 128 tiles with four K groups (25):
+    64 x 128 tiles with four K groups (25); 27 - 29: the 64-row builds with every lane loading its own row's pieces
+    (23 - 25 load int8 weights in the canonical layout by whole cache lines through LDS):
     ragged M and N, K of one macro step, an even and an odd number of 256-wide macro steps (the second
     K group is then the shorter one)."""
     from relax_amd import lib
@@ -307,6 +310,40 @@ def test_gemm_direct_weight_variants_match_oracle(variant, bits, m, n, k):
     got = run_matmul(x, wq, s, bits, g, kernel=lib.KERNEL_GEMM, variant=variant)
     want = c_oracle.wq_matmul(x, wq, s, bits, g, nthreads=16)
     assert_close(got, want, (variant, bits, m, n, k))
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 5120, 5120), (200, 5000, 1024), (64, 130, 512), (256, 15360, 5120),
+                                   (100, 5120, 13824), (256, 264, 2048), (33, 64, 1024), (65, 1, 256), (70, 4097, 768)])
+def test_gemm_line_wise_weight_loads_equal_the_direct_ones(m, n, k):
+    """int8 weights in the canonical layout, 64-row tiles: the builds that load whole cache lines of the weight rows
+    and hand the pieces to the lanes through wavefront-private LDS (variants 23 - 25) against the builds in which
+    every lane loads its own pieces (27 - 29).  Same lanes, same registers, same order of additions: bit for bit,
+    with the fused tails and on a ragged N (the last rows clamped), a single row and K of one and two macro steps."""
+    import relax_amd
+    from relax_amd import lib
+
+    x, wq, s, g = O.make_case(8800 + m + n + k, m, n, k, 8)
+    dx, dwq, ds = _dev(x), _dev(wq), _dev(s)
+    bias = _dev(np.linspace(-1, 1, n).astype(np.float16))
+    res = _dev(np.full((m, n), 0.25, dtype=np.float16))
+    ran = 0
+    for hop, direct in ((23, 27), (24, 28), (25, 29)):
+        for kw in ({}, {"bias": bias, "activation": "relu", "residual": res}):
+            try:
+                ya = relax_amd.wq_matmul(dx, dwq, ds, 8, g, kernel=lib.KERNEL_GEMM, variant=direct, **kw)
+            except lib.WqError:
+                continue  # (K too short for the K groups of this variant)
+            yb = relax_amd.wq_matmul(dx, dwq, ds, 8, g, kernel=lib.KERNEL_GEMM, variant=hop, **kw)
+            torch.cuda.synchronize()
+            assert torch.equal(ya.view(torch.int16), yb.view(torch.int16)), (m, n, k, hop, sorted(kw))
+            ran += 1
+    assert ran >= 2
+    if n % 2 == 0:
+        # the gated tail walks the weight rows in the interleaved gate / up order
+        ya = relax_amd.wq_matmul(dx, dwq, ds, 8, g, kernel=lib.KERNEL_GEMM, variant=27, activation="silu_mul")
+        yb = relax_amd.wq_matmul(dx, dwq, ds, 8, g, kernel=lib.KERNEL_GEMM, variant=23, activation="silu_mul")
+        torch.cuda.synchronize()
+        assert torch.equal(ya.view(torch.int16), yb.view(torch.int16)), (m, n, k, "gated")
 
 
 @pytest.mark.parametrize("bits,m,n,k", [(4, 600, 15323, 512), (8, 1000, 8200, 768)])
