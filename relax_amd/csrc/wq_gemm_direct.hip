@@ -207,6 +207,8 @@ __global__ __launch_bounds__(GROUPS * WAVES * 64, 1) void wq_gemm_direct_kernel(
   // into its own 4 KB of LDS (rows of 128 bytes, chunks XOR-swizzled like the activation rows: stores and loads
   // conflict-free) and every lane reads back the four chunks of its row in the order the direct loads deliver.
   // The hardware executes a wavefront's LDS instructions in order; the fences state the order for the compiler.
+  // (int4 was built the same way -- a line is four K steps there, the block stored twice -- and measured: bit-equal,
+  // -6 ... +3.5 % on the 4096- to 22016-row shapes at 128 to 512 rows; it has half the requests per k to begin with.)
   unsigned char* const hop = wq_gemm_direct_smem + GROUPS * 4 * STAGE + wave_id * 4096;
   uint32_t hg[2][4];   // global offset of this lane's chunk for request i4 of column tile j
   uint32_t hop_wr[2];  // LDS store offset for even / odd i4 (+ i4 * 1024)
@@ -833,6 +835,10 @@ int gemm_split_ways(const Problem& p) {
   }
   const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 255) / 256);
   if (tiles * (p.bits == 4 ? 8 : 2) > cu || tiles > kGemmSplitMaxTiles) return 1;
+  // (int8 in the canonical layout: since the plain call's 64-row tiles load the weight rows by whole cache lines,
+  // the split's 128-row tiles, which do not, only win with long K -- at 256 rows 5120 x 13824 64 against 78 us,
+  // but 15360 x 5120 59 against 60 and 5120 x 5120 34.1 against 33.5)
+  if (!p.tiled && p.bits == 8 && p.k < 8192) return 1;
   // (not where the plain call's 64 x 128 tiles fill three quarters of the CUs or more in one round:
   // 15360 x 5120 int8 at 128 rows, 240 tiles, 46 us plain against 49 us split)
   const int64_t plain = ((p.m + 63) / 64) * ((p.n + 127) / 128);

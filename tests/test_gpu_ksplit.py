@@ -164,7 +164,7 @@ def test_workspace_entry_called_vm_style():
     import relax_amd
 
     vm_harness.set_stream()
-    for bits, m, n, k in [(8, 8, 5120, 13824), (4, 16, 4096, 11008), (4, 8, 50, 512), (8, 256, 5120, 5120),
+    for bits, m, n, k in [(8, 8, 5120, 13824), (4, 16, 4096, 11008), (4, 8, 50, 512), (8, 256, 5120, 8192),
                           (4, 64, 4096, 11008)]:  # decode split, no split, the GEMM's split above and below 64 rows
         x, wq, s, g = O.make_case(60 + m, m, n, k, bits)
         need = relax_amd.wq_workspace_bytes(bits, g, n, k, m)
@@ -211,9 +211,10 @@ def test_k_split_is_stable_while_another_stream_keeps_the_gpu_busy():
     assert int(ws[:16384].view(torch.int32).abs().sum()) == 0
 
 
-# (bits, M, N, K): prefill-side shapes whose 128 x 256 tiles fill at most half of the CUs
-GEMM_CASES = [(8, 256, 5120, 5120), (8, 256, 5120, 13824), (8, 256, 15360, 5120), (4, 256, 4096, 11008),
-              (4, 160, 4096, 11008), (4, 200, 4090, 8192), (8, 200, 5120, 5120), (8, 384, 1000, 2048),
+# (bits, M, N, K): prefill-side shapes whose 128 x 256 tiles fill at most half of the CUs (int8 in the canonical
+# layout splits from K = 8192 on: below that the plain call's line-wise weight loads do as well)
+GEMM_CASES = [(8, 256, 5120, 8192), (8, 256, 5120, 13824), (8, 256, 15360, 8192), (4, 256, 4096, 11008),
+              (4, 160, 4096, 11008), (4, 200, 4090, 8192), (8, 200, 5120, 8192), (8, 384, 1000, 8192),
               # 17 .. 64 rows: 64 x 128 tiles, four K groups per workgroup
               (4, 64, 12288, 4096), (4, 56, 12288, 4096), (8, 25, 5120, 13824), (4, 41, 4090, 11008),
               (8, 60, 1000, 8192), (4, 64, 4096, 11008), (8, 64, 5120, 8192), (4, 33, 2000, 8448)]

@@ -339,7 +339,9 @@ def test_module_owned_workspace(bits, n, k, rows, flags):
         full = (dx.float() @ wd.t())
         err = (y.float() - full).abs()
         assert bool((err <= 2e-2 + 1e-2 * full.abs()).all()), float(err.max())
-    assert split_somewhere or (bits == 8 and n == 27648), "these shapes are meant to split K at some row count"
+    # (int8 with K = 5120: 27648 rows never split; the others only on tile-major weights, since the plain call loads
+    # the canonical layout by whole cache lines)
+    assert split_somewhere or (bits == 8 and k == 5120 and (n == 27648 or not tiled)), "these shapes are meant to split K at some row count"
     # more rows than the workspace was sized for: the plain call
     m = 300
     x, _, _, _ = O.make_case(61, m, 16, k, bits)
